@@ -1,0 +1,286 @@
+// Row-wise and element-wise kernels: embedding gather, (residual add +) RMSNorm,
+// per-head QK-norm + rotary embedding + cache write, SwiGLU.
+//
+// Formulas follow the reference's kernels; the fusions are ours (the reference launches each
+// op on its own and rounds to bf16 in between, src/qwen.cc:574-799):
+//   embedding   src/kernels/embedding.cu:22-38
+//   RMSNorm     src/kernels/rmsnorm.cu:56-97     y = x * rsqrt(mean(x^2) + eps) * w
+//   residual    src/kernels/add.cu:11-14         a + b in fp32
+//   QK-norm     src/qwen.cc:617-632              RMSNorm over head_dim, one [d] weight
+//   rotary      src/kernels/rope.cu:28-60        pairs (i, i + d/2), angle = pos / theta^(2i/d)
+//   cache write src/kernels/attention_paged.cu:26-44
+//   SwiGLU      src/kernels/swiglu.cu:8,31-35    g / (1 + exp(-g)) * u
+#include "common.h"
+
+#include <cstdarg>
+#include <cstdio>
+
+namespace lc {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+// ------------------------------------------------------------------------------- embedding
+template <typename TW>
+__global__ void embedding_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
+                                 float* __restrict__ out, int H, int V) {
+    const int t = blockIdx.x;
+    int id = ids[t];
+    if (id < 0 || id >= V) id = 0;  // the host has rejected such ids already
+    const TW* row = table + (size_t)id * H;
+    float* dst = out + (size_t)t * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = to_f32(row[i]);
+}
+
+// ------------------------------------------------------------------------------- RMSNorm
+// One workgroup per output row r.  src row = rows ? rows[r] : r.
+//   v = h[src] (+ delta[src]);  if (write_h) h[src] = v;  out[r] = v * rsqrt(mean(v^2)+eps) * w
+template <typename T>
+__global__ void rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delta,
+                               const int* __restrict__ rows, const float* __restrict__ w,
+                               float eps, T* __restrict__ out, int n, int write_h) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int src = rows ? rows[r] : r;
+    float* hr = h + (size_t)src * n;
+    const T* dr = delta ? delta + (size_t)src * n : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        float v = hr[i];
+        if (dr) {
+            v += to_f32(dr[i]);
+            if (write_h) hr[i] = v;
+        }
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = rsqrtf(ss / (float)n + eps);
+    T* o = out + (size_t)r * n;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        float v = hr[i];
+        if (dr && !write_h) v += to_f32(dr[i]);
+        o[i] = from_f32<T>(v * inv * w[i]);
+    }
+}
+
+// RMSNorm of rows held in the activation type (no residual stream involved).
+template <typename T>
+__global__ void rmsnorm_act_kernel(const T* __restrict__ x, const float* __restrict__ w,
+                                   float eps, T* __restrict__ out, int n) {
+    __shared__ float scratch[16];
+    const T* xr = x + (size_t)blockIdx.x * n;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        float v = to_f32(xr[i]);
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = rsqrtf(ss / (float)n + eps);
+    T* o = out + (size_t)blockIdx.x * n;
+    for (int i = threadIdx.x; i < n; i += blockDim.x)
+        o[i] = from_f32<T>(to_f32(xr[i]) * inv * w[i]);
+}
+
+// ------------------------------------------------------- QK-norm + rotary + cache write
+// qkv: [T, nh + 2 nkv, d] (q heads, then k heads, then v heads).  One wave per (token, head).
+//   q, k: optional RMSNorm over d, then rotation of the first `rot` dims with the angles of
+//   the token's position (cos in table[pos][0:rot/2], sin in table[pos][rot/2:rot]).
+//   q and k are written back in place; k and v also go to the cache page slot of the token.
+// Cache layout: [pages, nkv, page_size, d]; slot = page * page_size + offset; slot < 0 skips.
+template <typename T>
+__global__ void qk_norm_rope_write_kernel(T* __restrict__ qkv, int T_tokens, int nh, int nkv, int d,
+                                          const float* __restrict__ q_w,
+                                          const float* __restrict__ k_w, float eps,
+                                          const int* __restrict__ positions,
+                                          const float* __restrict__ rope_table, int rot,
+                                          T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                          const int* __restrict__ slots, int page_size) {
+    const int t = blockIdx.x;
+    const int wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int waves = blockDim.x / kWave;
+    const int heads = nh + 2 * nkv;
+    const int head = blockIdx.y * waves + wave;
+    if (head >= heads) return;
+    T* x = qkv + ((size_t)t * heads + head) * d;
+
+    const bool is_q = head < nh;
+    const bool is_k = !is_q && head < nh + nkv;
+    const int kvh = is_q ? 0 : (is_k ? head - nh : head - nh - nkv);
+
+    T* cache_row = nullptr;
+    if (!is_q && slots && k_cache) {
+        const int slot = slots[t];
+        if (slot >= 0) {
+            const int page = slot / page_size, off = slot - page * page_size;
+            T* base = is_k ? k_cache : v_cache;
+            cache_row = base + (((size_t)page * nkv + kvh) * page_size + off) * d;
+        }
+    }
+
+    if (!is_q && !is_k) {  // v: copy only
+        if (cache_row)
+            for (int i = lane; i < d; i += kWave) cache_row[i] = x[i];
+        return;
+    }
+
+    const float* w = is_q ? q_w : k_w;
+    float inv = 1.f;
+    if (w) {
+        float ss = 0.f;
+        for (int i = lane; i < d; i += kWave) {
+            float v = to_f32(x[i]);
+            ss += v * v;
+        }
+        ss = wave_sum(ss);
+        inv = rsqrtf(ss / (float)d + eps);
+    }
+    const int half = rot / 2;
+    const float* cs = rope_table ? rope_table + (size_t)positions[t] * rot : nullptr;
+    // rotated pairs
+    for (int i = lane; i < half; i += kWave) {
+        float a = to_f32(x[i]) * inv, b = to_f32(x[i + half]) * inv;
+        if (w) { a *= w[i]; b *= w[i + half]; }
+        float c = 1.f, s = 0.f;
+        if (cs) { c = cs[i]; s = cs[half + i]; }
+        const T ra = from_f32<T>(a * c - b * s);
+        const T rb = from_f32<T>(a * s + b * c);
+        x[i] = ra;
+        x[i + half] = rb;
+        if (cache_row) { cache_row[i] = ra; cache_row[i + half] = rb; }
+    }
+    // dims beyond the rotary part
+    for (int i = rot + lane; i < d; i += kWave) {
+        float a = to_f32(x[i]) * inv;
+        if (w) a *= w[i];
+        const T ra = from_f32<T>(a);
+        x[i] = ra;
+        if (cache_row) cache_row[i] = ra;
+    }
+}
+
+// ------------------------------------------------------------------------------- SwiGLU
+// gu: [T, 2 I] (gate columns, then up columns) -> out [T, I]
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t t = idx / I;
+        const int i = (int)(idx - t * I);
+        const float g = to_f32(gu[t * 2 * I + i]);
+        const float u = to_f32(gu[t * 2 * I + I + i]);
+        out[idx] = from_f32<T>(g / (1.f + expf(-g)) * u);
+    }
+}
+
+}  // namespace lc
+
+using namespace lc;
+
+LC_API const char* lc_last_error() { return g_error; }
+
+LC_API int lc_embedding(const int* ids, const void* table, int table_dt, float* out, int T, int H,
+                        int V, hipStream_t stream) {
+    LC_CHECK(T >= 0 && H > 0 && V > 0, "embedding: bad sizes T=%d H=%d V=%d", T, H, V);
+    if (T == 0) return 0;
+    LC_CHECK(ids && table && out, "embedding: null pointer");
+    const int threads = H >= 256 ? 256 : 64;
+    if (table_dt == DT_F32)
+        embedding_kernel<float><<<T, threads, 0, stream>>>(ids, (const float*)table, out, H, V);
+    else if (table_dt == DT_BF16)
+        embedding_kernel<bf16><<<T, threads, 0, stream>>>(ids, (const bf16*)table, out, H, V);
+    else
+        LC_CHECK(false, "embedding: unknown table dtype %d", table_dt);
+    LC_LAUNCH_CHECK("embedding");
+    return 0;
+}
+
+LC_API int lc_rmsnorm(float* h, const void* delta, const int* rows, const float* w, float eps,
+                      void* out, int dt, int R, int n, int write_h, hipStream_t stream) {
+    LC_CHECK(R >= 0 && n > 0, "rmsnorm: bad sizes R=%d n=%d", R, n);
+    if (R == 0) return 0;
+    LC_CHECK(h && w && out, "rmsnorm: null pointer");
+    LC_CHECK(!(rows && write_h), "rmsnorm: gathered rows cannot be written back");
+    const int threads = n >= 1024 ? 256 : (n >= 256 ? 128 : 64);
+    if (dt == DT_F32)
+        rmsnorm_kernel<float><<<R, threads, 0, stream>>>(h, (const float*)delta, rows, w, eps,
+                                                         (float*)out, n, write_h);
+    else if (dt == DT_BF16)
+        rmsnorm_kernel<bf16><<<R, threads, 0, stream>>>(h, (const bf16*)delta, rows, w, eps,
+                                                        (bf16*)out, n, write_h);
+    else
+        LC_CHECK(false, "rmsnorm: unknown dtype %d", dt);
+    LC_LAUNCH_CHECK("rmsnorm");
+    return 0;
+}
+
+LC_API int lc_rmsnorm_act(const void* x, const float* w, float eps, void* out, int dt, int R,
+                          int n, hipStream_t stream) {
+    LC_CHECK(R >= 0 && n > 0, "rmsnorm_act: bad sizes R=%d n=%d", R, n);
+    if (R == 0) return 0;
+    LC_CHECK(x && w && out, "rmsnorm_act: null pointer");
+    const int threads = n >= 1024 ? 256 : (n >= 256 ? 128 : 64);
+    if (dt == DT_F32)
+        rmsnorm_act_kernel<float><<<R, threads, 0, stream>>>((const float*)x, w, eps, (float*)out, n);
+    else if (dt == DT_BF16)
+        rmsnorm_act_kernel<bf16><<<R, threads, 0, stream>>>((const bf16*)x, w, eps, (bf16*)out, n);
+    else
+        LC_CHECK(false, "rmsnorm_act: unknown dtype %d", dt);
+    LC_LAUNCH_CHECK("rmsnorm_act");
+    return 0;
+}
+
+LC_API int lc_qk_norm_rope_write(void* qkv, int dt, int T, int nh, int nkv, int d,
+                                 const float* q_w, const float* k_w, float eps,
+                                 const int* positions, const float* rope_table, int rot,
+                                 void* k_cache, void* v_cache, const int* slots, int page_size,
+                                 hipStream_t stream) {
+    LC_CHECK(T >= 0 && nh > 0 && nkv > 0 && d > 0, "qk_norm_rope_write: bad sizes T=%d nh=%d nkv=%d d=%d",
+             T, nh, nkv, d);
+    if (T == 0) return 0;
+    LC_CHECK(qkv, "qk_norm_rope_write: null qkv");
+    LC_CHECK(rot >= 0 && rot <= d && rot % 2 == 0,
+             "qk_norm_rope_write: rotary dims %d must be even and at most head_dim %d", rot, d);
+    LC_CHECK(!rope_table || positions, "qk_norm_rope_write: rotary table without positions");
+    LC_CHECK(!(k_cache && slots) || (v_cache && page_size > 0),
+             "qk_norm_rope_write: cache write needs v_cache and a page size");
+    if (!rope_table) rot = 0;
+    const int waves = 4;
+    dim3 grid(T, (nh + 2 * nkv + waves - 1) / waves);
+    if (dt == DT_F32)
+        qk_norm_rope_write_kernel<float><<<grid, waves * kWave, 0, stream>>>(
+            (float*)qkv, T, nh, nkv, d, q_w, k_w, eps, positions, rope_table, rot,
+            (float*)k_cache, (float*)v_cache, slots, page_size);
+    else if (dt == DT_BF16)
+        qk_norm_rope_write_kernel<bf16><<<grid, waves * kWave, 0, stream>>>(
+            (bf16*)qkv, T, nh, nkv, d, q_w, k_w, eps, positions, rope_table, rot,
+            (bf16*)k_cache, (bf16*)v_cache, slots, page_size);
+    else
+        LC_CHECK(false, "qk_norm_rope_write: unknown dtype %d", dt);
+    LC_LAUNCH_CHECK("qk_norm_rope_write");
+    return 0;
+}
+
+LC_API int lc_swiglu(const void* gu, void* out, int dt, int T, int I, hipStream_t stream) {
+    LC_CHECK(T >= 0 && I > 0, "swiglu: bad sizes T=%d I=%d", T, I);
+    if (T == 0) return 0;
+    LC_CHECK(gu && out, "swiglu: null pointer");
+    const size_t total = (size_t)T * I;
+    const int threads = 256;
+    size_t blocks = (total + threads - 1) / threads;
+    if (blocks > 65536) blocks = 65536;
+    if (dt == DT_F32)
+        swiglu_kernel<float><<<(int)blocks, threads, 0, stream>>>((const float*)gu, (float*)out, I, total);
+    else if (dt == DT_BF16)
+        swiglu_kernel<bf16><<<(int)blocks, threads, 0, stream>>>((const bf16*)gu, (bf16*)out, I, total);
+    else
+        LC_CHECK(false, "swiglu: unknown dtype %d", dt);
+    LC_LAUNCH_CHECK("swiglu");
+    return 0;
+}

@@ -1,0 +1,173 @@
+"""The description of one step's batch, as the model and its kernels see it.
+
+The reference's ``InputMetadata`` (include/sequence.h:46-61) holds decode tokens first and
+then at most one prompt portion; here a batch is any list of (request, next tokens) entries:
+portions of prompts beside single decoded tokens, in any order and of any length >= 1.
+Everything the kernels index by is built on the host from the cache manager's tables and
+sent to the GPU in one copy.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager
+from ..kernels.ops import AttentionBatch
+
+PREFILL_TILE = 64   # query rows of one work item of the prefill attention kernel
+
+
+@dataclass
+class StepEntry:
+    """A request's next tokens, and the places among them whose logits are wanted."""
+
+    request: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class SiteView:
+    """What one site of the run order sees of the step: the batch and its own cache."""
+
+    batch: "StepBatch"
+    index: int
+    writes_cache: bool
+    page_size: int
+    kv: Optional[Tuple[torch.Tensor, torch.Tensor]] = None   # keys, values [pages, kvh, page, d]
+    attn: Optional[AttentionBatch] = None                    # of this site's page group
+    state: Optional[torch.Tensor] = None                     # [max_seqs, *shape]
+
+
+@dataclass
+class StepBatch:
+    num_tokens: int
+    num_requests: int
+    requests: List[Hashable]
+    q_start: List[int]            # host: token offset of each request in the batch, R + 1 entries
+    first_position: List[int]     # host: cached length of each request before this step
+    slot_list: List[int]          # host: state slot of each request
+    max_position: int
+    token_ids: torch.Tensor       # int32 [T]
+    positions: torch.Tensor       # int32 [T]
+    tok_req: torch.Tensor         # int32 [T]
+    want_rows: torch.Tensor       # int32 [W] rows of the batch whose logits are wanted
+    slot_ids: torch.Tensor        # int32 [R]
+    groups: List[AttentionBatch] = field(default_factory=list)
+    num_wanted: int = 0
+
+
+class _Packer:
+    """Collects int32 arrays, sends them in one copy, and hands out views of the device copy."""
+
+    def __init__(self) -> None:
+        self._arrays: List[np.ndarray] = []
+        self._offsets: List[int] = []
+        self._size = 0
+
+    def add(self, values, shape=None) -> int:
+        arr = np.asarray(values, dtype=np.int32).reshape(-1)
+        self._arrays.append(arr)
+        self._offsets.append(self._size)
+        self._size += int(arr.size)
+        self._size = (self._size + 3) & ~3   # keep every array 16-byte aligned
+        return len(self._arrays) - 1
+
+    def upload(self, device) -> None:
+        host = np.zeros(max(self._size, 4), dtype=np.int32)
+        for arr, off in zip(self._arrays, self._offsets):
+            host[off:off + arr.size] = arr
+        dev = torch.device(device)
+        if dev.type == "cuda":
+            staging = torch.empty(host.size, dtype=torch.int32, pin_memory=True)
+            staging.numpy()[:] = host
+            self._dev = staging.to(dev, non_blocking=True)
+        else:
+            self._dev = torch.from_numpy(host).to(dev)
+
+    def view(self, handle: int, shape=None) -> torch.Tensor:
+        off, n = self._offsets[handle], self._arrays[handle].size
+        t = self._dev[off:off + n]
+        return t.view(shape) if shape is not None else t
+
+
+def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device) -> StepBatch:
+    """Lay the entries out as one flat batch.  Pages for the new tokens must be reserved."""
+    bs = cache.block_size
+    requests, q_start, first_pos, slot_list = [], [0], [], []
+    token_ids: List[int] = []
+    positions: List[int] = []
+    tok_req: List[int] = []
+    want_rows: List[int] = []
+    for r, e in enumerate(entries):
+        n = len(e.tokens)
+        base = cache.length(e.request)
+        requests.append(e.request)
+        first_pos.append(base)
+        slot_list.append(cache.slot(e.request))
+        for w in e.want:
+            if not 0 <= int(w) < n:
+                raise ValueError(f"request {e.request!r}: wanted place {w} is outside its {n} tokens")
+            want_rows.append(q_start[-1] + int(w))
+        token_ids.extend(int(t) for t in e.tokens)
+        positions.extend(range(base, base + n))
+        tok_req.extend([r] * n)
+        q_start.append(q_start[-1] + n)
+    T, R = q_start[-1], len(entries)
+
+    pk = _Packer()
+    h_tok = pk.add(token_ids)
+    h_pos = pk.add(positions)
+    h_req = pk.add(tok_req)
+    h_want = pk.add(want_rows)
+    h_slot = pk.add(slot_list)
+    h_qs = pk.add(q_start)
+
+    ctx_len = [first_pos[r] + (q_start[r + 1] - q_start[r]) for r in range(R)]
+    h_ctx = pk.add(ctx_len)
+    decode_tokens = [q_start[r] for r in range(R) if q_start[r + 1] - q_start[r] == 1]
+    h_dec = pk.add(decode_tokens)
+    tiles: List[int] = []
+    for r in range(R):
+        n = q_start[r + 1] - q_start[r]
+        if n == 1:
+            continue
+        for t0 in range(0, n, PREFILL_TILE):
+            tiles.extend((r, q_start[r] + t0, min(PREFILL_TILE, n - t0), first_pos[r] + t0))
+    h_tiles = pk.add(tiles)
+
+    group_handles = []
+    for gi, g in enumerate(cache.groups):
+        tables = [g.tables[req] for req in requests]
+        mb = max((len(t) for t in tables), default=1) or 1
+        flat = np.full((R, mb), -1, dtype=np.int32)
+        for r, t in enumerate(tables):
+            flat[r, :len(t)] = t
+        slots = np.empty(T, dtype=np.int32)
+        for r in range(R):
+            tab = tables[r]
+            for i in range(q_start[r], q_start[r + 1]):
+                p = positions[i]
+                page = tab[p // bs]
+                slots[i] = page * bs + p % bs if page >= 0 else -1
+        group_handles.append((pk.add(flat), mb, pk.add(slots)))
+
+    pk.upload(device)
+    groups = []
+    for (h_bt, mb, h_sl) in group_handles:
+        groups.append(AttentionBatch(
+            tok_req=pk.view(h_req), positions=pk.view(h_pos),
+            block_table=pk.view(h_bt, (R, mb)), q_start=pk.view(h_qs), ctx_len=pk.view(h_ctx),
+            slots=pk.view(h_sl), num_decode=len(decode_tokens),
+            decode_tokens=pk.view(h_dec), prefill_tiles=pk.view(h_tiles, (len(tiles) // 4, 4)),
+            max_ctx=max(ctx_len, default=0), all_decode=len(decode_tokens) == R))
+    return StepBatch(
+        num_tokens=T, num_requests=R, requests=requests, q_start=q_start,
+        first_position=first_pos, slot_list=slot_list,
+        max_position=max(positions, default=0),
+        token_ids=pk.view(h_tok), positions=pk.view(h_pos), tok_req=pk.view(h_req),
+        want_rows=pk.view(h_want), slot_ids=pk.view(h_slot), groups=groups,
+        num_wanted=len(want_rows))

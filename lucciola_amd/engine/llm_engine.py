@@ -1,0 +1,109 @@
+"""The engine: model runner + scheduler + sampler, stepped synchronously.
+
+``LLMEngine.step`` is one turn of the reference's engine loop (src/async_engine.cc:113-160):
+schedule, run the model, pick tokens, apply the stop rules, free what has finished.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, Dict, List, Optional, Sequence as Seq
+
+import torch
+
+from ..config.engine_config import EngineConfig
+from ..sampling.sampler import Sampler, SamplingParams
+from .loading import load_model, random_model
+from .runner import ModelRunner
+from .scheduler import ScheduledStep, Scheduler
+from .sequence import Sequence
+
+
+@dataclass
+class StepOutput:
+    seq_id: int
+    token: int
+    finished: bool
+
+
+class LLMEngine:
+    def __init__(self, model, model_config, engine_config: EngineConfig):
+        self.model = model
+        self.model_config = model_config
+        self.config = engine_config
+        self.runner = ModelRunner(model, engine_config)
+        self.scheduler = Scheduler(self.runner.cache, engine_config.max_tokens_per_step,
+                                   engine_config.max_seqs,
+                                   max_model_len=model.spec.max_positions)
+        self.sampler = Sampler()
+        self.sequences: Dict[int, Sequence] = {}
+        self._next_id = 1
+        self.eos_token_ids = tuple(getattr(model_config, "eos_token_ids", ()) or ())
+
+    @classmethod
+    def from_folder(cls, model_path: str, engine_config: Optional[EngineConfig] = None):
+        engine_config = engine_config or EngineConfig()
+        model, cfg = load_model(model_path, engine_config.dtype, engine_config.device)
+        return cls(model, cfg, engine_config)
+
+    @classmethod
+    def from_random(cls, config_dict, seed: int, engine_config: Optional[EngineConfig] = None):
+        engine_config = engine_config or EngineConfig()
+        model, cfg = random_model(config_dict, seed, engine_config.dtype, engine_config.device)
+        return cls(model, cfg, engine_config)
+
+    # ------------------------------------------------------------------ requests
+    def add_request(self, prompt_token_ids: Seq[int], params: Optional[SamplingParams] = None) -> int:
+        params = params or SamplingParams()
+        if not params.eos_token_ids and self.eos_token_ids:
+            params.eos_token_ids = self.eos_token_ids
+        V = self.model.vocab_size
+        for t in prompt_token_ids:
+            if not 0 <= int(t) < V:
+                raise ValueError(f"token id {t} is outside the vocabulary of {V}")
+        seq = Sequence(self._next_id, prompt_token_ids, params)
+        self._next_id += 1
+        self.scheduler.add_request(seq)
+        self.sequences[seq.seq_id] = seq
+        return seq.seq_id
+
+    def has_unfinished_requests(self) -> bool:
+        return self.scheduler.has_unfinished_requests()
+
+    # ------------------------------------------------------------------ one step
+    def step(self) -> List[StepOutput]:
+        sched: ScheduledStep = self.scheduler.step()
+        if sched.num_seqs == 0:
+            if self.scheduler.has_unfinished_requests() and not sched.preempted:
+                raise RuntimeError("the scheduler has requests but can run none of them")
+            return []
+        logits = self.runner.step(sched.entries)
+        sampling = [seq for seq, s in zip(sched.seqs, sched.samples) if s]
+        outputs: List[StepOutput] = []
+        if sampling:
+            tokens = self.sampler.sample(logits, [s.params for s in sampling],
+                                         [s.num_generated for s in sampling])
+            for seq, token in zip(sampling, tokens):
+                finished = self.scheduler.on_token(seq, token)
+                if finished:
+                    self.scheduler.free_sequence(seq)
+                outputs.append(StepOutput(seq.seq_id, token, finished))
+        return outputs
+
+    # ------------------------------------------------------------------ whole requests
+    def generate(self, prompts: Seq[Seq[int]], params=None,
+                 on_token: Optional[Callable[[int, int, bool], None]] = None) -> List[List[int]]:
+        """Generate for every prompt (lists of token ids); returns the generated ids of each."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params] * len(prompts)
+        ids = []
+        for prompt, p in zip(prompts, params):
+            p = SamplingParams(**vars(p)) if p is not None else None
+            ids.append(self.add_request(prompt, p))
+        while self.has_unfinished_requests():
+            for out in self.step():
+                if on_token is not None:
+                    on_token(out.seq_id, out.token, out.finished)
+        result = [self.sequences[i].output_token_ids for i in ids]
+        for i in ids:
+            del self.sequences[i]
+        return result

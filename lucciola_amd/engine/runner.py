@@ -1,0 +1,130 @@
+"""The step function: one batch of (request, its next tokens) through the model, from the cache.
+
+``ModelRunner.step`` runs only the tokens it is given, as one batch, and returns float32
+logits at the wanted places.  It is what the scheduler, the entry points and the trace replay
+all call; nothing else runs the model.  The reference's counterpart is
+``QwenModel::step_with_paged_attention`` (src/qwen.cc:801-902), which also picks the next
+token and appends it to the sequences itself; here sampling is a stage of its own.
+"""
+from __future__ import annotations
+
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import torch
+
+from ..cache.manager import CacheManager
+from ..cache.page_pool import OutOfPages
+from ..config.engine_config import EngineConfig
+from ..models.causal_lm import CausalLM
+from .batch import SiteView, StepBatch, StepEntry, build_batch
+
+
+class ModelRunner:
+    def __init__(self, model: CausalLM, config: EngineConfig, num_blocks: Optional[int] = None):
+        self.model = model
+        self.config = config
+        self.device = model.ctx.device
+        needs = model.site_needs()
+        blocks = num_blocks if num_blocks is not None else config.max_blocks
+        if blocks <= 0:
+            blocks = self._blocks_from_free_memory(needs)
+        self.cache = CacheManager(needs, config.block_size, blocks, config.max_seqs)
+        self.cache.allocate_tensors(config.dtype, self.device)
+        self.steps = 0
+        self.tokens = 0
+
+    # ------------------------------------------------------------------ sizing
+    def _blocks_from_free_memory(self, needs) -> int:
+        """As the reference sizes its pools: a fraction of the free memory less a reserve
+        (src/qwen.cc:527-543)."""
+        probe = CacheManager(needs, self.config.block_size, 1, 1)
+        per_block = max(1, probe.bytes_per_block(self.config.dtype))
+        free, _ = torch.cuda.mem_get_info(self.device)
+        usable = int((free - self.config.memory_reserve) * self.config.memory_fraction)
+        blocks = usable // per_block
+        if blocks <= 0:
+            raise RuntimeError(f"no memory for the cache: {free} bytes free, a page of all "
+                               f"layers takes {per_block}")
+        return int(blocks)
+
+    # ------------------------------------------------------------------ the step
+    def can_run(self, entries: Sequence[StepEntry]) -> bool:
+        taken: Dict[int, int] = {}
+        new_requests = 0
+        for e in entries:
+            known = self.cache.has(e.request)
+            if not known:
+                new_requests += 1
+            if not self.cache.can_reserve(e.request if known else None, len(e.tokens), taken):
+                return False
+            have = (self.cache.length(e.request)) if known else 0
+            for gi, g in enumerate(self.cache.groups):
+                taken[gi] = taken.get(gi, 0) + self.cache.pages_needed(g, have, len(e.tokens))
+        return new_requests <= self.cache.slots.num_free()
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run the entries as one batch; returns float32 logits [wanted places, vocab] in the
+        order of the entries and of each entry's ``want``.
+
+        A request that the cache does not know is admitted.  Raises OutOfPages (and changes
+        nothing) if the pages or slots for the whole batch are not there."""
+        entries = [e for e in entries if len(e.tokens) > 0]
+        V = self.model.vocab_size
+        if not entries:
+            return torch.empty((0, V), dtype=torch.float32, device=self.device)
+        seen = set()
+        limit = self.model.spec.max_positions
+        for e in entries:
+            if e.request in seen:
+                raise ValueError(f"request {e.request!r} appears twice in one step")
+            seen.add(e.request)
+            for t in e.tokens:
+                if not 0 <= int(t) < V:
+                    raise ValueError(f"request {e.request!r}: token id {t} is outside the "
+                                     f"vocabulary of {V}")
+            have = self.cache.length(e.request) if self.cache.has(e.request) else 0
+            if limit and have + len(e.tokens) > limit:
+                raise ValueError(f"request {e.request!r}: {have + len(e.tokens)} tokens exceed "
+                                 f"the model's {limit} positions")
+        if not self.can_run(entries):
+            raise OutOfPages(f"the cache cannot take this step ({sum(len(e.tokens) for e in entries)}"
+                             f" tokens of {len(entries)} requests; "
+                             f"{self.cache.num_free_blocks()} pages free)")
+        fresh: List[int] = []
+        for e in entries:
+            if not self.cache.has(e.request):
+                self.cache.admit(e.request)
+            if self.cache.length(e.request) == 0:
+                fresh.append(self.cache.slot(e.request))
+            self.cache.reserve(e.request, len(e.tokens))
+        for site, state in self.cache.state.items():
+            for slot in fresh:
+                state[slot].zero_()
+
+        batch = build_batch(entries, self.cache, self.device)
+        logits = self.model.forward(batch, self._sites(batch))
+        for e in entries:
+            self.cache.commit(e.request)
+        self.steps += 1
+        self.tokens += batch.num_tokens
+        return logits
+
+    def _sites(self, batch: StepBatch) -> List[SiteView]:
+        sites = []
+        cache = self.cache
+        for index, entry in enumerate(self.model.spec.run_order):
+            owner = index if entry.cache_of is None else entry.cache_of
+            view = SiteView(batch=batch, index=index, writes_cache=entry.cache_of is None,
+                            page_size=cache.block_size)
+            if owner in cache.kv:
+                view.kv = cache.kv[owner]
+                view.attn = batch.groups[cache.site_group[owner]]
+            if owner in cache.state:
+                view.state = cache.state[owner]
+            sites.append(view)
+        return sites
+
+    def finish(self, request: Hashable) -> None:
+        """The request is over: its pages and its slot go back."""
+        if self.cache.has(request):
+            self.cache.release(request)

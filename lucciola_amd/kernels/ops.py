@@ -1,0 +1,307 @@
+"""The kernels as Python functions over torch tensors that live on the GPU.
+
+Every function here launches hand-written gfx950 code from ``liblucciola_hip.so`` on the
+current HIP stream; there is no other implementation behind these names.  Loading fails loudly
+if the library cannot be built or opened.  Parts call these through the module
+(``ops.gemm(...)``), never by importing the names.
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from ..csrc import build as _build
+
+_lib = None
+
+DT_F32, DT_BF16 = 0, 1
+
+# argument kinds: p pointer, i int, f float
+_ARG = {"p": ctypes.c_void_p, "i": ctypes.c_int, "f": ctypes.c_float}
+_SIGNATURES = {
+    "lc_embedding": "ppipiiip",
+    "lc_rmsnorm": "ppppfpiiiip",
+    "lc_rmsnorm_act": "ppfpiiip",
+    "lc_gemm_generic": "pipipiiiip",
+    "lc_qk_norm_rope_write": "piiiiippfppipppip",
+    "lc_attention_generic": "pipppipppiiiiiifip",
+    "lc_swiglu": "ppiiip",
+    "lc_sample": "ppppiip",
+}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return DT_F32
+    if t.dtype == torch.bfloat16:
+        return DT_BF16
+    raise KernelError(f"kernels take float32 or bfloat16 tensors, got {t.dtype}")
+
+
+def library():
+    """The loaded kernel library (built at the first call if there is no current build)."""
+    global _lib
+    if _lib is None:
+        path = _build.library_path(build_if_needed=True)
+        try:
+            lib = ctypes.CDLL(path)
+        except OSError as exc:
+            raise KernelError(f"cannot load the kernel library {path}: {exc}") from exc
+        lib.lc_last_error.restype = ctypes.c_char_p
+        for name, sig in _SIGNATURES.items():
+            fn = getattr(lib, name, None)
+            if fn is None:
+                raise KernelError(f"the kernel library {path} lacks the entry point {name}")
+            fn.restype = ctypes.c_int
+            fn.argtypes = [_ARG[c] for c in sig]
+        _lib = lib
+    return _lib
+
+
+def library_file() -> str:
+    library()
+    return _build.library_path(build_if_needed=False)
+
+
+def _call(name: str, *args) -> None:
+    lib = library()
+    fn = getattr(lib, name)
+    rc = fn(*args)
+    if rc != 0:
+        raise KernelError(lib.lc_last_error().decode("utf-8", "replace"))
+
+
+def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    if t is None:
+        return ctypes.c_void_p(0)
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(t: torch.Tensor, what: str, dtype=None, dim: Optional[int] = None) -> None:
+    if not t.is_cuda:
+        raise KernelError(f"{what}: tensor must be on the GPU (is on {t.device})")
+    if not t.is_contiguous():
+        raise KernelError(f"{what}: tensor must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{what}: expected {dtype}, got {t.dtype}")
+    if dim is not None and t.dim() != dim:
+        raise KernelError(f"{what}: expected {dim} dimensions, got shape {tuple(t.shape)}")
+
+
+_c_int, _c_float = ctypes.c_int, ctypes.c_float
+
+
+# ------------------------------------------------------------------------------ embedding
+def embedding(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """float32 [T, H] rows of ``table`` [V, H] picked by int32 ``ids`` [T]."""
+    _need(ids, "embedding ids", torch.int32, 1)
+    _need(table, "embedding table", None, 2)
+    T, (V, H) = ids.shape[0], table.shape
+    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    _call("lc_embedding", _ptr(ids), _ptr(table), _c_int(_dt(table)), _ptr(out), _c_int(T),
+          _c_int(H), _c_int(V), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------ norms
+def rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+            out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """RMSNorm of the float32 residual stream ``h`` [T, n], with the pending branch output
+    ``delta`` [T, n] added first.
+
+    Without ``rows``: ``h += delta`` in place and every row is normed.  With ``rows`` (int32
+    [R]): only those rows are normed (``h`` stays as it is) and the result is [R, n].
+    """
+    _need(h, "rmsnorm h", torch.float32, 2)
+    _need(weight, "rmsnorm weight", torch.float32, 1)
+    T, n = h.shape
+    if weight.shape[0] != n:
+        raise KernelError(f"rmsnorm: weight has {weight.shape[0]} entries for rows of {n}")
+    if delta is not None:
+        _need(delta, "rmsnorm delta", out_dtype, 2)
+        if tuple(delta.shape) != (T, n):
+            raise KernelError(f"rmsnorm: delta {tuple(delta.shape)} does not match h {(T, n)}")
+    if rows is not None:
+        _need(rows, "rmsnorm rows", torch.int32, 1)
+    R = T if rows is None else rows.shape[0]
+    out = torch.empty((R, n), dtype=out_dtype, device=h.device)
+    _call("lc_rmsnorm", _ptr(h), _ptr(delta), _ptr(rows), _ptr(weight), _c_float(eps), _ptr(out),
+          _c_int(_dt(out)), _c_int(R), _c_int(n),
+          _c_int(1 if (rows is None and delta is not None) else 0), _stream())
+    return out
+
+
+def rmsnorm_act(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """RMSNorm over the last dimension of an activation tensor."""
+    _need(x, "rmsnorm_act x")
+    _need(weight, "rmsnorm_act weight", torch.float32, 1)
+    n = x.shape[-1]
+    if weight.shape[0] != n:
+        raise KernelError(f"rmsnorm_act: weight has {weight.shape[0]} entries for rows of {n}")
+    out = torch.empty_like(x)
+    _call("lc_rmsnorm_act", _ptr(x), _ptr(weight), _c_float(eps), _ptr(out), _c_int(_dt(x)),
+          _c_int(x.numel() // n), _c_int(n), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------ products
+def gemm(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``x`` [M, K] times ``w`` [N, K] transposed -> [M, N]; float32 accumulation."""
+    _need(x, "gemm x", None, 2)
+    _need(w, "gemm w", None, 2)
+    M, K = x.shape
+    N, K2 = w.shape
+    if K != K2:
+        raise KernelError(f"gemm: x is [{M}, {K}] but w is [{N}, {K2}]")
+    out_dtype = out_dtype or x.dtype
+    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    if M == 0:
+        return out
+    if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and _fast_gemm_ok(M, N, K)):
+        _call("lc_gemm_bf16", _ptr(x), _ptr(w), _ptr(out), _c_int(_dt(out)), _c_int(M), _c_int(N),
+              _c_int(K), _stream())
+    else:
+        _call("lc_gemm_generic", _ptr(x), _c_int(_dt(x)), _ptr(w), _c_int(_dt(w)), _ptr(out),
+              _c_int(_dt(out)), _c_int(M), _c_int(N), _c_int(K), _stream())
+    return out
+
+
+def _fast_gemm_ok(M: int, N: int, K: int) -> bool:
+    lib = library()
+    fn = getattr(lib, "lc_gemm_bf16_supported", None)
+    return bool(fn and fn(_c_int(M), _c_int(N), _c_int(K)))
+
+
+# ------------------------------------------------------------------------------ attention
+def qk_norm_rope_write(qkv: torch.Tensor, nh: int, nkv: int, d: int,
+                       q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
+                       eps: float, positions: Optional[torch.Tensor],
+                       rope_table: Optional[torch.Tensor],
+                       k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                       slots: Optional[torch.Tensor], page_size: int) -> None:
+    """In place on ``qkv`` [T, (nh + 2 nkv) d]: per-head RMSNorm of q and k (if weights are
+    given), rotation by ``rope_table`` [positions, rot] (cos | sin halves) at each token's
+    position, and the write of k and v into their cache slot ``slots`` [T]
+    (page * page_size + offset; negative: no write).  Caches are [pages, nkv, page_size, d]."""
+    _need(qkv, "qkv", None, 2)
+    T = qkv.shape[0]
+    if qkv.shape[1] != (nh + 2 * nkv) * d:
+        raise KernelError(f"qkv has {qkv.shape[1]} columns, expected {(nh + 2 * nkv) * d}")
+    rot = 0
+    if rope_table is not None:
+        _need(rope_table, "rope table", torch.float32, 2)
+        _need(positions, "positions", torch.int32, 1)
+        rot = rope_table.shape[1]
+        if positions.shape[0] != T:
+            raise KernelError("positions do not match the tokens")
+    for wt, name in ((q_weight, "q norm weight"), (k_weight, "k norm weight")):
+        if wt is not None:
+            _need(wt, name, torch.float32, 1)
+            if wt.shape[0] != d:
+                raise KernelError(f"{name} has {wt.shape[0]} entries for head size {d}")
+    if k_cache is not None and slots is not None:
+        _need(k_cache, "k cache", qkv.dtype, 4)
+        _need(v_cache, "v cache", qkv.dtype, 4)
+        _need(slots, "slots", torch.int32, 1)
+        if tuple(k_cache.shape[1:]) != (nkv, page_size, d) or k_cache.shape != v_cache.shape:
+            raise KernelError(f"cache shape {tuple(k_cache.shape)} does not fit "
+                              f"[pages, {nkv}, {page_size}, {d}]")
+        if slots.shape[0] != T:
+            raise KernelError("slots do not match the tokens")
+    else:
+        k_cache = v_cache = slots = None
+    _call("lc_qk_norm_rope_write", _ptr(qkv), _c_int(_dt(qkv)), _c_int(T), _c_int(nh), _c_int(nkv),
+          _c_int(d), _ptr(q_weight), _ptr(k_weight), _c_float(eps), _ptr(positions),
+          _ptr(rope_table), _c_int(rot), _ptr(k_cache), _ptr(v_cache), _ptr(slots),
+          _c_int(page_size), _stream())
+
+
+@dataclass
+class AttentionBatch:
+    """What attention needs to know of a step's batch, for one group of cache pages.
+
+    All tensors are int32 on the GPU.  ``tok_req[t]`` is the row of ``block_table`` that token
+    t belongs to; ``positions[t]`` its absolute position; ``block_table`` [R, max_blocks] maps
+    position // page_size to a page.  ``q_start`` [R + 1] are the requests' token offsets in
+    the batch, ``ctx_len`` [R] their cached lengths after this step.  ``decode_rows`` and
+    ``prefill_tiles`` list the work of the decode and prefill kernels (None: not prepared).
+    """
+
+    tok_req: torch.Tensor
+    positions: torch.Tensor
+    block_table: torch.Tensor
+    q_start: Optional[torch.Tensor] = None
+    ctx_len: Optional[torch.Tensor] = None
+    slots: Optional[torch.Tensor] = None
+    num_decode: int = 0
+    decode_tokens: Optional[torch.Tensor] = None   # [ND] token rows of length-1 portions
+    prefill_tiles: Optional[torch.Tensor] = None   # [NT, 4]: request, first token row, rows, first position
+    max_ctx: int = 0                               # longest cached length in the batch
+    all_decode: bool = False
+
+
+def attention(qkv: torch.Tensor, batch: AttentionBatch, k_cache: torch.Tensor,
+              v_cache: torch.Tensor, nh: int, nkv: int, d: int, page_size: int, scale: float,
+              window: int = 0) -> torch.Tensor:
+    """Causal attention of the q heads in ``qkv`` [T, (nh + 2 nkv) d] over the cached keys and
+    values (the step's own have been written already) -> [T, nh d]."""
+    _need(qkv, "qkv", None, 2)
+    _need(k_cache, "k cache", qkv.dtype, 4)
+    _need(v_cache, "v cache", qkv.dtype, 4)
+    T = qkv.shape[0]
+    out = torch.empty((T, nh * d), dtype=qkv.dtype, device=qkv.device)
+    if T == 0:
+        return out
+    _need(batch.tok_req, "tok_req", torch.int32, 1)
+    _need(batch.positions, "positions", torch.int32, 1)
+    _need(batch.block_table, "block table", torch.int32, 2)
+    if tuple(k_cache.shape[1:]) != (nkv, page_size, d):
+        raise KernelError(f"cache shape {tuple(k_cache.shape)} does not fit "
+                          f"[pages, {nkv}, {page_size}, {d}]")
+    _call("lc_attention_generic", _ptr(qkv), _c_int(qkv.shape[1]), _ptr(k_cache), _ptr(v_cache),
+          _ptr(out), _c_int(_dt(qkv)), _ptr(batch.tok_req), _ptr(batch.positions),
+          _ptr(batch.block_table), _c_int(batch.block_table.shape[1]), _c_int(T), _c_int(nh),
+          _c_int(nkv), _c_int(d), _c_int(page_size), _c_float(scale), _c_int(window), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------ feed-forward
+def swiglu(gu: torch.Tensor) -> torch.Tensor:
+    """``gu`` [T, 2 I] (gate columns, then up columns) -> silu(gate) * up, [T, I]."""
+    _need(gu, "swiglu input", None, 2)
+    T, two_i = gu.shape
+    if two_i % 2:
+        raise KernelError("swiglu: the input needs an even number of columns")
+    out = torch.empty((T, two_i // 2), dtype=gu.dtype, device=gu.device)
+    _call("lc_swiglu", _ptr(gu), _ptr(out), _c_int(_dt(gu)), _c_int(T), _c_int(two_i // 2), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------ sampling
+def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,
+           uniform: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Token ids (int32 [R]) from float32 ``logits`` [R, V]: greedy where the row's temperature
+    is <= 0 (or none is given), else inverse-CDF sampling of softmax(logits / temperature) with
+    the row's uniform number in [0, 1)."""
+    _need(logits, "logits", torch.float32, 2)
+    R, V = logits.shape
+    if temperature is not None:
+        _need(temperature, "temperature", torch.float32, 1)
+        _need(uniform, "uniform", torch.float32, 1)
+        if temperature.shape[0] != R or uniform.shape[0] != R:
+            raise KernelError("sample: one temperature and one uniform number per row")
+    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    _call("lc_sample", _ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(out), _c_int(R),
+          _c_int(V), _stream())
+    return out

@@ -1,0 +1,2 @@
+"""Architectures: importing this package registers them."""
+from . import qwen3  # noqa: F401

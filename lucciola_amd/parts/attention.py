@@ -1,0 +1,89 @@
+"""Grouped-query attention over the paged cache, as a part.
+
+Order of operations as in the reference's layer (src/qwen.cc:592-738): q, k, v projections
+(one product here, the weights are stacked at load) -> RMSNorm over head_dim on every q and k
+head with one [d] weight each -> rotary embedding of q and k -> k, v written to the cache ->
+causal attention over all cached keys (kv head = h / (nh / nkv), scale 1/sqrt(d)) -> output
+projection.  Sizes, the scale, the norm, the position encoding and an optional window are
+parameters; nh * d need not equal the hidden size.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..cache.specs import PagedKV
+from ..config.registry import MIXERS, NORMS, POSITION_ENCODINGS
+from ..config.specs import PartSpec
+from ..kernels import ops
+from ..weights.loader import ParamDecl
+from .base import BuildContext, Part, build_part
+from .feed_forward import stack_rows
+
+
+@MIXERS.register("attention")
+class Attention(Part):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 scale: Optional[float] = None, qk_norm: Optional[PartSpec] = None,
+                 position: Optional[PartSpec] = None, window: Optional[int] = None):
+        super().__init__(hidden_size=hidden_size, num_heads=num_heads, num_kv_heads=num_kv_heads,
+                         head_dim=head_dim, scale=scale, qk_norm=qk_norm, position=position,
+                         window=window)
+        if num_heads % num_kv_heads:
+            raise ValueError(f"attention: {num_heads} heads are not a multiple of "
+                             f"{num_kv_heads} kv heads")
+        self.H, self.nh, self.nkv, self.d = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
+        self.scale = float(scale) if scale is not None else self.d ** -0.5
+        self.window = int(window) if window else None
+        self.q_norm = build_part(NORMS, qk_norm) if qk_norm else None
+        self.k_norm = build_part(NORMS, qk_norm) if qk_norm else None
+        self.position = build_part(POSITION_ENCODINGS, position) if position else None
+
+    def declare(self) -> Dict[str, ParamDecl]:
+        out = {"q_proj": ParamDecl((self.nh * self.d, self.H)),
+               "k_proj": ParamDecl((self.nkv * self.d, self.H)),
+               "v_proj": ParamDecl((self.nkv * self.d, self.H)),
+               "o_proj": ParamDecl((self.H, self.nh * self.d))}
+        if self.q_norm is not None:
+            for name, decl in self.q_norm.declare().items():
+                out["q_norm." + name] = decl
+            for name, decl in self.k_norm.declare().items():
+                out["k_norm." + name] = decl
+        return out
+
+    def bind(self, tensors, ctx: BuildContext) -> None:
+        self.qkv = stack_rows([tensors["q_proj"], tensors["k_proj"], tensors["v_proj"]])
+        self.o = tensors["o_proj"]
+        self.dtype = ctx.dtype
+        if self.q_norm is not None:
+            self.q_norm.bind({k[7:]: v for k, v in tensors.items() if k.startswith("q_norm.")}, ctx)
+            self.k_norm.bind({k[7:]: v for k, v in tensors.items() if k.startswith("k_norm.")}, ctx)
+            if self.q_norm.fused_rms() is None:
+                raise NotImplementedError("attention: the q/k norm must offer fused_rms()")
+        if self.position is not None:
+            self.position.bind({}, ctx)
+
+    def cache_need(self):
+        return PagedKV(self.nkv, self.d, self.window)
+
+    def forward(self, x: torch.Tensor, site) -> torch.Tensor:
+        qkv = ops.gemm(x, self.qkv, self.dtype)
+        attn = site.attn
+        q_w = k_w = None
+        eps = 0.0
+        if self.q_norm is not None:
+            q_w, eps = self.q_norm.fused_rms()
+            k_w, _ = self.k_norm.fused_rms()
+        table = None
+        if self.position is not None:
+            table = self.position.rotary_table(site.batch.max_position)
+            if table is None:
+                self.position.apply(qkv, self.nh, self.nkv, self.d, attn.positions)
+        k_cache, v_cache = site.kv
+        ops.qk_norm_rope_write(qkv, self.nh, self.nkv, self.d, q_w, k_w, eps, attn.positions, table,
+                               k_cache, v_cache, attn.slots if site.writes_cache else None,
+                               site.page_size)
+        o = ops.attention(qkv, attn, k_cache, v_cache, self.nh, self.nkv, self.d, site.page_size,
+                          self.scale, self.window or 0)
+        return ops.gemm(o, self.o, self.dtype)

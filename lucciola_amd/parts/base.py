@@ -1,0 +1,73 @@
+"""What every part of a layer has in common, and the residual stream that blocks pass along.
+
+A part is built from its sizes and constants alone (``PartSpec.params``), declares the tensors
+it wants under logical names, and gets them in ``bind``.  No part knows which model it is in
+or what the checkpoint calls its tensors: the architecture maps logical names to checkpoint
+names (``LayerSpec.names``).
+
+Interfaces (all tensors on the GPU; "act" is the engine's activation dtype):
+  Norm            add_norm(stream) -> act [T, n]; add_norm_rows(stream, rows) -> act [R, n];
+                  fused_rms() -> (weight float32 [n], eps) or None
+  PositionEncoding  rotary_table(max_position) -> float32 [positions, rot] or None;
+                  apply(qkv, nh, nkv, d, positions) in place, when there is no table
+  Mixer           forward(x act [T, H], site: SiteView) -> act [T, H]; cache_need() -> spec
+  FeedForward     forward(x act [T, H]) -> act [T, H]
+  Block           forward(stream, site) -> None (updates the stream)
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Dict, Optional
+
+import torch
+
+from ..config.registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Registry)
+from ..config.specs import PartSpec
+from ..weights.loader import ParamDecl
+
+
+@dataclass
+class BuildContext:
+    dtype: torch.dtype      # activation dtype of the engine: bfloat16 or float32
+    device: torch.device
+
+
+class ResidualStream:
+    """The float32 residual stream ``h`` [T, H] and the branch output that is still to be added.
+
+    The sum h + pending is formed in float32 inside the next norm's kernel (the reference adds
+    in float32 and rounds the stream to bf16, src/kernels/add.cu:11-14; here the stream itself
+    stays float32)."""
+
+    def __init__(self, h: torch.Tensor):
+        self.h = h
+        self.pending: Optional[torch.Tensor] = None
+
+
+class Part:
+    """Base of all parts.  Subclasses set ``self.p`` from keyword parameters in ``__init__``."""
+
+    def __init__(self, **params: Any):
+        self.params = dict(params)
+
+    def declare(self) -> Dict[str, ParamDecl]:
+        """Logical tensor name -> declaration."""
+        return {}
+
+    def bind(self, tensors: Dict[str, torch.Tensor], ctx: BuildContext) -> None:
+        """Take the declared tensors (already on the device, in their kept dtype)."""
+
+    def cache_need(self):
+        """Mixers: a cache spec (PagedKV, FixedState) or None."""
+        return None
+
+
+def build_part(registry: Registry, spec: PartSpec) -> Part:
+    cls = registry.get(spec.kind)
+    return cls(**spec.params)
+
+
+def require(params: Dict[str, Any], *keys: str, part: str) -> None:
+    missing = [k for k in keys if k not in params]
+    if missing:
+        raise TypeError(f"{part}: missing parameters {missing}")
