@@ -20,55 +20,12 @@ from lucciola_amd.weights.random_init import random_tensors
 from lucciola_amd.config.registry import architecture_for
 
 
+from helpers import compare, make_runner, prompts_for, random_weights, replay
+
+
 def make(cfg, seed, page, blocks, dtype="float32"):
-    arch = architecture_for(cfg)
-    spec = arch.model_spec(arch.read_config(cfg))
-    weights = dict(random_tensors(declared_tensors(spec), seed, cfg["initializer_range"],
-                                  torch.bfloat16))
-    from lucciola_amd.engine.loading import _build
-    from lucciola_amd.weights.loader import DictSource
-    model = _build(spec, DictSource(weights), dtype, "cpu")
-    runner = ModelRunner(model, EngineConfig(dtype=dtype, block_size=page, max_blocks=blocks,
-                                             max_seqs=4, device="cpu"))
-    return runner, weights
-
-
-def prompts_for(cfg, lengths, seed):
-    rng = random.Random(seed)
-    return {f"r{i}": [rng.randrange(cfg["vocab_size"]) for _ in range(n)]
-            for i, n in enumerate(lengths)}
-
-
-def replay(runner, steps):
-    got = {}
-    fed = {}
-    for entries, end in steps:
-        logits = runner.step([StepEntry(n, t, w) for n, t, w in entries])
-        row = 0
-        for name, tokens, want in entries:
-            base = fed.get(name, 0)
-            for w in want:
-                got[(name, base + w)] = logits[row].double()
-                row += 1
-            fed[name] = base + len(tokens)
-        for name in end:
-            runner.finish(name)
-            fed.pop(name, None)
-        runner.cache.check()
-    return got
-
-
-def compare(got, cfg, weights, prompts, tol):
-    worst = 0.0
-    for name, ids in prompts.items():
-        ref = plain_qwen3.forward(cfg, weights, ids)
-        for (n, pos), row in got.items():
-            if n != name:
-                continue
-            err = float((row - ref[pos]).abs().max() / ref[pos].abs().max())
-            worst = max(worst, err)
-            assert err < tol, f"{name} position {pos}: relative error {err:.3e}"
-    return worst
+    weights = random_weights(cfg, seed)
+    return make_runner(cfg, weights, page, blocks, dtype, "cpu"), weights
 
 
 @pytest.mark.parametrize("key", ["A", "B", "C"])

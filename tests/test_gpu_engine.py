@@ -1,0 +1,192 @@
+"""The engine on the GPU against the plain implementation, in float32 and in bfloat16: each
+request alone and whole; most of it in one step and the last 32 tokens one by one; portions of
+changing size; mixed batches with so few pages that they are used again; long decoding; the
+first tokens of a sequence; generation through the entry points; trace replay."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import configs
+import plain_qwen3
+import traces
+from helpers import compare, make_runner, prompts_for, random_weights, replay
+from lucciola_amd.config.engine_config import EngineConfig
+from lucciola_amd.engine.llm_engine import LLMEngine
+from lucciola_amd.engine.loading import _build, load_model
+from lucciola_amd.config.registry import architecture_for
+from lucciola_amd.sampling.sampler import SamplingParams, uniform_for
+from lucciola_amd.weights.loader import DictSource
+from lucciola_amd.weights.random_init import write_model_folder
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+# error of a row of logits: max |difference| / max |logit|
+TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+LENGTHS = {"A": [5, 11, 17, 40, 130], "B": [1, 9, 30, 64, 45, 200], "C": [70, 33, 50, 3, 61, 150]}
+
+_cache = {}
+
+
+def case(key):
+    if key not in _cache:
+        cfg, page, seed = configs.ALL[key]
+        weights = random_weights(cfg, seed)
+        prompts = prompts_for(cfg, LENGTHS[key], seed)
+        refs = {n: plain_qwen3.forward(cfg, weights, ids) for n, ids in prompts.items()}
+        _cache[key] = (cfg, page, weights, prompts, refs)
+    return _cache[key]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["A", "B", "C"])
+@pytest.mark.parametrize("family", ["whole", "tail", "chunked", "mixed"])
+def test_replay_families(dtype, key, family):
+    cfg, page, weights, prompts, refs = case(key)
+    steps = {"whole": traces.whole, "tail": traces.tail_decode, "chunked": traces.chunked,
+             "mixed": traces.mixed}[family](prompts)
+    blocks = traces.max_live_tokens(steps, page) // page
+    runner = make_runner(cfg, weights, page, blocks, dtype, DEV)
+    got = replay(runner, steps)
+    assert len(got) == sum(len(p) for p in prompts.values())
+    worst = compare(got, cfg, weights, prompts, TOL[dtype], refs)
+    print(f"{key} {family} {dtype}: worst relative error {worst:.3e}")
+    assert not runner.cache.requests
+    for g in runner.cache.groups:
+        assert g.pool.num_free() == blocks
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_pages_reused_with_stale_contents(dtype):
+    """Requests run one after the other in a pool that holds only one of them, after the pool
+    has been filled with large values: what a page held before must never show."""
+    cfg, page, weights, prompts, refs = case("B")
+    steps = traces.chunked(prompts, sizes=(9, 2, 30))
+    blocks = traces.max_live_tokens(steps, page) // page
+    runner = make_runner(cfg, weights, page, blocks, dtype, DEV)
+    for k, v in runner.cache.kv.values():
+        k.fill_(300.0)
+        v.fill_(-300.0)
+    compare(replay(runner, steps), cfg, weights, prompts, TOL[dtype], refs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["A", "C"])
+def test_long_decoding(dtype, key):
+    cfg, page, seed = configs.ALL[key]
+    weights = random_weights(cfg, seed)
+    prompts = prompts_for(cfg, [700], seed + 10)
+    steps = traces.tail_decode(prompts, tail=660)
+    runner = make_runner(cfg, weights, page, -(-700 // page), dtype, DEV)
+    compare(replay(runner, steps, check=False), cfg, weights, prompts, TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["A", "B", "C"])
+def test_first_tokens(dtype, key):
+    cfg, page, seed = configs.ALL[key]
+    weights = random_weights(cfg, seed)
+    prompts = prompts_for(cfg, [1, 2, 3, 4], seed + 20)
+    for family in (traces.whole, lambda p: traces.tail_decode(p, tail=3)):
+        runner = make_runner(cfg, weights, page, 8, dtype, DEV)
+        compare(replay(runner, family(prompts)), cfg, weights, prompts, TOL[dtype])
+
+
+def engine_for(cfg, weights, page, blocks, dtype, **kw):
+    arch = architecture_for(cfg)
+    config = arch.read_config(cfg)
+    model = _build(arch.model_spec(config), DictSource(weights), dtype, DEV)
+    return LLMEngine(model, config, EngineConfig(dtype=dtype, block_size=page, max_blocks=blocks,
+                                                 device=DEV, **kw))
+
+
+@pytest.mark.parametrize("key", ["A", "B", "C"])
+def test_greedy_generation_through_the_engine(key):
+    cfg, page, seed = configs.ALL[key]
+    weights = random_weights(cfg, seed, std=0.3)
+    prompts = list(prompts_for(cfg, [5, 11, 17], seed + 30).values())
+    engine = engine_for(cfg, weights, page, 64, "float32", max_tokens_per_step=16, max_seqs=4)
+    got = engine.generate(prompts, SamplingParams(max_new_tokens=8))
+    want = [plain_qwen3.greedy(cfg, weights, p, 8) for p in prompts]
+    assert got == want
+    engine.runner.cache.check()
+    assert not engine.runner.cache.requests
+
+
+def test_generation_survives_preemption():
+    """With so few pages that running requests are preempted and recomputed, the generated
+    tokens are those of an engine with plenty of pages."""
+    cfg, page, seed = configs.ALL["A"]
+    weights = random_weights(cfg, seed, std=0.3)
+    prompts = list(prompts_for(cfg, [9, 14, 6, 11], seed + 40).values())
+    roomy = engine_for(cfg, weights, page, 200, "float32", max_tokens_per_step=12, max_seqs=4)
+    want = roomy.generate(prompts, SamplingParams(max_new_tokens=20))
+    tight = engine_for(cfg, weights, page, 18, "float32", max_tokens_per_step=12, max_seqs=4)
+    got = tight.generate(prompts, SamplingParams(max_new_tokens=20))
+    assert tight.scheduler.num_preemptions > 0
+    assert got == want
+    tight.runner.cache.check()
+
+
+def test_temperature_sampling_through_the_engine():
+    cfg, page, seed = configs.ALL["B"]
+    weights = random_weights(cfg, seed, std=0.3)
+    prompts = list(prompts_for(cfg, [1, 9, 30], seed + 50).values())
+    engine = engine_for(cfg, weights, page, 64, "float32", max_tokens_per_step=16, max_seqs=4)
+    params = [SamplingParams(max_new_tokens=12, temperature=0.7, seed=100 + i) for i in range(3)]
+    got = engine.generate(prompts, params)
+    for prompt, p, tokens in zip(prompts, params, got):
+        ids = list(prompt)
+        for i, tok in enumerate(tokens):
+            logits = plain_qwen3.forward(cfg, weights, ids)[-1]
+            want = plain_qwen3.sample_token(logits, 0.7, uniform_for(p.seed, i))
+            if tok != want:   # only a rounding neighbour of the CDF boundary may differ
+                pr = torch.softmax(logits / 0.7, 0).cumsum(0)
+                assert abs(float(pr[min(tok, want)]) - uniform_for(p.seed, i)) < 1e-4
+            ids.append(tok)
+    # the same request alone gives the same tokens: the draw does not depend on the batch
+    alone = engine.generate([prompts[1]], [params[1]])
+    assert alone[0] == got[1]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(tmp_path, dtype):
+    cfg, page, seed = configs.ALL["C"]
+    folder = write_model_folder(str(tmp_path / "model"), cfg, seed)
+    model, _ = load_model(folder, "float32", "cpu") if False else (None, None)
+    from lucciola_amd.weights.safetensors_io import SafetensorsFile
+    with SafetensorsFile(os.path.join(folder, "model.safetensors")) as f:
+        weights = {n: f.get(n).clone() for n in f.names()}
+    prompts = prompts_for(cfg, [70, 33, 50, 3, 61], seed)
+    steps = traces.mixed(prompts, seed=3)
+    lines, index = [], {}
+    fed = {}
+    for i, (entries, end) in enumerate(steps):
+        lines.append(json.dumps({"step": i, "end": end, "entries": [
+            {"id": n, "tokens": t, "want": w} for n, t, w in entries]}))
+        rows = []
+        for n, t, w in entries:
+            rows += [(n, fed.get(n, 0) + k) for k in w]
+            fed[n] = fed.get(n, 0) + len(t)
+        index[i] = rows
+    out = tmp_path / "out"
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder,
+                           "--dtype", dtype, "--out", str(out), "--max-tokens",
+                           str(traces.max_live_tokens(steps, 64))],
+                          input="\n".join(lines) + "\n", text=True, capture_output=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split() == [x for i in range(len(steps)) for x in ("done", str(i))]
+    import numpy as np
+    got = {}
+    for i, rows in index.items():
+        if not rows:
+            assert not (out / f"{i}.f32").exists()
+            continue
+        data = np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(len(rows), cfg["vocab_size"])
+        for r, key in enumerate(rows):
+            got[key] = torch.from_numpy(data[r].astype("float64"))
+    compare(got, cfg, weights, prompts, TOL[dtype])

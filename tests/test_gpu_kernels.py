@@ -1,0 +1,223 @@
+"""Each kernel alone against its plain torch version (tests/reference_ops.py), at sizes other
+than the tiny models': widths and vocabularies that are no power of two, head sizes in steps
+of 16, odd head counts and groups, several page sizes, in float32 and bfloat16."""
+import random
+
+import pytest
+import torch
+
+import reference_ops as ref
+from lucciola_amd.kernels import ops
+from lucciola_amd.kernels.ops import AttentionBatch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype):
+    return dict(rtol=2e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1e-3)
+
+
+def close(got, want, dtype, scale=1.0):
+    t = tol(dtype)
+    torch.testing.assert_close(got.double().cpu(), want.double().cpu(), rtol=t["rtol"],
+                               atol=t["atol"] * scale)
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,H,V", [(1, 16, 7), (5, 200, 331), (130, 1000, 50)])
+def test_embedding(dtype, T, H, V):
+    table = rnd(V, H, dtype=dtype, seed=1)
+    ids = torch.randint(0, V, (T,), generator=torch.Generator().manual_seed(2)).int().to(DEV)
+    got = ops.embedding(ids, table)
+    assert got.dtype == torch.float32
+    assert torch.equal(got, ref.embedding(ids, table))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,n", [(1, 16), (7, 200), (33, 1000), (3, 4100)])
+def test_rmsnorm_with_residual(dtype, T, n):
+    h = rnd(T, n, seed=3, scale=2.0)
+    delta = rnd(T, n, dtype=dtype, seed=4)
+    w = 1 + rnd(n, seed=5, scale=0.1)
+    h_ref = h.clone()
+    want = ref.rmsnorm(h_ref, delta, w, 1e-5, dtype)
+    got = ops.rmsnorm(h, delta, w, 1e-5, dtype)
+    torch.testing.assert_close(h, h_ref, rtol=1e-6, atol=1e-6)     # the stream took the sum
+    close(got, want, dtype)
+    # without a pending branch, and at chosen rows only (the stream must stay untouched)
+    h2 = rnd(T, n, seed=6)
+    keep = h2.clone()
+    rows = torch.tensor([T - 1, 0], dtype=torch.int32, device=DEV)
+    got = ops.rmsnorm(h2, delta, w, 1e-6, dtype, rows=rows)
+    want = ref.rmsnorm(keep.clone(), delta, w, 1e-6, dtype, rows=rows)
+    assert torch.equal(h2, keep)
+    close(got, want, dtype)
+    close(ops.rmsnorm(h2, None, w, 1e-6, dtype), ref.rmsnorm(keep.clone(), None, w, 1e-6, dtype), dtype)
+
+
+def test_rmsnorm_eps_matters():
+    x = torch.full((1, 64), 1e-3, device=DEV)
+    w = torch.ones(64, device=DEV)
+    a = ops.rmsnorm(x.clone(), None, w, 1e-6, torch.float32)
+    b = ops.rmsnorm(x.clone(), None, w, 1e-5, torch.float32)
+    assert abs(float(a[0, 0]) - 1e-3 / (2e-6) ** 0.5) < 1e-3
+    assert abs(float(b[0, 0]) - 1e-3 / (1.1e-5) ** 0.5) < 1e-3
+
+
+@pytest.mark.parametrize("dt_x,dt_w,dt_o", [
+    (torch.float32, torch.float32, torch.float32), (torch.float32, torch.bfloat16, torch.float32),
+    (torch.bfloat16, torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.bfloat16, torch.float32),
+    (torch.bfloat16, torch.float32, torch.bfloat16)])
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (3, 331, 72), (65, 130, 200), (64, 64, 16), (17, 1000, 257)])
+def test_gemm_generic(dt_x, dt_w, dt_o, M, N, K):
+    x = rnd(M, K, dtype=dt_x, seed=7)
+    w = rnd(N, K, dtype=dt_w, seed=8)
+    got = ops.gemm(x, w, dt_o)
+    want = ref.gemm(x, w, dt_o)
+    close(got, want, dt_o, scale=K ** 0.5)
+
+
+def make_rope_table(positions, rot, theta):
+    i = torch.arange(rot // 2, dtype=torch.float64)
+    inv = 1.0 / theta ** (2 * i / rot)
+    ang = torch.arange(positions, dtype=torch.float64)[:, None] * inv[None]
+    return torch.cat([ang.cos(), ang.sin()], 1).float().to(DEV)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 4), (6, 2, 48, 16), (5, 5, 32, 8), (8, 1, 128, 16),
+                                           (3, 1, 80, 2), (2, 2, 256, 32)])
+def test_qk_norm_rope_write(dtype, nh, nkv, d, page):
+    T, pages = 37, 40
+    qkv = rnd(T, (nh + 2 * nkv) * d, dtype=dtype, seed=9)
+    qw, kw = 1 + rnd(d, seed=10, scale=0.2), 1 + rnd(d, seed=11, scale=0.2)
+    positions = torch.randint(0, 500, (T,), generator=torch.Generator().manual_seed(12)).int().to(DEV)
+    table = make_rope_table(512, d, 10000.0)
+    slots = torch.randperm(pages * page, generator=torch.Generator().manual_seed(13))[:T].int()
+    slots[5] = -1
+    slots = slots.to(DEV)
+    kc = torch.zeros(pages, nkv, page, d, dtype=dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    qkv_ref, kc_ref, vc_ref = qkv.clone(), kc.clone(), vc.clone()
+    ref.qk_norm_rope_write(qkv_ref, nh, nkv, d, qw, kw, 1e-6, positions, table, kc_ref, vc_ref, slots, page)
+    ops.qk_norm_rope_write(qkv, nh, nkv, d, qw, kw, 1e-6, positions, table, kc, vc, slots, page)
+    close(qkv, qkv_ref, dtype)
+    close(kc, kc_ref, dtype)
+    assert torch.equal(vc, vc_ref)
+    # no norm, no rotation, no cache: nothing changes
+    again = qkv.clone()
+    ops.qk_norm_rope_write(again, nh, nkv, d, None, None, 0.0, None, None, None, None, None, page)
+    assert torch.equal(again, qkv)
+
+
+def paged_case(lengths, new, nh, nkv, d, page, dtype, seed, spare=3):
+    """Requests with ``lengths[r]`` cached tokens of which the last ``new[r]`` are this step's."""
+    rng = random.Random(seed)
+    R = len(lengths)
+    need = sum(-(-n // page) for n in lengths)
+    ids = list(range(need + spare))
+    rng.shuffle(ids)
+    kc = rnd(need + spare, nkv, page, d, dtype=dtype, seed=seed + 1)
+    vc = rnd(need + spare, nkv, page, d, dtype=dtype, seed=seed + 2)
+    mb = max(-(-n // page) for n in lengths)
+    table = torch.full((R, mb), -1, dtype=torch.int32)
+    for r, n in enumerate(lengths):
+        for j in range(-(-n // page)):
+            table[r, j] = ids.pop()
+    tok_req, positions, q_start = [], [], [0]
+    for r, (n, k) in enumerate(zip(lengths, new)):
+        tok_req += [r] * k
+        positions += list(range(n - k, n))
+        q_start.append(q_start[-1] + k)
+    T = len(tok_req)
+    qkv = rnd(T, (nh + 2 * nkv) * d, dtype=dtype, seed=seed + 3)
+    dec = [q_start[r] for r in range(R) if new[r] == 1]
+    tiles = []
+    for r in range(R):
+        if new[r] > 1:
+            for t0 in range(0, new[r], 64):
+                tiles += [r, q_start[r] + t0, min(64, new[r] - t0), lengths[r] - new[r] + t0]
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    batch = AttentionBatch(tok_req=i32(tok_req), positions=i32(positions), block_table=table.to(DEV),
+                           q_start=i32(q_start), ctx_len=i32(lengths), num_decode=len(dec),
+                           decode_tokens=i32(dec), prefill_tiles=i32(tiles).view(-1, 4),
+                           max_ctx=max(lengths), all_decode=len(dec) == R)
+    return qkv, batch, kc, vc
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,page,window", [
+    (4, 2, 16, 4, 0), (6, 2, 48, 16, 0), (8, 1, 32, 8, 0), (5, 5, 80, 16, 0), (32, 8, 128, 16, 0),
+    (6, 2, 48, 16, 24), (4, 4, 64, 8, 5), (2, 1, 256, 16, 0)])
+def test_attention_mixed_batch(dtype, nh, nkv, d, page, window):
+    lengths = [1, 300, 17, 64, 130]
+    new = [1, 1, 17, 2, 70]
+    qkv, batch, kc, vc = paged_case(lengths, new, nh, nkv, d, page, dtype, seed=20)
+    got = ops.attention(qkv, batch, kc, vc, nh, nkv, d, page, d ** -0.5, window)
+    want = ref.attention(qkv.cpu(), AttentionBatch(batch.tok_req.cpu(), batch.positions.cpu(),
+                                                   batch.block_table.cpu()),
+                         kc.cpu(), vc.cpu(), nh, nkv, d, page, d ** -0.5, window)
+    close(got, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_far_key_stands_out(dtype):
+    """One key among many hundreds gets a large score: the output must be its value row, so a
+    kernel that drops or misplaces far keys fails."""
+    nh, nkv, d, page = 4, 2, 32, 16
+    for far in (0, 15, 16, 511, 777):
+        qkv, batch, kc, vc = paged_case([900], [1], nh, nkv, d, page, dtype, seed=30)
+        table = batch.block_table[0].tolist()
+        q = torch.zeros(1, nh + 2 * nkv, d, dtype=dtype, device=DEV)
+        q[0, :nh, 3] = 40.0
+        kc[table[far // page], :, far % page, :] = 0
+        kc[table[far // page], :, far % page, 3] = 40.0
+        got = ops.attention(q.view(1, -1), batch, kc, vc, nh, nkv, d, page, d ** -0.5, 0).view(nh, d)
+        for h in range(nh):
+            close(got[h], vc[table[far // page], h // 2, far % page], dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,I", [(1, 8), (5, 200), (70, 1001)])
+def test_swiglu(dtype, T, I):
+    gu = rnd(T, 2 * I, dtype=dtype, seed=40, scale=3.0)
+    close(ops.swiglu(gu), ref.swiglu(gu), dtype)
+    z = torch.zeros(1, 2 * I, dtype=dtype, device=DEV)
+    assert float(ops.swiglu(z).abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("V", [7, 331, 151936])
+def test_sampling(V):
+    logits = rnd(6, V, seed=50, scale=2.0)
+    logits[1, V // 2] = logits[1, 0] = 50.0            # a tie: the lowest index wins
+    got = ops.sample(logits)
+    assert got.tolist() == logits.argmax(dim=1).tolist()
+    assert int(got[1]) == 0
+    temps = torch.tensor([0.7, 0.0, 1.3, 0.7, 2.0, 0.05], device=DEV)
+    us = torch.tensor([0.0, 0.3, 0.999999, 0.5, 0.25, 0.9], device=DEV)
+    got = ops.sample(logits, temps, us).tolist()
+    want = ref.sample(logits.cpu(), temps.cpu(), us.cpu()).tolist()
+    p = torch.softmax(logits.double().cpu() / temps.double().cpu().clamp(min=1e-9)[:, None], 1)
+    cdf = p.cumsum(1)
+    for r in range(6):
+        if got[r] != want[r]:   # only a float32-rounding neighbour of the boundary may differ
+            lo = cdf[r, min(got[r], want[r])]
+            assert abs(float(lo) - float(us[r])) < 1e-4, (r, got[r], want[r])
+    assert got[1] == 0
+
+
+def test_sampling_follows_the_distribution():
+    logits = torch.tensor([[0.0, 1.0, 2.0, -1.0, 0.5]], device=DEV).repeat(4000, 1).contiguous()
+    temps = torch.full((4000,), 0.7, device=DEV)
+    us = torch.rand(4000, generator=torch.Generator().manual_seed(1)).to(DEV)
+    got = ops.sample(logits, temps, us)
+    freq = torch.bincount(got.cpu().long(), minlength=5).double() / 4000
+    p = torch.softmax(logits[0].double().cpu() / 0.7, 0)
+    assert float((freq - p).abs().max()) < 0.03
