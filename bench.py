@@ -1,0 +1,164 @@
+"""Decode and prefill throughput of the engine on one MI355X, with roofline fractions.
+
+Default run: the layer sizes of the Qwen3-8B-shaped configuration (36 layers, hidden 4096, 32
+query heads, 8 kv heads, head size 128, intermediate 12288, vocabulary 151936), random
+weights, bfloat16, a batch of 8 requests at a context of 8,192 tokens.  One "step" is one
+decode step of the whole batch through the engine's own step function and sampler (greedy),
+the sampled tokens being fed to the next step.  The cache of the live requests is filled with
+random keys and values instead of running their 8,191-token prompts (a decode step's cost
+does not depend on what the cache holds); the prefill figure is a real 2,048-token prompt in
+one step.  Prints ONE JSON line.
+
+    python bench.py --gpus 1 --steps 20 --warmup 3
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+SIZES_8B = dict(num_hidden_layers=36, hidden_size=4096, num_attention_heads=32,
+                num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936,
+                rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
+                max_position_embeddings=40960, initializer_range=0.02)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=8192)
+    ap.add_argument("--layers", type=int, default=SIZES_8B["num_hidden_layers"])
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--points", default="1,64", help="further decode batch sizes (comma list, '' for none)")
+    ap.add_argument("--block-size", type=int, default=16)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    from lucciola_amd.config.engine_config import EngineConfig
+    from lucciola_amd.engine.batch import StepEntry
+    from lucciola_amd.engine.loading import random_model
+    from lucciola_amd.engine.runner import ModelRunner
+    from lucciola_amd.sampling.sampler import Sampler, SamplingParams
+
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    cfg = dict(SIZES_8B, architectures=["Qwen3ForCausalLM"], num_hidden_layers=args.layers)
+    points = [int(p) for p in args.points.split(",") if p]
+    max_batch = max([args.batch] + points)
+    steps_total = args.steps + args.warmup + 8
+    per_request = args.context + steps_total
+    bs = args.block_size
+    blocks = max_batch * (-(-per_request // bs)) + (-(-args.prefill_tokens // bs)) + 8
+
+    t0 = time.time()
+    model, mcfg = random_model(cfg, seed=0, dtype=dtype, device=dev)
+    runner = ModelRunner(model, EngineConfig(dtype=dtype, block_size=bs, max_blocks=blocks,
+                                             max_seqs=max_batch + 2, device=dev))
+    for k, v in runner.cache.kv.values():
+        k.normal_(0, 0.5)
+        v.normal_(0, 0.5)
+    sampler = Sampler()
+    torch.cuda.synchronize()
+    print(f"[bench] model and cache ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+
+    L, H, nh, nkv, d = args.layers, mcfg.hidden_size, mcfg.num_attention_heads, mcfg.num_key_value_heads, mcfg.head_dim
+    I, V = mcfg.intermediate_size, mcfg.vocab_size
+    esize = 2 if args.dtype == "bf16" else 4
+    layer_params = (nh + 2 * nkv) * d * H + nh * d * H + 3 * I * H
+    weight_bytes = (L * layer_params + V * H) * esize + (2 * L + 1) * H * 4 + 2 * L * d * 4
+    kv_bytes_per_token = 2 * L * nkv * d * esize
+
+    def decode_run(batch, steps, warmup):
+        """Time ``steps`` decode steps of ``batch`` requests at the context length."""
+        names = [f"d{batch}_{i}" for i in range(batch)]
+        cache = runner.cache
+        for n in names:
+            cache.admit(n)
+            cache.reserve(n, args.context - 1)
+            cache.commit(n)
+        gen = torch.Generator().manual_seed(batch)
+        tokens = torch.randint(0, V, (batch,), generator=gen).tolist()
+        params = [SamplingParams(max_new_tokens=1 << 30)] * batch
+
+        def one():
+            nonlocal tokens
+            logits = runner.step([StepEntry(n, [t], [0]) for n, t in zip(names, tokens)])
+            tokens = sampler.sample(logits, params, [0] * batch)
+        for _ in range(warmup):
+            one()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            one()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t) * 1e3 / steps
+        ctx_mid = args.context + warmup + steps / 2.0
+        for n in names:
+            runner.finish(n)
+        bytes_step = weight_bytes + batch * H * esize + batch * ctx_mid * kv_bytes_per_token
+        return ms, batch / (ms / 1e3), bytes_step
+
+    def prefill_run(tokens, reps=3):
+        gen = torch.Generator().manual_seed(7)
+        best = None
+        for r in range(reps + 1):
+            ids = torch.randint(0, V, (tokens,), generator=gen).tolist()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            logits = runner.step([StepEntry(f"p{r}", ids, [tokens - 1])])
+            sampler.sample(logits, [SamplingParams()], [0])
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t) * 1e3
+            runner.finish(f"p{r}")
+            if r > 0:
+                best = ms if best is None else min(best, ms)
+        flops = 2.0 * tokens * L * layer_params + 2.0 * tokens * tokens * nh * d * L + 2.0 * V * H
+        return best, flops
+
+    ms, tps, bytes_step = decode_run(args.batch, args.steps, args.warmup)
+    print(f"[bench] decode batch {args.batch}: {ms:.3f} ms/step", file=sys.stderr, flush=True)
+    achieved = bytes_step / (ms / 1e3) / 1e9
+    pms, pflops = prefill_run(args.prefill_tokens)
+    print(f"[bench] prefill {args.prefill_tokens}: {pms:.2f} ms", file=sys.stderr, flush=True)
+    point_values = {}
+    for b in points:
+        pm, ptps, _ = decode_run(b, max(3, min(args.steps, 10)), 2)
+        point_values[f"decode_b{b}"] = round(ptps, 2)
+        print(f"[bench] decode batch {b}: {pm:.3f} ms/step", file=sys.stderr, flush=True)
+
+    line = {
+        "metric": "decode tok/s (Qwen3-8B-shaped, batch 8, context 8192)",
+        "value": round(tps, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
+        "data": "synthetic: random weights, random token ids, cache of the live requests filled with random keys/values",
+        "config": {"model": "Qwen3-8B-shaped", "layers": L, "layers_full": SIZES_8B["num_hidden_layers"],
+                   "hidden": H, "heads": nh, "kv_heads": nkv, "head_dim": d, "intermediate": I,
+                   "vocab": V, "global_batch": args.batch, "seq_len": args.context,
+                   "page_size": bs, "prefill_tokens": args.prefill_tokens, "parallelism": "single GPU"},
+        "prefill": {"value": round(args.prefill_tokens / (pms / 1e3), 1), "tokens": args.prefill_tokens,
+                    "ms": round(pms, 3), "frac": round(pflops / (pms / 1e3) / MFMA_PEAK[args.dtype], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "points": point_values,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -26,7 +26,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 # error of a row of logits: max |difference| / max |logit|
-TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+TOL = {"float32": 2e-5, "bfloat16": 3e-2}
 LENGTHS = {"A": [5, 11, 17, 40, 130], "B": [1, 9, 30, 64, 45, 200], "C": [70, 33, 50, 3, 61, 150]}
 
 _cache = {}
@@ -157,7 +157,6 @@ def test_temperature_sampling_through_the_engine():
 def test_trace_run_program(tmp_path, dtype):
     cfg, page, seed = configs.ALL["C"]
     folder = write_model_folder(str(tmp_path / "model"), cfg, seed)
-    model, _ = load_model(folder, "float32", "cpu") if False else (None, None)
     from lucciola_amd.weights.safetensors_io import SafetensorsFile
     with SafetensorsFile(os.path.join(folder, "model.safetensors")) as f:
         weights = {n: f.get(n).clone() for n in f.names()}
