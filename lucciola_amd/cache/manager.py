@@ -88,13 +88,15 @@ class CacheManager:
         return total
 
     def allocate_tensors(self, dtype: torch.dtype, device) -> None:
-        """Keys and values per paged site: [num_blocks, kv_heads, block_size, head_dim];
+        """Per paged site: keys [num_blocks, kv_heads, block_size, head_dim] and values
+        [num_blocks, kv_heads, head_dim, block_size] (transposed inside a page);
         state per state site: [max_seqs, *shape]."""
         for g in self.groups:
-            shape = (self.num_blocks, g.spec.num_kv_heads, self.block_size, g.spec.head_dim)
+            k_shape = (self.num_blocks, g.spec.num_kv_heads, self.block_size, g.spec.head_dim)
+            v_shape = (self.num_blocks, g.spec.num_kv_heads, g.spec.head_dim, self.block_size)
             for site in g.sites:
-                self.kv[site] = (torch.zeros(shape, dtype=dtype, device=device),
-                                 torch.zeros(shape, dtype=dtype, device=device))
+                self.kv[site] = (torch.zeros(k_shape, dtype=dtype, device=device),
+                                 torch.zeros(v_shape, dtype=dtype, device=device))
         for site in self.state_sites:
             spec = self.site_specs[site]
             self.state[site] = torch.zeros((self.max_seqs,) + tuple(spec.shape), dtype=spec.dtype,

@@ -9,8 +9,9 @@
 // src/kernels/attention_paged.cu:80-81) the key loop streams chunks of 256 keys with a running
 // maximum and sum, so any context length works.
 //
-// Cache layout: [pages, nkv, page_size, d].  A key at position j of request r lives in page
-// block_table[r][j / page_size], slot j % page_size.
+// Cache layouts: keys [pages, nkv, page_size, d], values [pages, nkv, d, page_size].  The key
+// and value at position j of request r live in page block_table[r][j / page_size], slot
+// j % page_size.
 #include "common.h"
 
 namespace lc {
@@ -50,8 +51,9 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
         long long off = 0;
         if (valid) {
             const int page = table[j / page_size];
-            off = (((long long)page * nkv + kvh) * page_size + (j % page_size)) * d;
-            const T* krow = k_cache + off;
+            const long long head = (long long)page * nkv + kvh;
+            off = head * d * page_size + (j % page_size);          // of the value column
+            const T* krow = k_cache + (head * page_size + (j % page_size)) * d;
             float dot = 0.f;
             for (int i = 0; i < d; ++i) dot = fmaf(qs[i], to_f32(krow[i]), dot);
             s = dot;
@@ -69,7 +71,7 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
         if (pv_active) {
             const int count = min(AG_THREADS, p - c0 + 1);
             for (int jj = g; jj < count; jj += groups)
-                acc = fmaf(ps[jj], to_f32(v_cache[voff[jj] + di]), acc);
+                acc = fmaf(ps[jj], to_f32(v_cache[voff[jj] + (long long)di * page_size]), acc);
         }
         __syncthreads();  // ps/voff are rewritten by the next chunk
     }

@@ -92,7 +92,9 @@ __global__ void rmsnorm_act_kernel(const T* __restrict__ x, const float* __restr
 //   q, k: optional RMSNorm over d, then rotation of the first `rot` dims with the angles of
 //   the token's position (cos in table[pos][0:rot/2], sin in table[pos][rot/2:rot]).
 //   q and k are written back in place; k and v also go to the cache page slot of the token.
-// Cache layout: [pages, nkv, page_size, d]; slot = page * page_size + offset; slot < 0 skips.
+// Cache layouts: keys [pages, nkv, page_size, d], values transposed [pages, nkv, d, page_size]
+// (a value's positions lie next to each other, which is how the matrix cores want the P.V
+// operand); slot = page * page_size + offset; slot < 0 skips.
 template <typename T>
 __global__ void qk_norm_rope_write_kernel(T* __restrict__ qkv, int T_tokens, int nh, int nkv, int d,
                                           const float* __restrict__ q_w,
@@ -114,19 +116,21 @@ __global__ void qk_norm_rope_write_kernel(T* __restrict__ qkv, int T_tokens, int
     const bool is_k = !is_q && head < nh + nkv;
     const int kvh = is_q ? 0 : (is_k ? head - nh : head - nh - nkv);
 
-    T* cache_row = nullptr;
+    T* cache_row = nullptr;   // k: the slot's row of d entries;  v: the slot's column (stride page_size)
     if (!is_q && slots && k_cache) {
         const int slot = slots[t];
         if (slot >= 0) {
             const int page = slot / page_size, off = slot - page * page_size;
-            T* base = is_k ? k_cache : v_cache;
-            cache_row = base + (((size_t)page * nkv + kvh) * page_size + off) * d;
+            if (is_k)
+                cache_row = k_cache + (((size_t)page * nkv + kvh) * page_size + off) * d;
+            else
+                cache_row = v_cache + ((size_t)page * nkv + kvh) * d * page_size + off;
         }
     }
 
-    if (!is_q && !is_k) {  // v: copy only
+    if (!is_q && !is_k) {  // v: copy only, transposed into the page
         if (cache_row)
-            for (int i = lane; i < d; i += kWave) cache_row[i] = x[i];
+            for (int i = lane; i < d; i += kWave) cache_row[(size_t)i * page_size] = x[i];
         return;
     }
 

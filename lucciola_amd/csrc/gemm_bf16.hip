@@ -1,0 +1,230 @@
+// bfloat16 matrix products on the matrix cores: out[M, N] = x[M, K] . w[N, K]^T, float32
+// accumulation, output bfloat16 or float32.  Two kernels:
+//
+//  * skinny (M <= 64, decode): bound by reading w once from HBM.  A workgroup owns 16 rows of
+//    w; its waves split K in interleaved blocks of 128, each wave streaming its part of the
+//    rows straight from global memory into v_mfma_f32_16x16x32_bf16 operands (w is the A
+//    operand, x^T the B operand); the waves' partial sums meet in LDS.  No split-K workspace,
+//    no atomics: the order of the sums is fixed.
+//  * tiled (M > 64, prefill): 128x128x64 workgroup tiles in LDS (rows padded to 144 bytes so
+//    that operand reads are conflict free), 4 waves of 64x64 built from
+//    v_mfma_f32_32x32x16_bf16, next tile prefetched into registers while the current one is
+//    multiplied.  Workgroups are renumbered so that each XCD's L2 sees neighbouring tiles.
+//
+// The reference's linear kernel computes the same product with one thread per output element
+// and no matrix instruction (src/kernels/linear.cu:7-56).
+#include "common.h"
+
+namespace lc {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+template <typename TO> __device__ __forceinline__ void store_out(TO* p, float v);
+template <> __device__ __forceinline__ void store_out<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void store_out<bf16>(bf16* p, float v) { *p = static_cast<bf16>(v); }
+
+// ------------------------------------------------------------------------------- skinny
+constexpr int SK_ROWS = 16;    // rows of w per workgroup
+constexpr int SK_KBLOCK = 128; // k elements per wave iteration
+
+template <int MT, int WAVES, typename TO>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __restrict__ x,
+                                                                 const bf16* __restrict__ w,
+                                                                 TO* __restrict__ out, int M, int N,
+                                                                 int K) {
+    __shared__ float red[WAVES * MT * 256];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * SK_ROWS;
+    const int row = min(n0 + r, N - 1);
+    const bf16* wp = w + (size_t)row * K + g * 8;
+    const bf16* xp[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) xp[mt] = x + (size_t)min(mt * 16 + r, M - 1) * K + g * 8;
+
+    floatx4 acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const int kblocks = K / SK_KBLOCK;
+#pragma unroll 2
+    for (int kb = wave; kb < kblocks; kb += WAVES) {
+        const int k0 = kb * SK_KBLOCK;
+        bf16x8 a[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) a[j] = *reinterpret_cast<const bf16x8*>(wp + k0 + j * 32);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            bf16x8 b[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = *reinterpret_cast<const bf16x8*>(xp[mt] + k0 + j * 32);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[j], acc[mt], 0, 0, 0);
+        }
+    }
+    // acc[mt][v] = partial out[m = mt*16 + lane%16][n = n0 + (lane/16)*4 + v]
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[(wave * MT + mt) * 256 + v * 64 + lane] = acc[mt][v];
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < MT * 256; idx += WAVES * 64) {
+        float total = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < WAVES; ++wv) total += red[wv * MT * 256 + idx];
+        const int mt = idx >> 8, v = (idx >> 6) & 3, l = idx & 63;
+        const int m = mt * 16 + (l & 15), n = n0 + (l >> 4) * 4 + v;
+        if (m < M && n < N) store_out<TO>(out + (size_t)m * N + n, total);
+    }
+}
+
+// ------------------------------------------------------------------------------- tiled
+constexpr int TB_M = 128, TB_N = 128, TB_K = 64;
+constexpr int TB_LD = TB_K + 8;   // padded row length in LDS (144 bytes)
+
+template <typename TO>
+__global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ x,
+                                                         const bf16* __restrict__ w,
+                                                         TO* __restrict__ out, int M, int N, int K,
+                                                         int tiles_m, int tiles_n) {
+    __shared__ __attribute__((aligned(16))) bf16 As[TB_M * TB_LD];
+    __shared__ __attribute__((aligned(16))) bf16 Bs[TB_N * TB_LD];
+
+    // renumber: workgroups go round-robin over 8 XCDs; give each XCD a contiguous run of
+    // tiles, m fastest, so that one XCD's L2 keeps the w tile that its workgroups share
+    const int total = tiles_m * tiles_n;
+    int id = blockIdx.x;
+    {
+        const int q = total >> 3, rem = total & 7;
+        const int xcd = id & 7, local = id >> 3;
+        id = xcd * q + min(xcd, rem) + local;   // a bijection of [0, total) for any total
+    }
+    const int tm = id % tiles_m, tn = id / tiles_m;
+    const int m0 = tm * TB_M, n0 = tn * TB_N;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    const int lr = lane & 31, lk = (lane >> 5) * 8;
+
+    // global -> register staging: 4 chunks of 16 bytes per thread and operand
+    const bf16* xg[4];
+    const bf16* wg[4];
+    int soff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = tid + i * 256;
+        const int row = c >> 3, col = (c & 7) * 8;
+        xg[i] = x + (size_t)min(m0 + row, M - 1) * K + col;
+        wg[i] = w + (size_t)min(n0 + row, N - 1) * K + col;
+        soff[i] = row * TB_LD + col;
+    }
+    bf16x8 ra[4], rb[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        ra[i] = *reinterpret_cast<const bf16x8*>(xg[i]);
+        rb[i] = *reinterpret_cast<const bf16x8*>(wg[i]);
+    }
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    for (int k0 = 0; k0 < K; k0 += TB_K) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<bf16x8*>(As + soff[i]) = ra[i];
+            *reinterpret_cast<bf16x8*>(Bs + soff[i]) = rb[i];
+        }
+        __syncthreads();
+        if (k0 + TB_K < K) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                ra[i] = *reinterpret_cast<const bf16x8*>(xg[i] + k0 + TB_K);
+                rb[i] = *reinterpret_cast<const bf16x8*>(wg[i] + k0 + TB_K);
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < TB_K; ks += 16) {
+            bf16x8 a[2], b[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                a[i] = *reinterpret_cast<const bf16x8*>(As + (wm + i * 32 + lr) * TB_LD + ks + lk);
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                b[j] = *reinterpret_cast<const bf16x8*>(Bs + (wn + j * 32 + lr) * TB_LD + ks + lk);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+    // acc[i][j][v]: row m = (v/4)*8 + (lane/32)*4 + v%4, column n = lane%32 of the 32x32 tile
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int n = n0 + wn + j * 32 + lr;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + wm + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                if (m < M && n < N) store_out<TO>(out + (size_t)m * N + n, acc[i][j][v]);
+            }
+        }
+}
+
+template <int MT, typename TO>
+static void launch_skinny(const bf16* x, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
+    constexpr int WAVES = 8;
+    gemm_skinny_kernel<MT, WAVES, TO><<<(N + SK_ROWS - 1) / SK_ROWS, WAVES * 64, 0, s>>>(x, w, out, M, N, K);
+}
+
+template <typename TO>
+static int launch_bf16(const bf16* x, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
+    if (M <= 64) {
+        switch ((M + 15) / 16) {
+            case 1: launch_skinny<1, TO>(x, w, out, M, N, K, s); break;
+            case 2: launch_skinny<2, TO>(x, w, out, M, N, K, s); break;
+            case 3: launch_skinny<3, TO>(x, w, out, M, N, K, s); break;
+            default: launch_skinny<4, TO>(x, w, out, M, N, K, s); break;
+        }
+        LC_LAUNCH_CHECK("gemm_skinny");
+    } else {
+        const int tiles_m = (M + TB_M - 1) / TB_M, tiles_n = (N + TB_N - 1) / TB_N;
+        gemm_tiled_kernel<TO><<<tiles_m * tiles_n, 256, 0, s>>>(x, w, out, M, N, K, tiles_m, tiles_n);
+        LC_LAUNCH_CHECK("gemm_tiled");
+    }
+    return 0;
+}
+
+}  // namespace lc
+
+using namespace lc;
+
+// Sizes the matrix-core kernels take; everything else goes to the generic kernel.
+LC_API int lc_gemm_bf16_supported(int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    if (K % SK_KBLOCK != 0) return 0;
+    if ((size_t)((M + TB_M - 1) / TB_M) * ((N + TB_N - 1) / TB_N) > 0x7fffffffu) return 0;
+    return 1;
+}
+
+LC_API int lc_gemm_bf16(const void* x, const void* w, void* out, int out_dt, int M, int N, int K,
+                        hipStream_t stream) {
+    LC_CHECK(lc_gemm_bf16_supported(M, N, K), "gemm_bf16: sizes M=%d N=%d K=%d are not supported "
+             "(K must be a multiple of %d)", M, N, K, SK_KBLOCK);
+    LC_CHECK(x && w && out, "gemm_bf16: null pointer");
+    LC_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_bf16: operands must be 16-byte aligned");
+    if (out_dt == DT_BF16) return launch_bf16<bf16>((const bf16*)x, (const bf16*)w, (bf16*)out, M, N, K, stream);
+    if (out_dt == DT_F32) return launch_bf16<float>((const bf16*)x, (const bf16*)w, (float*)out, M, N, K, stream);
+    LC_CHECK(false, "gemm_bf16: unknown output dtype %d", out_dt);
+    return 0;
+}

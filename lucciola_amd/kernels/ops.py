@@ -26,8 +26,14 @@ _SIGNATURES = {
     "lc_rmsnorm": "ppppfpiiiip",
     "lc_rmsnorm_act": "ppfpiiip",
     "lc_gemm_generic": "pipipiiiip",
+    "lc_gemm_bf16": "pppiiiip",
+    "lc_gemm_bf16_supported": "iii",
     "lc_qk_norm_rope_write": "piiiiippfppipppip",
     "lc_attention_generic": "pipppipppiiiiiifip",
+    "lc_attn_bf16_supported": "iiii",
+    "lc_attn_decode_splits": "iii",
+    "lc_attn_decode_bf16": "pippppppppp" + "iiiiii" + "f" + "ii" + "p",
+    "lc_attn_prefill_bf16": "pippppp" + "iiiiii" + "f" + "i" + "p",
     "lc_swiglu": "ppiiip",
     "lc_sample": "ppppiip",
 }
@@ -178,9 +184,7 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = No
 
 
 def _fast_gemm_ok(M: int, N: int, K: int) -> bool:
-    lib = library()
-    fn = getattr(lib, "lc_gemm_bf16_supported", None)
-    return bool(fn and fn(_c_int(M), _c_int(N), _c_int(K)))
+    return bool(library().lc_gemm_bf16_supported(M, N, K))
 
 
 # ------------------------------------------------------------------------------ attention
@@ -193,7 +197,8 @@ def qk_norm_rope_write(qkv: torch.Tensor, nh: int, nkv: int, d: int,
     """In place on ``qkv`` [T, (nh + 2 nkv) d]: per-head RMSNorm of q and k (if weights are
     given), rotation by ``rope_table`` [positions, rot] (cos | sin halves) at each token's
     position, and the write of k and v into their cache slot ``slots`` [T]
-    (page * page_size + offset; negative: no write).  Caches are [pages, nkv, page_size, d]."""
+    (page * page_size + offset; negative: no write).  Key cache [pages, nkv, page_size, d],
+    value cache [pages, nkv, d, page_size]."""
     _need(qkv, "qkv", None, 2)
     T = qkv.shape[0]
     if qkv.shape[1] != (nh + 2 * nkv) * d:
@@ -214,9 +219,7 @@ def qk_norm_rope_write(qkv: torch.Tensor, nh: int, nkv: int, d: int,
         _need(k_cache, "k cache", qkv.dtype, 4)
         _need(v_cache, "v cache", qkv.dtype, 4)
         _need(slots, "slots", torch.int32, 1)
-        if tuple(k_cache.shape[1:]) != (nkv, page_size, d) or k_cache.shape != v_cache.shape:
-            raise KernelError(f"cache shape {tuple(k_cache.shape)} does not fit "
-                              f"[pages, {nkv}, {page_size}, {d}]")
+        _check_caches(k_cache, v_cache, nkv, page_size, d)
         if slots.shape[0] != T:
             raise KernelError("slots do not match the tokens")
     else:
@@ -225,6 +228,16 @@ def qk_norm_rope_write(qkv: torch.Tensor, nh: int, nkv: int, d: int,
           _c_int(d), _ptr(q_weight), _ptr(k_weight), _c_float(eps), _ptr(positions),
           _ptr(rope_table), _c_int(rot), _ptr(k_cache), _ptr(v_cache), _ptr(slots),
           _c_int(page_size), _stream())
+
+
+def _check_caches(k_cache, v_cache, nkv, page_size, d) -> None:
+    if tuple(k_cache.shape[1:]) != (nkv, page_size, d):
+        raise KernelError(f"key cache shape {tuple(k_cache.shape)} does not fit "
+                          f"[pages, {nkv}, {page_size}, {d}]")
+    if tuple(v_cache.shape) != (k_cache.shape[0], nkv, d, page_size):
+        raise KernelError(f"value cache shape {tuple(v_cache.shape)} does not fit "
+                          f"[{k_cache.shape[0]}, {nkv}, {d}, {page_size}] (values are transposed "
+                          f"inside a page)")
 
 
 @dataclass
@@ -266,9 +279,29 @@ def attention(qkv: torch.Tensor, batch: AttentionBatch, k_cache: torch.Tensor,
     _need(batch.tok_req, "tok_req", torch.int32, 1)
     _need(batch.positions, "positions", torch.int32, 1)
     _need(batch.block_table, "block table", torch.int32, 2)
-    if tuple(k_cache.shape[1:]) != (nkv, page_size, d):
-        raise KernelError(f"cache shape {tuple(k_cache.shape)} does not fit "
-                          f"[pages, {nkv}, {page_size}, {d}]")
+    _check_caches(k_cache, v_cache, nkv, page_size, d)
+    lib = library()
+    if qkv.dtype == torch.bfloat16 and batch.decode_tokens is not None \
+            and batch.prefill_tiles is not None \
+            and lib.lc_attn_bf16_supported(nh, nkv, d, page_size):
+        mb = batch.block_table.shape[1]
+        nd = batch.num_decode
+        if nd > 0:
+            splits = lib.lc_attn_decode_splits(nd, nkv, batch.max_ctx)
+            part_o = part_ml = None
+            if splits > 1:
+                part_o = torch.empty((nd * nh * splits * d,), dtype=torch.float32, device=qkv.device)
+                part_ml = torch.empty((nd * nh * splits * 2,), dtype=torch.float32, device=qkv.device)
+            _call("lc_attn_decode_bf16", _ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
+                  _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(batch.decode_tokens),
+                  _ptr(batch.tok_req), _ptr(batch.positions), _ptr(batch.block_table), mb, nd, nh,
+                  nkv, d, page_size, scale, window, splits, _stream())
+        nt = batch.prefill_tiles.shape[0]
+        if nt > 0:
+            _call("lc_attn_prefill_bf16", _ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
+                  _ptr(out), _ptr(batch.prefill_tiles), _ptr(batch.block_table), mb, nt, nh, nkv, d,
+                  page_size, scale, window, _stream())
+        return out
     _call("lc_attention_generic", _ptr(qkv), _c_int(qkv.shape[1]), _ptr(k_cache), _ptr(v_cache),
           _ptr(out), _c_int(_dt(qkv)), _ptr(batch.tok_req), _ptr(batch.positions),
           _ptr(batch.block_table), _c_int(batch.block_table.shape[1]), _c_int(T), _c_int(nh),

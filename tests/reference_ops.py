@@ -64,7 +64,7 @@ def qk_norm_rope_write(qkv, nh, nkv, d, q_weight, k_weight, eps, positions, rope
                 continue
             page, off = divmod(s, page_size)
             k_cache[page, :, off, :] = x[t, nh:nh + nkv]
-            v_cache[page, :, off, :] = v[t]
+            v_cache[page, :, :, off] = v[t]
 
 
 def attention(qkv, batch, k_cache, v_cache, nh, nkv, d, page_size, scale, window=0):
@@ -84,7 +84,7 @@ def attention(qkv, batch, k_cache, v_cache, nh, nkv, d, page_size, scale, window
         assert (pages >= 0).all(), "attention reads a page that was given back"
         offs = torch.tensor([j % page_size for j in js], dtype=torch.long)
         keys = k_cache[pages, :, offs, :].to(F64)      # [n, nkv, d]
-        vals = v_cache[pages, :, offs, :].to(F64)
+        vals = v_cache[pages, :, :, offs].to(F64)
         for h in range(nh):
             s = (keys[:, h // group, :] @ q[t, h]) * scale
             w = torch.softmax(s, dim=0)

@@ -19,10 +19,17 @@ def tol(dtype):
     return dict(rtol=2e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1e-3)
 
 
-def close(got, want, dtype, scale=1.0):
+def close(got, want, dtype, scale=1.0, atol=None):
     t = tol(dtype)
     torch.testing.assert_close(got.double().cpu(), want.double().cpu(), rtol=t["rtol"],
-                               atol=t["atol"] * scale)
+                               atol=t["atol"] * scale if atol is None else atol)
+
+
+def attention_atol(dtype, v_cache):
+    """The matrix-core kernels round the softmax weights to bfloat16 before the P.V product:
+    each weight is off by at most 2^-9 of itself, so an output (a convex combination of value
+    rows) is off by at most 2^-9 max|v|, beside its own rounding."""
+    return None if dtype == torch.float32 else float(v_cache.abs().max()) * 2.0 ** -9
 
 
 def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
@@ -104,7 +111,7 @@ def test_qk_norm_rope_write(dtype, nh, nkv, d, page):
     slots[5] = -1
     slots = slots.to(DEV)
     kc = torch.zeros(pages, nkv, page, d, dtype=dtype, device=DEV)
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(pages, nkv, d, page, dtype=dtype, device=DEV)
     qkv_ref, kc_ref, vc_ref = qkv.clone(), kc.clone(), vc.clone()
     ref.qk_norm_rope_write(qkv_ref, nh, nkv, d, qw, kw, 1e-6, positions, table, kc_ref, vc_ref, slots, page)
     ops.qk_norm_rope_write(qkv, nh, nkv, d, qw, kw, 1e-6, positions, table, kc, vc, slots, page)
@@ -125,7 +132,7 @@ def paged_case(lengths, new, nh, nkv, d, page, dtype, seed, spare=3):
     ids = list(range(need + spare))
     rng.shuffle(ids)
     kc = rnd(need + spare, nkv, page, d, dtype=dtype, seed=seed + 1)
-    vc = rnd(need + spare, nkv, page, d, dtype=dtype, seed=seed + 2)
+    vc = rnd(need + spare, nkv, d, page, dtype=dtype, seed=seed + 2)
     mb = max(-(-n // page) for n in lengths)
     table = torch.full((R, mb), -1, dtype=torch.int32)
     for r, n in enumerate(lengths):
@@ -155,7 +162,8 @@ def paged_case(lengths, new, nh, nkv, d, page, dtype, seed, spare=3):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,d,page,window", [
     (4, 2, 16, 4, 0), (6, 2, 48, 16, 0), (8, 1, 32, 8, 0), (5, 5, 80, 16, 0), (32, 8, 128, 16, 0),
-    (6, 2, 48, 16, 24), (4, 4, 64, 8, 5), (2, 1, 256, 16, 0)])
+    (6, 2, 48, 16, 24), (4, 4, 64, 8, 5), (2, 1, 256, 16, 0), (4, 2, 64, 16, 0), (6, 2, 96, 16, 24),
+    (16, 1, 32, 16, 0), (32, 8, 128, 16, 40), (12, 4, 128, 16, 7)])
 def test_attention_mixed_batch(dtype, nh, nkv, d, page, window):
     lengths = [1, 300, 17, 64, 130]
     new = [1, 1, 17, 2, 70]
@@ -164,7 +172,7 @@ def test_attention_mixed_batch(dtype, nh, nkv, d, page, window):
     want = ref.attention(qkv.cpu(), AttentionBatch(batch.tok_req.cpu(), batch.positions.cpu(),
                                                    batch.block_table.cpu()),
                          kc.cpu(), vc.cpu(), nh, nkv, d, page, d ** -0.5, window)
-    close(got, want, dtype)
+    close(got, want, dtype, atol=attention_atol(dtype, vc))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -181,7 +189,7 @@ def test_attention_far_key_stands_out(dtype):
         kc[table[far // page], :, far % page, 3] = 40.0
         got = ops.attention(q.view(1, -1), batch, kc, vc, nh, nkv, d, page, d ** -0.5, 0).view(nh, d)
         for h in range(nh):
-            close(got[h], vc[table[far // page], h // 2, far % page], dtype)
+            close(got[h], vc[table[far // page], h // 2, :, far % page], dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -221,3 +229,50 @@ def test_sampling_follows_the_distribution():
     freq = torch.bincount(got.cpu().long(), minlength=5).double() / 4000
     p = torch.softmax(logits[0].double().cpu() / 0.7, 0)
     assert float((freq - p).abs().max()) < 0.03
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M,N,K", [(1, 16, 128), (8, 100, 256), (17, 4096, 1024), (64, 331, 384),
+                                   (65, 128, 128), (128, 257, 512), (300, 1000, 640), (2048, 512, 1024),
+                                   (3, 151936 // 8, 256)])
+def test_gemm_bf16_matrix_cores(out_dtype, M, N, K):
+    x = rnd(M, K, dtype=torch.bfloat16, seed=60)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=61)
+    assert ops._fast_gemm_ok(M, N, K)
+    got = ops.gemm(x, w, out_dtype)
+    want = ref.gemm(x, w, out_dtype)
+    close(got, want, out_dtype, scale=K ** 0.5)
+
+
+def test_gemm_bf16_one_hot_rows_and_columns():
+    """x picks single columns of w: the product must return exactly those entries, so a wrong
+    operand layout (rows, k order) shows as a wrong element, not as a small error."""
+    M, N, K = 40, 48, 256
+    w = rnd(N, K, dtype=torch.bfloat16, seed=62)
+    x = torch.zeros(M, K, dtype=torch.bfloat16, device=DEV)
+    cols = [(7 * m + 3) % K for m in range(M)]
+    for m, c in enumerate(cols):
+        x[m, c] = 1.0
+    got = ops.gemm(x, w, torch.float32)
+    want = w.float()[:, cols].T.contiguous()
+    assert torch.equal(got, want)
+    xb = torch.zeros(200, K, dtype=torch.bfloat16, device=DEV)
+    cols = [(11 * m + 5) % K for m in range(200)]
+    for m, c in enumerate(cols):
+        xb[m, c] = 1.0
+    assert torch.equal(ops.gemm(xb, w, torch.float32), w.float()[:, cols].T.contiguous())
+
+
+@pytest.mark.parametrize("nh,nkv,d,window", [(32, 8, 128, 0), (8, 2, 64, 0), (4, 4, 96, 1000), (16, 1, 32, 0)])
+def test_attention_bf16_long_contexts(nh, nkv, d, window):
+    """Decode over thousands of keys (the pages are shared out over several workgroups and
+    joined) beside a long prompt portion with history."""
+    lengths = [5000, 1, 17, 2049, 700]
+    new = [1, 1, 1, 1, 300]
+    qkv, batch, kc, vc = paged_case(lengths, new, nh, nkv, d, 16, torch.bfloat16, seed=70)
+    assert ops.library().lc_attn_bf16_supported(nh, nkv, d, 16)
+    got = ops.attention(qkv, batch, kc, vc, nh, nkv, d, 16, d ** -0.5, window)
+    want = ref.attention(qkv.cpu(), AttentionBatch(batch.tok_req.cpu(), batch.positions.cpu(),
+                                                   batch.block_table.cpu()),
+                         kc.cpu(), vc.cpu(), nh, nkv, d, 16, d ** -0.5, window)
+    close(got, want, torch.bfloat16, atol=attention_atol(torch.bfloat16, vc))
