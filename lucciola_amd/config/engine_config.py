@@ -38,6 +38,9 @@ class EngineConfig:
     max_tokens_per_step: int = 576
     max_seqs: int = 256             # live requests (also the number of state slots)
     device: str = "cuda:0"
+    use_graphs: bool = True         # replay decode steps from HIP graphs (bfloat16 on the GPU)
+    graph_max_batch: int = 256      # largest decode batch that is captured
+    graph_cache_size: int = 16      # captured steps kept
 
     def __post_init__(self) -> None:
         self.dtype = parse_dtype(self.dtype)

@@ -204,25 +204,34 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 }
 
 // Joins the shares of a request's pages: out = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).
+// The factors are worked out once (one thread per share) and left in LDS, so that the sum over
+// the shares is a run of independent loads.
 template <int D>
-__global__ void attn_decode_join_kernel(const float* __restrict__ part_o,
-                                        const float* __restrict__ part_ml,
-                                        const int* __restrict__ decode_tokens,
-                                        bf16* __restrict__ out, int nh, int splits) {
-    const int di = blockIdx.x, h = blockIdx.y;
+__global__ __launch_bounds__(128) void attn_decode_join_kernel(const float* __restrict__ part_o,
+                                                               const float* __restrict__ part_ml,
+                                                               const int* __restrict__ decode_tokens,
+                                                               bf16* __restrict__ out, int nh,
+                                                               int splits) {
+    __shared__ float f[64];
+    __shared__ float inv_l;
+    const int di = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int t = decode_tokens[di];
     const size_t base = ((size_t)di * nh + h) * splits;
-    float m = -INFINITY;
-    for (int s = 0; s < splits; ++s) m = fmaxf(m, part_ml[(base + s) * 2]);
-    for (int dim = threadIdx.x; dim < D; dim += blockDim.x) {
-        float o = 0.f, l = 0.f;
-        for (int s = 0; s < splits; ++s) {
-            const float ms = part_ml[(base + s) * 2];
-            const float f = (ms == -INFINITY) ? 0.f : exp2f(ms - m);
-            o += f * part_o[(base + s) * D + dim];
-            l += f * part_ml[(base + s) * 2 + 1];
-        }
-        out[((size_t)t * nh + h) * D + dim] = static_cast<bf16>(o / l);
+    if (tid < 64) {
+        const float ms = tid < splits ? part_ml[(base + tid) * 2] : -INFINITY;
+        const float ls = tid < splits ? part_ml[(base + tid) * 2 + 1] : 0.f;
+        const float m = wave_max(ms);
+        const float fs = (ms == -INFINITY) ? 0.f : exp2f(ms - m);
+        f[tid] = fs;
+        const float l = wave_sum(fs * ls);
+        if (tid == 0) inv_l = 1.f / l;
+    }
+    __syncthreads();
+    for (int dim = tid; dim < D; dim += 128) {
+        float o = 0.f;
+#pragma unroll 8
+        for (int s = 0; s < splits; ++s) o += f[s] * part_o[(base + s) * D + dim];
+        out[((size_t)t * nh + h) * D + dim] = static_cast<bf16>(o * inv_l);
     }
 }
 
@@ -286,7 +295,7 @@ static int launch_decode(const bf16* qkv, int q_stride, const bf16* k, const bf1
                                                nh, nkv, scale_log2, window, splits);
     LC_LAUNCH_CHECK("attn_decode");
     if (splits > 1) {
-        attn_decode_join_kernel<D><<<dim3(ND, nh), D >= 128 ? 128 : 64, 0, s>>>(
+        attn_decode_join_kernel<D><<<dim3(ND, nh), 128, 0, s>>>(
             part_o, part_ml, decode_tokens, out, nh, splits);
         LC_LAUNCH_CHECK("attn_decode_join");
     }

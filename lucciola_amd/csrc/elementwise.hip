@@ -69,6 +69,76 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delt
     }
 }
 
+// The same for rows of up to 8192 entries whose length is a multiple of 8: every thread keeps
+// its entries in registers between the sum of squares and the scaling, and all of a thread's
+// loads are issued before the first is used (the plain kernel above walks a row with one
+// dependent load after the other).
+template <typename T> struct Pack8;
+template <> struct Pack8<float> {
+    float4 a, b;
+    __device__ __forceinline__ float get(int i) const { return i < 4 ? (&a.x)[i] : (&b.x)[i - 4]; }
+    __device__ __forceinline__ void set(int i, float v) { if (i < 4) (&a.x)[i] = v; else (&b.x)[i - 4] = v; }
+};
+template <> struct Pack8<bf16> {
+    typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+    bf16x8 v;
+    __device__ __forceinline__ float get(int i) const { return static_cast<float>(v[i]); }
+    __device__ __forceinline__ void set(int i, float f) { v[i] = static_cast<bf16>(f); }
+};
+
+constexpr int RN_THREADS = 256, RN_CHUNKS = 4;   // 256 threads x 4 chunks x 8 entries = 8192
+
+template <typename T>
+__global__ __launch_bounds__(RN_THREADS) void rmsnorm_vec_kernel(
+    float* __restrict__ h, const T* __restrict__ delta, const int* __restrict__ rows,
+    const float* __restrict__ w, float eps, T* __restrict__ out, int n, int write_h) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int src = rows ? rows[r] : r;
+    float* hr = h + (size_t)src * n;
+    const T* dr = delta ? delta + (size_t)src * n : nullptr;
+    const int chunks = n / 8;
+    Pack8<float> hv[RN_CHUNKS];
+    Pack8<T> dv[RN_CHUNKS];
+#pragma unroll
+    for (int c = 0; c < RN_CHUNKS; ++c) {
+        const int chunk = threadIdx.x + c * RN_THREADS;
+        if (chunk < chunks) {
+            hv[c] = *reinterpret_cast<const Pack8<float>*>(hr + chunk * 8);
+            if (dr) dv[c] = *reinterpret_cast<const Pack8<T>*>(dr + chunk * 8);
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < RN_CHUNKS; ++c) {
+        const int chunk = threadIdx.x + c * RN_THREADS;
+        if (chunk < chunks) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float v = hv[c].get(i);
+                if (dr) v += dv[c].get(i);
+                hv[c].set(i, v);
+                ss += v * v;
+            }
+            if (dr && write_h) *reinterpret_cast<Pack8<float>*>(hr + chunk * 8) = hv[c];
+        }
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = rsqrtf(ss / (float)n + eps);
+    T* o = out + (size_t)r * n;
+#pragma unroll
+    for (int c = 0; c < RN_CHUNKS; ++c) {
+        const int chunk = threadIdx.x + c * RN_THREADS;
+        if (chunk < chunks) {
+            const Pack8<float> wv = *reinterpret_cast<const Pack8<float>*>(w + chunk * 8);
+            Pack8<T> ov;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ov.set(i, hv[c].get(i) * inv * wv.get(i));
+            *reinterpret_cast<Pack8<T>*>(o + chunk * 8) = ov;
+        }
+    }
+}
+
 // RMSNorm of rows held in the activation type (no residual stream involved).
 template <typename T>
 __global__ void rmsnorm_act_kernel(const T* __restrict__ x, const float* __restrict__ w,
@@ -212,14 +282,26 @@ LC_API int lc_rmsnorm(float* h, const void* delta, const int* rows, const float*
     LC_CHECK(h && w && out, "rmsnorm: null pointer");
     LC_CHECK(!(rows && write_h), "rmsnorm: gathered rows cannot be written back");
     const int threads = n >= 1024 ? 256 : (n >= 256 ? 128 : 64);
-    if (dt == DT_F32)
-        rmsnorm_kernel<float><<<R, threads, 0, stream>>>(h, (const float*)delta, rows, w, eps,
-                                                         (float*)out, n, write_h);
-    else if (dt == DT_BF16)
-        rmsnorm_kernel<bf16><<<R, threads, 0, stream>>>(h, (const bf16*)delta, rows, w, eps,
-                                                        (bf16*)out, n, write_h);
-    else
+    const bool vec = n % 8 == 0 && n >= 512 && n <= RN_THREADS * RN_CHUNKS * 8 &&
+                     (uintptr_t)h % 16 == 0 && (uintptr_t)delta % 16 == 0 && (uintptr_t)out % 16 == 0 &&
+                     (uintptr_t)w % 16 == 0;
+    if (dt == DT_F32) {
+        if (vec)
+            rmsnorm_vec_kernel<float><<<R, RN_THREADS, 0, stream>>>(h, (const float*)delta, rows, w, eps,
+                                                                    (float*)out, n, write_h);
+        else
+            rmsnorm_kernel<float><<<R, threads, 0, stream>>>(h, (const float*)delta, rows, w, eps,
+                                                             (float*)out, n, write_h);
+    } else if (dt == DT_BF16) {
+        if (vec)
+            rmsnorm_vec_kernel<bf16><<<R, RN_THREADS, 0, stream>>>(h, (const bf16*)delta, rows, w, eps,
+                                                                   (bf16*)out, n, write_h);
+        else
+            rmsnorm_kernel<bf16><<<R, threads, 0, stream>>>(h, (const bf16*)delta, rows, w, eps,
+                                                            (bf16*)out, n, write_h);
+    } else {
         LC_CHECK(false, "rmsnorm: unknown dtype %d", dt);
+    }
     LC_LAUNCH_CHECK("rmsnorm");
     return 0;
 }

@@ -26,57 +26,69 @@ template <> __device__ __forceinline__ void store_out<float>(float* p, float v) 
 template <> __device__ __forceinline__ void store_out<bf16>(bf16* p, float v) { *p = static_cast<bf16>(v); }
 
 // ------------------------------------------------------------------------------- skinny
-constexpr int SK_ROWS = 16;    // rows of w per workgroup
 constexpr int SK_KBLOCK = 128; // k elements per wave iteration
 
-template <int MT, int WAVES, typename TO>
+// MT: tiles of 16 rows of x; NT: tiles of 16 rows of w per workgroup; the WAVES waves of a
+// workgroup take the k blocks in turn.
+template <int MT, int NT, int WAVES, int UNROLL, typename TO>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __restrict__ x,
                                                                  const bf16* __restrict__ w,
                                                                  TO* __restrict__ out, int M, int N,
                                                                  int K) {
-    __shared__ float red[WAVES * MT * 256];
+    __shared__ float red[WAVES * MT * NT * 256];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * SK_ROWS;
-    const int row = min(n0 + r, N - 1);
-    const bf16* wp = w + (size_t)row * K + g * 8;
+    const int n0 = blockIdx.x * (16 * NT);
+    const bf16* wp[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) wp[nt] = w + (size_t)min(n0 + nt * 16 + r, N - 1) * K + g * 8;
     const bf16* xp[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) xp[mt] = x + (size_t)min(mt * 16 + r, M - 1) * K + g * 8;
 
-    floatx4 acc[MT];
+    floatx4 acc[NT][MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     const int kblocks = K / SK_KBLOCK;
-#pragma unroll 2
+#pragma unroll UNROLL
     for (int kb = wave; kb < kblocks; kb += WAVES) {
         const int k0 = kb * SK_KBLOCK;
-        bf16x8 a[4];
+        bf16x8 a[NT][4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) a[j] = *reinterpret_cast<const bf16x8*>(wp + k0 + j * 32);
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) a[nt][j] = *reinterpret_cast<const bf16x8*>(wp[nt] + k0 + j * 32);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             bf16x8 b[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) b[j] = *reinterpret_cast<const bf16x8*>(xp[mt] + k0 + j * 32);
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[j], acc[mt], 0, 0, 0);
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][j], b[j], acc[nt][mt], 0, 0, 0);
         }
     }
-    // acc[mt][v] = partial out[m = mt*16 + lane%16][n = n0 + (lane/16)*4 + v]
+    // acc[nt][mt][v] = partial out[m = mt*16 + lane%16][n = n0 + nt*16 + (lane/16)*4 + v]
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) red[(wave * MT + mt) * 256 + v * 64 + lane] = acc[mt][v];
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                red[((wave * NT + nt) * MT + mt) * 256 + v * 64 + lane] = acc[nt][mt][v];
     __syncthreads();
-    for (int idx = threadIdx.x; idx < MT * 256; idx += WAVES * 64) {
+    for (int idx = threadIdx.x; idx < NT * MT * 256; idx += WAVES * 64) {
         float total = 0.f;
 #pragma unroll
-        for (int wv = 0; wv < WAVES; ++wv) total += red[wv * MT * 256 + idx];
-        const int mt = idx >> 8, v = (idx >> 6) & 3, l = idx & 63;
-        const int m = mt * 16 + (l & 15), n = n0 + (l >> 4) * 4 + v;
+        for (int wv = 0; wv < WAVES; ++wv) total += red[wv * NT * MT * 256 + idx];
+        const int tile = idx >> 8, v = (idx >> 6) & 3, l = idx & 63;
+        const int nt = tile / MT, mt = tile % MT;
+        const int m = mt * 16 + (l & 15), n = n0 + nt * 16 + (l >> 4) * 4 + v;
         if (m < M && n < N) store_out<TO>(out + (size_t)m * N + n, total);
     }
 }
@@ -181,20 +193,20 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
         }
 }
 
-template <int MT, typename TO>
+template <int MT, int NT, int WAVES, int UNROLL, typename TO>
 static void launch_skinny(const bf16* x, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
-    constexpr int WAVES = 8;
-    gemm_skinny_kernel<MT, WAVES, TO><<<(N + SK_ROWS - 1) / SK_ROWS, WAVES * 64, 0, s>>>(x, w, out, M, N, K);
+    const int rows = 16 * NT;
+    gemm_skinny_kernel<MT, NT, WAVES, UNROLL, TO><<<(N + rows - 1) / rows, WAVES * 64, 0, s>>>(x, w, out, M, N, K);
 }
 
 template <typename TO>
 static int launch_bf16(const bf16* x, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
     if (M <= 64) {
         switch ((M + 15) / 16) {
-            case 1: launch_skinny<1, TO>(x, w, out, M, N, K, s); break;
-            case 2: launch_skinny<2, TO>(x, w, out, M, N, K, s); break;
-            case 3: launch_skinny<3, TO>(x, w, out, M, N, K, s); break;
-            default: launch_skinny<4, TO>(x, w, out, M, N, K, s); break;
+            case 1: launch_skinny<1, 1, 16, 2, TO>(x, w, out, M, N, K, s); break;
+            case 2: launch_skinny<2, 1, 16, 1, TO>(x, w, out, M, N, K, s); break;
+            case 3: launch_skinny<3, 2, 8, 1, TO>(x, w, out, M, N, K, s); break;
+            default: launch_skinny<4, 2, 8, 1, TO>(x, w, out, M, N, K, s); break;
         }
         LC_LAUNCH_CHECK("gemm_skinny");
     } else {

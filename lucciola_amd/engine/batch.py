@@ -58,6 +58,7 @@ class StepBatch:
     slot_ids: torch.Tensor        # int32 [R]
     groups: List[AttentionBatch] = field(default_factory=list)
     num_wanted: int = 0
+    buffer: Optional[torch.Tensor] = None   # the one device buffer all of the above view
 
 
 class _Packer:
@@ -76,17 +77,30 @@ class _Packer:
         self._size = (self._size + 3) & ~3   # keep every array 16-byte aligned
         return len(self._arrays) - 1
 
-    def upload(self, device) -> None:
+    def upload(self, device, into: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Send everything in one copy; ``into``: a device buffer of an earlier batch with the
+        very same layout, which is overwritten (so that kernels captured in a graph see the
+        new values at the old addresses)."""
         host = np.zeros(max(self._size, 4), dtype=np.int32)
         for arr, off in zip(self._arrays, self._offsets):
             host[off:off + arr.size] = arr
         dev = torch.device(device)
+        if into is not None and into.numel() != host.size:
+            raise ValueError("the batch does not have the layout of the buffer it is to reuse")
         if dev.type == "cuda":
             staging = torch.empty(host.size, dtype=torch.int32, pin_memory=True)
             staging.numpy()[:] = host
-            self._dev = staging.to(dev, non_blocking=True)
+            if into is not None:
+                into.copy_(staging, non_blocking=True)
+                self._dev = into
+            else:
+                self._dev = staging.to(dev, non_blocking=True)
+        elif into is not None:
+            into.copy_(torch.from_numpy(host))
+            self._dev = into
         else:
             self._dev = torch.from_numpy(host).to(dev)
+        return self._dev
 
     def view(self, handle: int, shape=None) -> torch.Tensor:
         off, n = self._offsets[handle], self._arrays[handle].size
@@ -94,8 +108,12 @@ class _Packer:
         return t.view(shape) if shape is not None else t
 
 
-def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device) -> StepBatch:
-    """Lay the entries out as one flat batch.  Pages for the new tokens must be reserved."""
+def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
+                pad_blocks: Optional[int] = None, into: Optional[torch.Tensor] = None) -> StepBatch:
+    """Lay the entries out as one flat batch.  Pages for the new tokens must be reserved.
+
+    ``pad_blocks``: width of the block tables (at least the longest table), so that batches of
+    the same make-up have the same layout; ``into``: the buffer of such an earlier batch."""
     bs = cache.block_size
     requests, q_start, first_pos, slot_list = [], [0], [], []
     token_ids: List[int] = []
@@ -143,6 +161,10 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device) -> St
     for gi, g in enumerate(cache.groups):
         tables = [g.tables[req] for req in requests]
         mb = max((len(t) for t in tables), default=1) or 1
+        if pad_blocks is not None:
+            if pad_blocks < mb:
+                raise ValueError(f"pad_blocks {pad_blocks} is below the longest block table {mb}")
+            mb = pad_blocks
         flat = np.full((R, mb), -1, dtype=np.int32)
         for r, t in enumerate(tables):
             flat[r, :len(t)] = t
@@ -155,7 +177,10 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device) -> St
                 slots[i] = page * bs + p % bs if page >= 0 else -1
         group_handles.append((pk.add(flat), mb, pk.add(slots)))
 
-    pk.upload(device)
+    buffer = pk.upload(device, into)
+    max_ctx = max(ctx_len, default=0)
+    if pad_blocks is not None:
+        max_ctx = pad_blocks * bs      # what the layout allows, not what this batch holds
     groups = []
     for (h_bt, mb, h_sl) in group_handles:
         groups.append(AttentionBatch(
@@ -163,11 +188,11 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device) -> St
             block_table=pk.view(h_bt, (R, mb)), q_start=pk.view(h_qs), ctx_len=pk.view(h_ctx),
             slots=pk.view(h_sl), num_decode=len(decode_tokens),
             decode_tokens=pk.view(h_dec), prefill_tiles=pk.view(h_tiles, (len(tiles) // 4, 4)),
-            max_ctx=max(ctx_len, default=0), all_decode=len(decode_tokens) == R))
+            max_ctx=max_ctx, all_decode=len(decode_tokens) == R))
     return StepBatch(
         num_tokens=T, num_requests=R, requests=requests, q_start=q_start,
         first_position=first_pos, slot_list=slot_list,
         max_position=max(positions, default=0),
         token_ids=pk.view(h_tok), positions=pk.view(h_pos), tok_req=pk.view(h_req),
         want_rows=pk.view(h_want), slot_ids=pk.view(h_slot), groups=groups,
-        num_wanted=len(want_rows))
+        num_wanted=len(want_rows), buffer=buffer)

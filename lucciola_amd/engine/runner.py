@@ -19,6 +19,11 @@ from ..models.causal_lm import CausalLM
 from .batch import SiteView, StepBatch, StepEntry, build_batch
 
 
+class _CapturedStep:
+    def __init__(self, graph, batch, sites, logits):
+        self.graph, self.batch, self.sites, self.logits = graph, batch, sites, logits
+
+
 class ModelRunner:
     def __init__(self, model: CausalLM, config: EngineConfig, num_blocks: Optional[int] = None):
         self.model = model
@@ -32,6 +37,12 @@ class ModelRunner:
         self.cache.allocate_tensors(config.dtype, self.device)
         self.steps = 0
         self.tokens = 0
+        # decode steps replayed from HIP graphs: (requests, block-table width) -> captured step
+        self.use_graphs = (config.use_graphs and self.device.type == "cuda"
+                           and config.dtype == torch.bfloat16 and model.graph_safe())
+        self._graphs: Dict[tuple, "_CapturedStep"] = {}
+        self._graph_epoch = None
+        self.graph_replays = 0
 
     # ------------------------------------------------------------------ sizing
     def _blocks_from_free_memory(self, needs) -> int:
@@ -101,13 +112,53 @@ class ModelRunner:
             for slot in fresh:
                 state[slot].zero_()
 
-        batch = build_batch(entries, self.cache, self.device)
-        logits = self.model.forward(batch, self._sites(batch))
+        if self.use_graphs and len(entries) <= self.config.graph_max_batch and all(
+                len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+            logits, num_tokens = self._graph_step(entries), len(entries)
+        else:
+            batch = build_batch(entries, self.cache, self.device)
+            logits, num_tokens = self.model.forward(batch, self._sites(batch)), batch.num_tokens
         for e in entries:
             self.cache.commit(e.request)
         self.steps += 1
-        self.tokens += batch.num_tokens
+        self.tokens += num_tokens
         return logits
+
+    # ------------------------------------------------------------------ graph replay
+    def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """A step of single tokens, one per request, each wanting its logits: captured once per
+        (number of requests, block-table width) as a HIP graph and replayed afterwards.  Only the
+        batch description changes between replays, and it lives in one device buffer that is
+        overwritten in place.  """
+        widest = max((len(g.tables[e.request]) for g in self.cache.groups for e in entries),
+                     default=1)
+        pad = max(64, -(-widest // 64) * 64)
+        epoch = self.model.position_epoch()
+        if epoch != self._graph_epoch:      # a position table was made anew: addresses changed
+            self._graphs.clear()
+            self._graph_epoch = epoch
+        key = (len(entries), pad)
+        captured = self._graphs.get(key)
+        next_position = max(self.cache.length(e.request) for e in entries)
+        if captured is None or not self.model.positions_ready(next_position):
+            batch = build_batch(entries, self.cache, self.device, pad_blocks=pad)
+            sites = self._sites(batch)
+            logits = self.model.forward(batch, sites)       # runs the step (and grows tables)
+            if self.model.position_epoch() != epoch:
+                self._graphs.clear()
+                self._graph_epoch = self.model.position_epoch()
+            if len(self._graphs) >= self.config.graph_cache_size:
+                self._graphs.pop(next(iter(self._graphs)))
+            torch.cuda.synchronize(self.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                static_logits = self.model.forward(batch, sites)
+            self._graphs[key] = _CapturedStep(graph, batch, sites, static_logits)
+            return logits
+        build_batch(entries, self.cache, self.device, pad_blocks=pad, into=captured.batch.buffer)
+        captured.graph.replay()
+        self.graph_replays += 1
+        return captured.logits.clone()      # the next replay overwrites the graph's own output
 
     def _sites(self, batch: StepBatch) -> List[SiteView]:
         sites = []

@@ -35,7 +35,8 @@ _SIGNATURES = {
     "lc_attn_decode_bf16": "pippppppppp" + "iiiiii" + "f" + "ii" + "p",
     "lc_attn_prefill_bf16": "pippppp" + "iiiiii" + "f" + "i" + "p",
     "lc_swiglu": "ppiiip",
-    "lc_sample": "ppppiip",
+    "lc_sample": "pppppiip",
+    "lc_sample_workspace": "i",
 }
 
 
@@ -335,6 +336,8 @@ def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,
         if temperature.shape[0] != R or uniform.shape[0] != R:
             raise KernelError("sample: one temperature and one uniform number per row")
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
-    _call("lc_sample", _ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(out), _c_int(R),
-          _c_int(V), _stream())
+    workspace = torch.empty((max(1, library().lc_sample_workspace(R)),), dtype=torch.float32,
+                            device=logits.device)
+    _call("lc_sample", _ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(out), _ptr(workspace),
+          _c_int(R), _c_int(V), _stream())
     return out

@@ -99,6 +99,27 @@ class CausalLM:
                          else self.layers[entry.layer].mixer.cache_need())
         return needs
 
+    def graph_safe(self) -> bool:
+        """Whether every part of every layer may be captured in a HIP graph."""
+        return all(getattr(part, "graph_safe", False)
+                   for layer in self.layers for _, part in layer.parts()) \
+            and getattr(self.final_norm, "graph_safe", False)
+
+    # ------------------------------------------------------------------ position tables
+    def _position_parts(self):
+        for layer in self.layers:
+            pos = getattr(layer.mixer, "position", None)
+            if pos is not None and hasattr(pos, "generation"):
+                yield pos
+
+    def position_epoch(self) -> int:
+        """Changes whenever a position table has been made anew (its address has changed)."""
+        return sum(p.generation for p in self._position_parts())
+
+    def positions_ready(self, position: int) -> bool:
+        """Whether every position table already covers ``position``."""
+        return all(p.capacity() > position for p in self._position_parts())
+
     # ------------------------------------------------------------------ forward
     def forward(self, batch: StepBatch, sites: List[SiteView]) -> torch.Tensor:
         """Run the batch's tokens through every site; float32 logits [wanted, vocab]."""

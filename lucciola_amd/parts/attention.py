@@ -24,6 +24,8 @@ from .feed_forward import stack_rows
 
 @MIXERS.register("attention")
 class Attention(Part):
+    graph_safe = True   # launches only kernels whose arguments stay put between steps
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  scale: Optional[float] = None, qk_norm: Optional[PartSpec] = None,
                  position: Optional[PartSpec] = None, window: Optional[int] = None):

@@ -47,6 +47,11 @@ class ResidualStream:
 class Part:
     """Base of all parts.  Subclasses set ``self.p`` from keyword parameters in ``__init__``."""
 
+    # True if ``forward`` only launches kernels on tensors whose addresses and shapes depend
+    # on nothing but the batch layout (no host-side reads of batch values, no loops over
+    # requests): such a part may be captured in a HIP graph and replayed.
+    graph_safe = False
+
     def __init__(self, **params: Any):
         self.params = dict(params)
 

@@ -23,6 +23,8 @@ def stack_rows(tensors):
 
 @FEED_FORWARDS.register("gated_mlp")
 class GatedMLP(Part):
+    graph_safe = True   # launches only kernels whose arguments stay put between steps
+
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
         super().__init__(hidden_size=hidden_size, intermediate_size=intermediate_size,
                          activation=activation)

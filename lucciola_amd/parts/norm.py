@@ -15,6 +15,8 @@ from .base import BuildContext, Part, ResidualStream
 
 @NORMS.register("rms")
 class RMSNorm(Part):
+    graph_safe = True   # launches only kernels whose arguments stay put between steps
+
     def __init__(self, size: int, eps: float):
         super().__init__(size=size, eps=eps)
         self.size, self.eps = int(size), float(eps)

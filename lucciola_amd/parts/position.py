@@ -26,6 +26,7 @@ class Rotary(Part):
         self.initial = int(max_positions)
         self._table: Optional[torch.Tensor] = None
         self._device = None
+        self.generation = 0      # counts how often the table has been made anew
 
     def bind(self, tensors, ctx: BuildContext) -> None:
         self._device = ctx.device
@@ -43,11 +44,16 @@ class Rotary(Part):
         """float32 [positions, rot]: cosines in the first half of a row, sines in the second."""
         need = max_position + 1
         if self._table is None or self._table.shape[0] < need:
-            count = max(need, min(self.initial, 8192), 256)
+            count = max(need, min(self.initial, 16384), 256)
             if self._table is not None:
                 count = max(count, 2 * self._table.shape[0])
             self._table = self._make(count)
+            self.generation += 1
         return self._table
+
+    def capacity(self) -> int:
+        """Positions the present table covers."""
+        return 0 if self._table is None else int(self._table.shape[0])
 
     def apply(self, qkv, nh, nkv, d, positions) -> None:  # the table path covers this part
         raise NotImplementedError

@@ -189,3 +189,39 @@ def test_trace_run_program(tmp_path, dtype):
         for r, key in enumerate(rows):
             got[key] = torch.from_numpy(data[r].astype("float64"))
     compare(got, cfg, weights, prompts, TOL[dtype])
+
+
+def test_graph_replay_matches_eager():
+    """Decode steps replayed from a captured HIP graph, with eager steps (prompt portions of
+    other requests, synchronisations) between the replays: every replay gives the logits of an
+    engine that never uses graphs."""
+    cfg, page, seed = configs.ALL["C"]
+    weights = random_weights(cfg, seed)
+    prompts = prompts_for(cfg, [40, 75, 20], seed + 60)
+    extra = prompts_for(cfg, [90], seed + 61)["r0"]
+    results = {}
+    for use_graphs in (False, True):
+        arch = architecture_for(cfg)
+        model = _build(arch.model_spec(arch.read_config(cfg)), DictSource(weights), "bfloat16", DEV)
+        from lucciola_amd.engine.runner import ModelRunner
+        from lucciola_amd.engine.batch import StepEntry
+        runner = ModelRunner(model, EngineConfig(dtype="bfloat16", block_size=page, max_blocks=64,
+                                                 max_seqs=8, device=DEV, use_graphs=use_graphs))
+        rows = []
+        for name, ids in prompts.items():
+            runner.step([StepEntry(name, ids[:10], [])])
+        fed = {name: 10 for name in prompts}
+        for step in range(10):
+            entries = [StepEntry(n, [prompts[n][fed[n]]], [0]) for n in prompts]
+            rows.append(runner.step(entries).float().cpu())
+            for n in prompts:
+                fed[n] += 1
+            if step % 3 == 1:      # eager work between replays
+                runner.step([StepEntry("extra", extra[step * 5:step * 5 + 5], [4])])
+                torch.cuda.synchronize()
+        results[use_graphs] = torch.stack(rows)
+        if use_graphs:
+            assert runner.graph_replays >= 8
+        else:
+            assert runner.graph_replays == 0
+    assert torch.equal(results[True], results[False])
