@@ -11,6 +11,7 @@ import json
 import mmap
 import os
 import struct
+import warnings
 from dataclasses import dataclass
 from typing import Dict, Iterable, Iterator, List, Tuple
 
@@ -90,8 +91,10 @@ class SafetensorsFile:
         count = int(np.prod(entry.shape, dtype=np.int64))
         if count == 0:
             return torch.empty(entry.shape, dtype=entry.dtype)
-        flat = torch.frombuffer(self._map, dtype=entry.dtype, count=count,
-                                offset=self._base + entry.begin)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore", UserWarning)   # the mapping is read-only, and is only read
+            flat = torch.frombuffer(self._map, dtype=entry.dtype, count=count,
+                                    offset=self._base + entry.begin)
         return flat.view(entry.shape)
 
     def close(self) -> None:

@@ -1,0 +1,146 @@
+"""The cache manager's bookkeeping: no page lost, held twice or freed twice, under random
+orders of requests; groups with a window give back the pages the window has passed; slots."""
+import random
+
+import pytest
+
+from lucciola_amd.cache.manager import CacheManager
+from lucciola_amd.cache.page_pool import OutOfPages, PagePool, SlotPool
+from lucciola_amd.cache.specs import FixedState, PagedKV
+
+FULL = PagedKV(2, 16)
+WINDOW = PagedKV(2, 16, window=10)
+
+
+def test_pool_is_first_in_first_out():
+    # src/block_manager.cc:26-40: allocate pops the front, free pushes to the back
+    pool = PagePool(4)
+    assert [pool.allocate() for _ in range(4)] == [0, 1, 2, 3]
+    with pytest.raises(OutOfPages):
+        pool.allocate()
+    pool.free(2)
+    pool.free(0)
+    assert [pool.allocate(), pool.allocate()] == [2, 0]
+    with pytest.raises(ValueError, match="not held"):
+        pool.free(7)
+    pool.free(1)
+    with pytest.raises(ValueError, match="freed twice"):
+        pool.free(1)
+    pool.check()
+
+
+def test_slots():
+    slots = SlotPool(3)
+    a, b, c = slots.allocate(), slots.allocate(), slots.allocate()
+    assert (a, b, c) == (0, 1, 2)
+    with pytest.raises(OutOfPages):
+        slots.allocate()
+    slots.free(b)
+    assert slots.allocate() == 1
+    with pytest.raises(ValueError):
+        slots.free(5)
+    slots.check()
+
+
+def test_groups_are_formed_by_equal_needs():
+    cm = CacheManager([FULL, WINDOW, FULL, None, FixedState((3,)), WINDOW], 4, 20, 4)
+    assert [g.sites for g in cm.groups] == [[0, 2], [1, 5]]
+    assert cm.state_sites == [4]
+    assert cm.site_group == {0: 0, 2: 0, 1: 1, 5: 1}
+
+
+def test_pages_follow_the_length():
+    cm = CacheManager([FULL], 4, 10, 2)
+    cm.admit("a")
+    cm.reserve("a", 5)
+    assert cm.block_table(0, "a") == [0, 1] and cm.length("a") == 0
+    cm.commit("a")
+    assert cm.length("a") == 5
+    for expect in ([0, 1], [0, 1], [0, 1], [0, 1, 2]):     # lengths 6, 7, 8, 9
+        cm.reserve("a", 1)
+        cm.commit("a")
+        assert cm.block_table(0, "a") == expect
+    assert cm.slot_of_token(0, "a", 8) == 2 * 4 + 0
+    cm.release("a")
+    assert cm.groups[0].pool.num_free() == 10
+    cm.check()
+
+
+def test_reserve_takes_all_or_nothing():
+    cm = CacheManager([FULL, WINDOW], 4, 3, 2)
+    cm.admit("a")
+    cm.reserve("a", 8)                      # two pages in each group
+    cm.admit("b")
+    assert not cm.can_reserve("b", 5)       # needs two, one is free
+    with pytest.raises(OutOfPages):
+        cm.reserve("b", 5)
+    assert cm.block_table(0, "b") == [] and cm.block_table(1, "b") == []
+    assert cm.can_reserve("b", 4) and not cm.can_reserve("b", 4, {0: 1})
+    assert cm.can_reserve(None, 4) and not cm.can_reserve(None, 5)
+    cm.check()
+
+
+def test_window_gives_pages_back():
+    cm = CacheManager([FULL, WINDOW], 4, 50, 2)      # window of 10 positions
+    cm.admit("a")
+    cm.reserve("a", 30)
+    cm.commit("a")
+    # the next query is at position 30 and reads keys 21..30: pages 0..4 (keys 0..19) are passed
+    assert cm.block_table(1, "a")[:5] == [-1] * 5 and all(p >= 0 for p in cm.block_table(1, "a")[5:])
+    assert all(p >= 0 for p in cm.block_table(0, "a"))
+    assert cm.groups[1].pool.num_free() == 50 - 3 and cm.groups[0].pool.num_free() == 50 - 8
+    with pytest.raises(RuntimeError, match="given back"):
+        cm.slot_of_token(1, "a", 3)
+    for _ in range(40):
+        cm.reserve("a", 1)
+        cm.commit("a")
+        held = [p for p in cm.block_table(1, "a") if p >= 0]
+        assert len(held) <= 4                    # ceil(10 / 4) + 1
+        cm.check()
+    cm.release("a")
+    assert all(g.pool.num_free() == 50 for g in cm.groups)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_orders_of_requests(seed):
+    rng = random.Random(seed)
+    bs = rng.choice([1, 4, 16])
+    cm = CacheManager([FULL, WINDOW, FixedState((2,))], bs, 40, 5)
+    lengths = {}
+    for step in range(600):
+        action = rng.random()
+        if action < 0.2 and cm.can_admit():
+            name = f"r{step}"
+            cm.admit(name)
+            lengths[name] = 0
+        elif action < 0.85 and lengths:
+            name = rng.choice(list(lengths))
+            n = rng.choice([1, 1, 1, 2, 7, 20])
+            if cm.can_reserve(name, n):
+                cm.reserve(name, n)
+                if rng.random() < 0.9:
+                    cm.commit(name)
+                    lengths[name] += n
+                else:               # a step that is given up before it ran
+                    cm.release(name)
+                    del lengths[name]
+            else:
+                with pytest.raises(OutOfPages):
+                    cm.reserve(name, n)
+        elif lengths:
+            name = rng.choice(list(lengths))
+            cm.release(name)
+            del lengths[name]
+        cm.check()
+        used = sum(-(-n // bs) for n in lengths.values())
+        assert cm.groups[0].pool.num_free() == 40 - used
+        for name, n in lengths.items():
+            assert cm.length(name) == n
+            table = cm.block_table(1, name)
+            first_needed = max(0, n - 10 + 1)
+            for idx, page in enumerate(table):
+                assert (page < 0) == ((idx + 1) * bs <= first_needed)
+    for name in list(lengths):
+        cm.release(name)
+    cm.check()
+    assert all(g.pool.num_free() == 40 for g in cm.groups) and cm.slots.num_free() == 5
