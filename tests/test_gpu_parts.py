@@ -1,0 +1,310 @@
+"""Each part of a layer alone against the plain implementation, a run order that names a
+layer twice and lets a site read another site's cache, and a toy architecture with a mixer
+that keeps state of its own: registered, built and stepped from this file alone."""
+import math
+
+import pytest
+import torch
+
+import configs
+import plain_qwen3 as plain
+import traces
+from helpers import compare, prompts_for, random_weights, replay
+from lucciola_amd import parts  # noqa: F401  (registers the built-in parts)
+from lucciola_amd.cache.manager import CacheManager
+from lucciola_amd.cache.specs import FixedState, PagedKV
+from lucciola_amd.config.engine_config import EngineConfig
+from lucciola_amd.config.registry import ARCHITECTURES, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Architecture
+from lucciola_amd.config.specs import LayerSpec, ModelSpec, PartSpec, RunEntry
+from lucciola_amd.engine.batch import SiteView, StepEntry, build_batch
+from lucciola_amd.engine.loading import _build
+from lucciola_amd.engine.runner import ModelRunner
+from lucciola_amd.kernels import ops
+from lucciola_amd.models.causal_lm import declared_tensors
+from lucciola_amd.models.qwen3 import qwen3_model_spec
+from lucciola_amd.parts.base import BuildContext, Part, ResidualStream, build_part
+from lucciola_amd.weights.loader import DictSource, ParamDecl
+from lucciola_amd.weights.random_init import random_tensors
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+DTYPES = [torch.float32, torch.bfloat16]
+F64 = torch.float64
+
+
+def rnd(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def rel(got, want):
+    return float((got.double().cpu() - want.double().cpu()).abs().max() / want.double().abs().max())
+
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_norm_part(dtype):
+    ctx = BuildContext(dtype, DEV)
+    norm = build_part(NORMS, PartSpec("rms", {"size": 200, "eps": 1e-5}))
+    assert norm.declare()["weight"].shape == (200,) and norm.declare()["weight"].init == "ones_plus_normal"
+    w = 1 + rnd(200, seed=1, scale=0.1)
+    norm.bind({"weight": w}, ctx)
+    h, delta = rnd(9, 200, seed=2), rnd(9, 200, seed=3, dtype=dtype)
+    stream = ResidualStream(h.clone())
+    stream.pending = delta
+    want_h = h.double() + delta.double()
+    x = norm.add_norm(stream)
+    assert stream.pending is None and x.dtype == dtype
+    torch.testing.assert_close(stream.h.double(), want_h, rtol=1e-6, atol=1e-6)
+    assert rel(x, plain.rmsnorm(want_h.cpu(), w.cpu(), 1e-5)) < TOL[dtype]
+    rows = torch.tensor([8, 2], dtype=torch.int32, device=DEV)
+    stream.pending = delta
+    picked = norm.add_norm_rows(stream, rows)
+    want = plain.rmsnorm((want_h + delta.double())[rows.long()].cpu(), w.cpu(), 1e-5)
+    assert rel(picked, want) < TOL[dtype]
+
+
+def test_rotary_part():
+    rot = build_part(POSITION_ENCODINGS, PartSpec("rotary", {"rotary_dim": 48, "theta": 50000.0,
+                                                              "max_positions": 300}))
+    rot.bind({}, BuildContext(torch.float32, DEV))
+    table = rot.rotary_table(100)
+    assert table.shape[1] == 48 and table.shape[0] > 100
+    x = rnd(5, 3, 48, seed=4).cpu().double()
+    positions = [0, 1, 17, 99, 100]
+    want = plain.rope(x, positions, 50000.0)
+    cs = table[torch.tensor(positions)].cpu().double()
+    cos, sin = cs[:, None, :24], cs[:, None, 24:]
+    got = torch.cat([x[..., :24] * cos - x[..., 24:] * sin, x[..., :24] * sin + x[..., 24:] * cos], -1)
+    torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-6)
+    epoch = rot.generation
+    bigger = rot.rotary_table(5000)           # grows on demand
+    assert bigger.shape[0] > 5000 and rot.generation == epoch + 1
+    torch.testing.assert_close(bigger[:table.shape[0]], table)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_feed_forward_part(dtype):
+    ff = build_part(FEED_FORWARDS, PartSpec("gated_mlp", {"hidden_size": 72, "intermediate_size": 200}))
+    assert {k: v.shape for k, v in ff.declare().items()} == {
+        "gate_proj": (200, 72), "up_proj": (200, 72), "down_proj": (72, 200)}
+    w = {"gate_proj": rnd(200, 72, seed=5, scale=0.1, dtype=torch.bfloat16),
+         "up_proj": rnd(200, 72, seed=6, scale=0.1, dtype=torch.bfloat16),
+         "down_proj": rnd(72, 200, seed=7, scale=0.1, dtype=torch.bfloat16)}
+    ff.bind(w, BuildContext(dtype, DEV))
+    x = rnd(11, 72, seed=8, dtype=dtype)
+    named = {"m.gate_proj.weight": w["gate_proj"].cpu(), "m.up_proj.weight": w["up_proj"].cpu(),
+             "m.down_proj.weight": w["down_proj"].cpu()}
+    assert rel(ff.forward(x), plain.mlp_block(x.cpu(), named, "m.")) < TOL[dtype]
+    with pytest.raises(ValueError, match="activation"):
+        build_part(FEED_FORWARDS, PartSpec("gated_mlp", {"hidden_size": 8, "intermediate_size": 8,
+                                                         "activation": "gelu"}))
+
+
+def attention_site(part, T, page, dtype, first=0):
+    """A one-request batch and a cache for one attention part."""
+    cache = CacheManager([part.cache_need()], page, 64, 2)
+    cache.allocate_tensors(dtype, DEV)
+    cache.admit("r")
+    if first:
+        cache.reserve("r", first)
+        cache.commit("r")
+    cache.reserve("r", T)
+    batch = build_batch([StepEntry("r", list(range(T)), [])], cache, DEV)
+    return SiteView(batch=batch, index=0, writes_cache=True, page_size=page, kv=cache.kv[0],
+                    attn=batch.groups[0]), cache
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,page,window", [(4, 2, 16, 4, None), (6, 2, 48, 16, 9), (8, 1, 32, 16, None),
+                                                  (4, 4, 64, 16, None)])
+def test_attention_part(dtype, nh, nkv, d, page, window):
+    H, T, eps, theta = 40, 37, 1e-5, 1e4
+    spec = PartSpec("attention", {
+        "hidden_size": H, "num_heads": nh, "num_kv_heads": nkv, "head_dim": d, "window": window,
+        "qk_norm": PartSpec("rms", {"size": d, "eps": eps}),
+        "position": PartSpec("rotary", {"rotary_dim": d, "theta": theta, "max_positions": 64})})
+    part = build_part(MIXERS, spec)
+    assert part.cache_need() == PagedKV(nkv, d, window)
+    names = {"q_proj": (nh * d, H), "k_proj": (nkv * d, H), "v_proj": (nkv * d, H), "o_proj": (H, nh * d),
+             "q_norm.weight": (d,), "k_norm.weight": (d,)}
+    assert {k: v.shape for k, v in part.declare().items()} == names
+    w = {}
+    for i, (name, shape) in enumerate(names.items()):
+        if name.endswith("norm.weight"):
+            w[name] = 1 + rnd(*shape, seed=20 + i, scale=0.2)
+        else:
+            w[name] = rnd(*shape, seed=20 + i, scale=0.3, dtype=torch.bfloat16)
+    part.bind(dict(w), BuildContext(dtype, DEV))
+    x = rnd(T, H, seed=30, dtype=dtype)
+    site, _ = attention_site(part, T, page, dtype)
+    got = part.forward(x, site)
+    cfg = {"num_attention_heads": nh, "num_key_value_heads": nkv, "head_dim": d,
+           "rms_norm_eps": eps, "rope_theta": theta}
+    named = {"a." + k + ("" if k.endswith(".weight") else ".weight"): v.cpu() for k, v in w.items()}
+    want, _ = plain.attention_block(x.cpu(), named, "a.", cfg, list(range(T)), window)
+    assert rel(got, want) < TOL[dtype] * (2 if dtype == torch.bfloat16 else 1)
+
+
+# ------------------------------------------------------------------ the run order is data
+def looped_spec(cfg_dict):
+    """Qwen3 parts in another order: layer 0 runs twice (two sites, two caches), and the last
+    site runs layer 1 on the cache that layer 1's first site wrote."""
+    from lucciola_amd.config.model_config import Qwen3Config
+    from dataclasses import replace
+    spec = qwen3_model_spec(Qwen3Config.from_dict(cfg_dict))
+    return replace(spec, run_order=[RunEntry(0), RunEntry(1), RunEntry(0), RunEntry(1, cache_of=1)])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_run_order_names_a_layer_twice_and_shares_a_cache(dtype):
+    cfg, page, seed = configs.ALL["A"]
+    ARCHITECTURES.register("LoopedQwen3", Architecture("LoopedQwen3", read_config=lambda d: d,
+                                                       model_spec=looped_spec), replace=True)
+    try:
+        cfg = dict(cfg, architectures=["LoopedQwen3"])
+        weights = random_weights(cfg, seed, std=0.05)
+        model = _build(looped_spec(cfg), DictSource(weights), dtype, DEV)
+        assert model.site_needs()[3] is None and model.site_needs()[0] == model.site_needs()[2]
+        prompts = prompts_for(cfg, [30, 9, 21], seed)
+        refs = {n: plain.forward(cfg, weights, ids, run_order=[(0, None), (1, None), (0, None), (1, 1)])
+                for n, ids in prompts.items()}
+        for family in (traces.whole, traces.chunked, traces.mixed):
+            steps = family(prompts)
+            runner = ModelRunner(model, EngineConfig(dtype=dtype, block_size=page, max_seqs=4, device="cuda:0",
+                                                     max_blocks=traces.max_live_tokens(steps, page) // page))
+            assert len(runner.cache.kv) == 3          # three sites own a cache, one borrows
+            got = replay(runner, steps)
+            compare(got, cfg, weights, prompts, 2e-5 if dtype == "float32" else 3e-2, refs)
+    finally:
+        ARCHITECTURES.unregister("LoopedQwen3")
+
+
+# ------------------------------------------------------------------ a toy architecture
+class ToyDecay(Part):
+    """s_t = decay * s_{t-1} + W_in x_t;  y_t = W_out s_t.  The state s lives in the request's
+    slot; tokens of a portion are taken in order."""
+
+    def __init__(self, hidden_size, state_size, decay):
+        super().__init__(hidden_size=hidden_size, state_size=state_size, decay=decay)
+        self.H, self.S, self.decay = hidden_size, state_size, decay
+
+    def declare(self):
+        return {"in_proj": ParamDecl((self.S, self.H)), "out_proj": ParamDecl((self.H, self.S))}
+
+    def bind(self, tensors, ctx):
+        self.w_in, self.w_out, self.dtype = tensors["in_proj"], tensors["out_proj"], ctx.dtype
+
+    def cache_need(self):
+        return FixedState((self.S,), torch.float32)
+
+    def forward(self, x, site):
+        u = ops.gemm(x, self.w_in, torch.float32)                 # [T, S]
+        states = torch.empty_like(u)
+        batch = site.batch
+        for r, slot in enumerate(batch.slot_list):
+            s = site.state[slot]
+            for t in range(batch.q_start[r], batch.q_start[r + 1]):
+                s = self.decay * s + u[t]
+                states[t] = s
+            site.state[slot] = s
+        return ops.gemm(states.to(self.dtype), self.w_out, self.dtype)
+
+
+class ToyScale(Part):
+    """A feed-forward of one matrix."""
+
+    def __init__(self, hidden_size):
+        super().__init__(hidden_size=hidden_size)
+        self.H = hidden_size
+
+    def declare(self):
+        return {"proj": ParamDecl((self.H, self.H))}
+
+    def bind(self, tensors, ctx):
+        self.w, self.dtype = tensors["proj"], ctx.dtype
+
+    def forward(self, x):
+        return ops.gemm(x, self.w, self.dtype)
+
+
+TOY = {"architectures": ["ToyForCausalLM"], "hidden_size": 24, "vocab_size": 50, "state_size": 10,
+       "decay": 0.8, "eps": 1e-5, "heads": 2, "head_dim": 16}
+
+
+def toy_spec(c):
+    norm = PartSpec("rms", {"size": c["hidden_size"], "eps": c["eps"]})
+    attn = PartSpec("attention", {"hidden_size": c["hidden_size"], "num_heads": c["heads"],
+                                  "num_kv_heads": 1, "head_dim": c["head_dim"],
+                                  "position": PartSpec("rotary", {"rotary_dim": c["head_dim"], "theta": 100.0})})
+    decay = PartSpec("toy_decay", {"hidden_size": c["hidden_size"], "state_size": c["state_size"],
+                                   "decay": c["decay"]})
+    ff = PartSpec("toy_scale", {"hidden_size": c["hidden_size"]})
+    layers = []
+    for i, mixer in enumerate([decay, attn, decay]):
+        names = {"mixer_norm.weight": f"l{i}.n1", "feed_forward_norm.weight": f"l{i}.n2",
+                 "feed_forward.proj": f"l{i}.ff"}
+        if mixer is attn:
+            names.update({f"mixer.{k}_proj": f"l{i}.{k}" for k in "qkvo"})
+        else:
+            names.update({"mixer.in_proj": f"l{i}.in", "mixer.out_proj": f"l{i}.out"})
+        layers.append(LayerSpec("prenorm_residual", mixer, ff, norm, norm, names))
+    return ModelSpec(hidden_size=c["hidden_size"], vocab_size=c["vocab_size"], embedding_name="emb",
+                     layers=layers, run_order=[RunEntry(0), RunEntry(1), RunEntry(2), RunEntry(0)],
+                     final_norm=norm, final_norm_names={"weight": "final"}, head_name="head", init_std=0.2)
+
+
+def toy_plain(c, w, ids):
+    """Whole sequence, float64, no cache."""
+    w = {k: v.double() for k, v in w.items()}
+    T = len(ids)
+    h = w["emb"][torch.tensor(ids)]
+    for layer in (0, 1, 2, 0):
+        x = plain.rmsnorm(h, w[f"l{layer}.n1"], c["eps"])
+        if layer == 1:
+            q = plain.rope((x @ w["l1.q"].T).view(T, c["heads"], c["head_dim"]), range(T), 100.0)
+            k = plain.rope((x @ w["l1.k"].T).view(T, 1, c["head_dim"]), range(T), 100.0)
+            v = (x @ w["l1.v"].T).view(T, 1, c["head_dim"])
+            a = plain.attention(q, k, v, list(range(T))).reshape(T, -1) @ w["l1.o"].T
+        else:
+            u = x @ w[f"l{layer}.in"].T
+            s = torch.zeros(c["state_size"], dtype=F64)
+            states = []
+            for t in range(T):
+                s = c["decay"] * s + u[t]
+                states.append(s)
+            a = torch.stack(states) @ w[f"l{layer}.out"].T
+        h = h + a
+        h = h + plain.rmsnorm(h, w[f"l{layer}.n2"], c["eps"]) @ w[f"l{layer}.ff"].T
+    return plain.rmsnorm(h, w["final"], c["eps"]) @ w["head"].T
+
+
+def test_toy_architecture_with_a_stateful_mixer():
+    MIXERS.register("toy_decay", ToyDecay, replace=True)
+    FEED_FORWARDS.register("toy_scale", ToyScale, replace=True)
+    ARCHITECTURES.register("ToyForCausalLM", Architecture("ToyForCausalLM", read_config=dict,
+                                                          model_spec=toy_spec), replace=True)
+    try:
+        spec = toy_spec(TOY)
+        weights = dict(random_tensors(declared_tensors(spec), 5, spec.init_std, torch.float32))
+        model = _build(spec, DictSource(weights), "float32", "cuda:0")
+        needs = model.site_needs()
+        assert isinstance(needs[0], FixedState) and isinstance(needs[1], PagedKV) and needs[3] == needs[0]
+        assert not model.graph_safe()
+        prompts = prompts_for({"vocab_size": 50}, [25, 7, 40, 13, 31], 3)
+        refs = {n: toy_plain(TOY, weights, ids) for n, ids in prompts.items()}
+        for family in (traces.whole, traces.tail_decode, traces.chunked, traces.mixed):
+            steps = family(prompts)
+            runner = ModelRunner(model, EngineConfig(dtype="float32", block_size=4, max_seqs=4, device="cuda:0",
+                                                     max_blocks=traces.max_live_tokens(steps, 4) // 4))
+            assert sorted(runner.cache.state) == [0, 2, 3] and sorted(runner.cache.kv) == [1]
+            for state in runner.cache.state.values():
+                state.fill_(7.0)                       # a new request must not see an old state
+            got = replay(runner, steps)
+            compare(got, TOY, weights, prompts, 2e-5, refs)
+    finally:
+        MIXERS.unregister("toy_decay")
+        FEED_FORWARDS.unregister("toy_scale")
+        ARCHITECTURES.unregister("ToyForCausalLM")
