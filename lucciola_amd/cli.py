@@ -1,0 +1,106 @@
+"""The command line, in the manner of the reference's ``lucciola_chat``
+(examples/qwen_dynamic.cc:40-106: load the model, make the paged cache with ``max_blocks`` pages
+of ``block_size`` tokens, read a request per input line until ``exit``, run the scheduler loop
+and stream what is generated, at most 100 tokens a request).
+
+Requests are token ids here (there is no tokenizer): a line of ids separated by blanks or
+commas.  Options carry the reference's names where it has them: ``--max-blocks`` and
+``--block-size`` are the arguments of ``AsyncEngine(model_path, max_blocks, block_size)``
+(include/async_engine.h:24-25), ``--max-new-tokens`` that of ``generate_async``.
+
+    python -m lucciola_amd --model DIR                       # ids from standard input
+    python -m lucciola_amd --model DIR --prompt-ids 1,2,3 --prompt-ids 4,5
+    python -m lucciola_amd --random-config config.json --seed 0 --write-model DIR
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import re
+import sys
+from typing import List
+
+
+def _ids(text: str) -> List[int]:
+    return [int(t) for t in re.split(r"[,\s]+", text.strip()) if t]
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="lucciola_amd", description=__doc__,
+                                 formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--model", help="folder with config.json and model.safetensors")
+    ap.add_argument("--max-blocks", type=int, default=0,
+                    help="pages of the cache; 0 sizes it from free memory (the reference's default)")
+    ap.add_argument("--block-size", type=int, default=16, help="tokens in a page")
+    ap.add_argument("--max-new-tokens", type=int, default=100)
+    ap.add_argument("--temperature", type=float, default=0.0, help="0 is greedy")
+    ap.add_argument("--seed", type=int, default=0, help="of the sampler, or of --random-config")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--max-tokens-per-step", type=int, default=576)
+    ap.add_argument("--max-seqs", type=int, default=256)
+    ap.add_argument("--ignore-eos", action="store_true")
+    ap.add_argument("--prompt-ids", action="append", default=[],
+                    help="a request as comma-separated token ids (may be given several times)")
+    ap.add_argument("--prompt-ids-file", help="a file with one request of token ids per line")
+    ap.add_argument("--random-config", help="a config.json to make random weights for")
+    ap.add_argument("--write-model", help="with --random-config: the model folder to write")
+    ap.add_argument("--device", default="cuda:0")
+    args = ap.parse_args(argv)
+
+    if args.random_config:
+        if not args.write_model:
+            ap.error("--random-config needs --write-model DIR")
+        from .weights.random_init import write_model_folder
+        with open(args.random_config, "r", encoding="utf-8") as fh:
+            config = json.load(fh)
+        folder = write_model_folder(args.write_model, config, args.seed)
+        print(f"wrote {folder}")
+        if not args.model:
+            return 0
+    if not args.model:
+        ap.error("--model is required")
+
+    from .config.engine_config import EngineConfig
+    from .engine.llm_engine import LLMEngine
+    from .sampling.sampler import SamplingParams
+
+    engine = LLMEngine.from_folder(args.model, EngineConfig(
+        dtype=args.dtype, block_size=args.block_size, max_blocks=args.max_blocks,
+        max_tokens_per_step=args.max_tokens_per_step, max_seqs=args.max_seqs, device=args.device))
+    print(f"model ready: {len(engine.model.layers)} layers, {engine.runner.cache.num_blocks} pages "
+          f"of {args.block_size} tokens", file=sys.stderr, flush=True)
+
+    def params(i: int) -> SamplingParams:
+        return SamplingParams(max_new_tokens=args.max_new_tokens, temperature=args.temperature,
+                              seed=args.seed + i, ignore_eos=args.ignore_eos)
+
+    prompts = [_ids(p) for p in args.prompt_ids]
+    if args.prompt_ids_file:
+        with open(args.prompt_ids_file, "r", encoding="utf-8") as fh:
+            prompts += [_ids(line) for line in fh if line.strip()]
+    if prompts:
+        outputs = engine.generate(prompts, [params(i) for i in range(len(prompts))])
+        for out in outputs:
+            print(" ".join(str(t) for t in out), flush=True)
+        return 0
+
+    # interactive: a request per line, generated ids streamed as they come
+    count = 0
+    for line in sys.stdin:
+        line = line.strip()
+        if line == "exit":
+            break
+        if not line:
+            continue
+        try:
+            prompt = _ids(line)
+            engine.generate([prompt], [params(count)],
+                            on_token=lambda _id, tok, done: print(tok, end="\n" if done else " ", flush=True))
+        except ValueError as exc:
+            print(f"error: {exc}", file=sys.stderr, flush=True)
+        count += 1
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

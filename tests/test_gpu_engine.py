@@ -225,3 +225,48 @@ def test_graph_replay_matches_eager():
         else:
             assert runner.graph_replays == 0
     assert torch.equal(results[True], results[False])
+
+
+def test_command_line_and_async_engine(tmp_path):
+    """The command line and ``AsyncEngine(model_path, max_blocks, block_size)`` /
+    ``generate_async(prompt, max_new_tokens, callback)`` give the plain greedy tokens."""
+    import threading
+    from lucciola_amd import AsyncEngine
+    from lucciola_amd.weights.safetensors_io import SafetensorsFile
+    cfg, page, seed = configs.ALL["B"]
+    folder = write_model_folder(str(tmp_path / "model"), cfg, seed, std=0.3)
+    with SafetensorsFile(os.path.join(folder, "model.safetensors")) as f:
+        weights = {n: f.get(n).clone() for n in f.names()}
+    prompts = list(prompts_for(cfg, [4, 13], seed + 70).values())
+    want = [plain_qwen3.greedy(cfg, weights, p, 6) for p in prompts]
+
+    cmd = [sys.executable, "-m", "lucciola_amd", "--model", folder, "--dtype", "float32",
+           "--max-blocks", "32", "--block-size", str(page), "--max-new-tokens", "6"]
+    for p in prompts:
+        cmd += ["--prompt-ids", ",".join(map(str, p))]
+    proc = subprocess.run(cmd, cwd=ROOT, text=True, capture_output=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [[int(t) for t in line.split()] for line in proc.stdout.strip().splitlines()] == want
+    # interactive: a request per line until "exit"
+    proc = subprocess.run(cmd[:cmd.index("--prompt-ids")], cwd=ROOT, text=True, capture_output=True,
+                          timeout=600, input=" ".join(map(str, prompts[0])) + "\nexit\n")
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [int(t) for t in proc.stdout.split()] == want[0]
+
+    engine = AsyncEngine(folder, max_blocks=32, block_size=page, dtype="float32")
+    got = {0: [], 1: []}
+    done = [threading.Event(), threading.Event()]
+
+    def callback(i):
+        def cb(token, finished):
+            got[i].append(token)
+            if finished:
+                done[i].set()
+        return cb
+    try:
+        for i, p in enumerate(prompts):
+            engine.generate_async(p, 6, callback(i))
+        assert all(d.wait(120) for d in done)
+    finally:
+        engine.stop()
+    assert [got[0], got[1]] == want
