@@ -4,7 +4,8 @@
 //     the partial results (max, sum, unnormalised output) go to a workspace and a second
 //     kernel joins them.  The query heads that share a kv head form the columns of one
 //     matrix-core tile, so keys and values are read once per group.
-//   * prefill: a workgroup owns 64 query rows of one request and one head; each wave 16 rows.
+//   * prefill: a workgroup owns 64 query rows of one request and one or two heads of a kv
+//     head; pages go through LDS once per workgroup.
 //
 // Both run the same inner step on one page of 16 keys, written for the operand layouts of
 // the matrix instructions:
@@ -31,10 +32,11 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int PAGE = 16;
 
-template <int D>
+// QT: query column tiles (of 16 columns) that one wave carries; they share every K/V load.
+template <int D, int QT>
 struct AttnState {
-    float m, l;              // running maximum (log2 domain) and this lane's share of the sum
-    floatx4 o[D / 16];       // O^T tiles: o[t][v] = O[dim = 16 t + 4 (lane/16) + v][q = lane%16]
+    float m[QT], l[QT];      // running maximum and this lane's share of the sum
+    floatx4 o[QT][D / 16];   // O^T tiles: o[c][t][v] = O[dim = 16 t + 4 (lane/16) + v][q = 16 c + lane%16]
 };
 
 template <int D>
@@ -62,62 +64,69 @@ __device__ __forceinline__ short bf16_bits(float f) {
 }
 
 // One page of 16 keys starting at position `key0`.  lo/hi: the lowest and highest position
-// this lane's query column may see.
-template <int D>
-__device__ __forceinline__ void attend_page(AttnState<D>& st, const PageRegs<D>& r,
-                                            const bf16x8 (&bq)[D / 32], int key0, int lo, int hi,
+// this lane's query column (of each column tile) may see.
+template <int D, int QT>
+__device__ __forceinline__ void attend_page(AttnState<D, QT>& st, const PageRegs<D>& r,
+                                            const bf16x8 (&bq)[QT][D / 32], int key0,
+                                            const int (&lo)[QT], const int (&hi)[QT],
                                             float scale_log2, int lane) {
-    floatx4 s = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int i = 0; i < D / 32; ++i)
-        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(r.k[i], bq[i], s, 0, 0, 0);
     const int j0 = key0 + (lane >> 4) * 4;
-    float mx = -INFINITY;
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-        const int j = j0 + v;
-        s[v] = (j >= lo && j <= hi) ? s[v] * scale_log2 : -INFINITY;
-        mx = fmaxf(mx, s[v]);
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(st.m, mx);
-    const float alpha = (st.m == -INFINITY) ? 0.f : exp2f(st.m - m_new);
-    float p[4], psum = 0.f;
+    for (int c = 0; c < QT; ++c) {
+        floatx4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-        p[v] = (s[v] == -INFINITY) ? 0.f : exp2f(s[v] - m_new);
-        psum += p[v];
-    }
-    st.l = st.l * alpha + psum;
-    st.m = m_new;
-    short4v pb;
+        for (int i = 0; i < D / 32; ++i)
+            s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(r.k[i], bq[c][i], s, 0, 0, 0);
+        float mx = -INFINITY;
 #pragma unroll
-    for (int v = 0; v < 4; ++v) pb[v] = bf16_bits(p[v]);
+        for (int v = 0; v < 4; ++v) {
+            const int j = j0 + v;
+            s[v] = (j >= lo[c] && j <= hi[c]) ? s[v] * scale_log2 : -INFINITY;
+            mx = fmaxf(mx, s[v]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(st.m[c], mx);
+        const float alpha = (st.m[c] == -INFINITY) ? 0.f : exp2f(st.m[c] - m_new);
+        float p[4], psum = 0.f;
 #pragma unroll
-    for (int t = 0; t < D / 16; ++t) {
-        st.o[t] *= alpha;
-        st.o[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(r.v[t], pb, st.o[t], 0, 0, 0);
+        for (int v = 0; v < 4; ++v) {
+            p[v] = (s[v] == -INFINITY) ? 0.f : exp2f(s[v] - m_new);
+            psum += p[v];
+        }
+        st.l[c] = st.l[c] * alpha + psum;
+        st.m[c] = m_new;
+        short4v pb;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) pb[v] = bf16_bits(p[v]);
+#pragma unroll
+        for (int t = 0; t < D / 16; ++t) {
+            st.o[c][t] *= alpha;
+            st.o[c][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(r.v[t], pb, st.o[c][t], 0, 0, 0);
+        }
     }
 }
 
-template <int D>
-__device__ __forceinline__ void init_state(AttnState<D>& st) {
-    st.m = -INFINITY;
-    st.l = 0.f;
+template <int D, int QT>
+__device__ __forceinline__ void init_state(AttnState<D, QT>& st) {
 #pragma unroll
-    for (int t = 0; t < D / 16; ++t) st.o[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < QT; ++c) {
+        st.m[c] = -INFINITY;
+        st.l[c] = 0.f;
+#pragma unroll
+        for (int t = 0; t < D / 16; ++t) st.o[c][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
 }
 
 // Walk pages [begin, end) with stride `step`, the next page's loads in flight while the
 // current one is multiplied.
-template <int D>
-__device__ __forceinline__ void attend_range(AttnState<D>& st, const bf16x8 (&bq)[D / 32],
+template <int D, int QT>
+__device__ __forceinline__ void attend_range(AttnState<D, QT>& st, const bf16x8 (&bq)[QT][D / 32],
                                              const bf16* __restrict__ k_cache,
                                              const bf16* __restrict__ v_cache,
                                              const int* __restrict__ table, int begin, int end,
-                                             int step, int nkv, int kvh, int lo, int hi,
-                                             float scale_log2, int lane) {
+                                             int step, int nkv, int kvh, const int (&lo)[QT],
+                                             const int (&hi)[QT], float scale_log2, int lane) {
     if (begin >= end) return;
     PageRegs<D> cur, nxt;
     load_page<D>(cur, k_cache, v_cache, table[begin], nkv, kvh, lane);
@@ -128,7 +137,7 @@ __device__ __forceinline__ void attend_range(AttnState<D>& st, const bf16x8 (&bq
             load_page<D>(nxt, k_cache, v_cache, next_page, nkv, kvh, lane);
             if (pg + 2 * step < end) next_page = table[pg + 2 * step];
         }
-        attend_page<D>(st, cur, bq, pg * PAGE, lo, hi, scale_log2, lane);
+        attend_page<D, QT>(st, cur, bq, pg * PAGE, lo, hi, scale_log2, lane);
         if (more) cur = nxt;
     }
 }
@@ -158,26 +167,27 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const int end = min(begin + per, last_page + 1);
     const int* table = block_table + (size_t)req * max_blocks;
 
-    bf16x8 bq[D / 32];
+    bf16x8 bq[1][D / 32];
     {
         const bf16* qrow = qkv + (size_t)t * q_stride + (size_t)(kvh * G + min(q, G - 1)) * D + kg * 8;
 #pragma unroll
-        for (int i = 0; i < D / 32; ++i) bq[i] = *reinterpret_cast<const bf16x8*>(qrow + i * 32);
+        for (int i = 0; i < D / 32; ++i) bq[0][i] = *reinterpret_cast<const bf16x8*>(qrow + i * 32);
     }
-    AttnState<D> st;
-    init_state<D>(st);
-    attend_range<D>(st, bq, k_cache, v_cache, table, begin + wave, end, 4, nkv, kvh, j_lo, p,
-                    scale_log2, lane);
+    AttnState<D, 1> st;
+    init_state<D, 1>(st);
+    const int lo[1] = {j_lo}, hi[1] = {p};
+    attend_range<D, 1>(st, bq, k_cache, v_cache, table, begin + wave, end, 4, nkv, kvh, lo, hi,
+                       scale_log2, lane);
 
     // the waves' results meet in LDS
-    float l = st.l;
+    float l = st.l[0];
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
-    if (kg == 0) { sm_m[wave][q] = st.m; sm_l[wave][q] = l; }
+    if (kg == 0) { sm_m[wave][q] = st.m[0]; sm_l[wave][q] = l; }
 #pragma unroll
     for (int tt = 0; tt < D / 16; ++tt)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) sm_o[wave][(tt * 16 + kg * 4 + v) * 16 + q] = st.o[tt][v];
+        for (int v = 0; v < 4; ++v) sm_o[wave][(tt * 16 + kg * 4 + v) * 16 + q] = st.o[0][tt][v];
     __syncthreads();
     for (int idx = threadIdx.x; idx < D * 16; idx += 256) {
         const int dim = idx >> 4, qq = idx & 15;
@@ -236,51 +246,204 @@ __global__ __launch_bounds__(128) void attn_decode_join_kernel(const float* __re
 }
 
 // ------------------------------------------------------------------------------- prefill
-// tiles: [NT, 4] = (request, first token row, rows (<= 64), position of the first row)
-template <int D>
+// tiles: [NT, 4] = (request, first token row, rows (<= 64), position of the first row).
+// A workgroup takes one tile and HPW heads of one kv head and walks the pages the tile can
+// see, PF_NP pages (64 keys) at a time.  Its 256 threads bring a group of pages into LDS
+// together (the next group's loads are in flight in registers meanwhile), and every wave
+// builds its matrix-core operands from LDS: keys and values cross the memory system once per
+// workgroup.  One softmax update (maximum, rescale) serves the whole group of pages, and every
+// key or value operand read from LDS serves all of the wave's column tiles.
+// HPW = 2 (an even number of heads per kv head): wave w works on head w / 2 of the pair and on
+// rows [32 (w % 2), +32) as two column tiles; HPW = 1: wave w works on rows [16 w, +16).
+// Key rows are padded by 16 bytes in LDS, which spreads the 16 keys of an operand read over
+// all banks.
+constexpr int PF_NP = 4;
+
+template <int D, int HPW>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const bf16* __restrict__ qkv, int q_stride, const bf16* __restrict__ k_cache,
     const bf16* __restrict__ v_cache, bf16* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ block_table, int max_blocks, int nh, int nkv, float scale_log2,
     int window) {
+    constexpr int QT = HPW, NP = PF_NP;
+    constexpr int KLD = D + 8;
+    constexpr int KPAGE = PAGE * KLD, VPAGE = D * PAGE;   // elements of a page in LDS
+    constexpr int CHUNKS = 4 * D;                         // 8-byte chunks of a key (or value) page
+    constexpr int CH = (CHUNKS + 255) / 256;
+    __shared__ __attribute__((aligned(16))) bf16 ks[2][NP * KPAGE];
+    __shared__ __attribute__((aligned(16))) bf16 vs[2][NP * VPAGE];
+
     const int* tile = tiles + (size_t)blockIdx.x * 4;
     const int req = tile[0], row0 = tile[1], rows = tile[2], pos0 = tile[3];
-    const int h = blockIdx.y, kvh = h / (nh / nkv);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int q = lane & 15, kg = lane >> 4;
-    const int wrow = wave * 16;
-    if (wrow >= rows) return;
-    const int my = wrow + q;                      // this lane's query row inside the tile
-    const bool valid = my < rows;
-    const int p = pos0 + min(my, rows - 1);
-    const int hi = valid ? p : 0x7fffffff;        // idle columns see everything (never stored)
-    const int lo = (valid && window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-    const int p_min = pos0 + wrow, p_max = pos0 + min(wrow + 15, rows - 1);
-    const int j_lo = (window > 0 && p_min - window + 1 > 0) ? p_min - window + 1 : 0;
+    const int G = nh / nkv;
+    const int h = HPW == 2 ? blockIdx.y * 2 + (wave >> 1) : blockIdx.y;
+    const int wrow = HPW == 2 ? (wave & 1) * 32 : wave * 16;
+    const int kvh = (blockIdx.y * HPW) / G;
+    const bool active = h < nh && wrow < rows;
     const int* table = block_table + (size_t)req * max_blocks;
 
-    bf16x8 bq[D / 32];
-    {
-        const bf16* qrow = qkv + (size_t)(row0 + min(my, rows - 1)) * q_stride + (size_t)h * D + kg * 8;
+    bf16x8 bq[QT][D / 32];
+    int lo[QT], hi[QT];
+    bool valid[QT];
 #pragma unroll
-        for (int i = 0; i < D / 32; ++i) bq[i] = *reinterpret_cast<const bf16x8*>(qrow + i * 32);
+    for (int c = 0; c < QT; ++c) {
+        const int my = wrow + c * 16 + q;                 // this lane's query row inside the tile
+        valid[c] = active && my < rows;
+        const int p = pos0 + min(my, rows - 1);
+        hi[c] = valid[c] ? p : 0x7fffffff;                // idle columns see everything (never stored)
+        lo[c] = (valid[c] && window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+        const bf16* qrow = qkv + (size_t)(row0 + min(my, rows - 1)) * q_stride +
+                           (size_t)min(h, nh - 1) * D + kg * 8;
+#pragma unroll
+        for (int i = 0; i < D / 32; ++i) bq[c][i] = *reinterpret_cast<const bf16x8*>(qrow + i * 32);
     }
-    AttnState<D> st;
-    init_state<D>(st);
-    attend_range<D>(st, bq, k_cache, v_cache, table, j_lo / PAGE, p_max / PAGE + 1, 1, nkv, kvh, lo,
-                    hi, scale_log2, lane);
-    float l = st.l;
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
-    if (!valid) return;
-    const float inv = 1.f / l;
-    bf16* orow = out + ((size_t)(row0 + my) * nh + h) * D + kg * 4;
+    // pages the workgroup walks, and the part of them this wave needs
+    const int t_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+    const int first = t_lo / PAGE, last = (pos0 + rows - 1) / PAGE;
+    const int w_min = pos0 + min(wrow, rows - 1), w_max = pos0 + min(wrow + 16 * QT - 1, rows - 1);
+    const int w_lo = (window > 0 && w_min - window + 1 > 0) ? w_min - window + 1 : 0;
+    const int w_first = w_lo / PAGE, w_last = w_max / PAGE;
+    const int w_lo_max = (window > 0 && w_max - window + 1 > 0) ? w_max - window + 1 : 0;
+
+    AttnState<D, QT> st;
+    init_state<D, QT>(st);
+
+    // a group's pages on their way from global memory to LDS: 32 bytes a thread and page
+    short4v kreg[NP][CH], vreg[NP][CH];
+    auto fetch = [&](int pg0) {
 #pragma unroll
-    for (int tt = 0; tt < D / 16; ++tt) {
-        short4v packed;
+        for (int n = 0; n < NP; ++n) {
+            const int pg = pg0 + n;
+            const bool there = pg <= last;
+            const size_t head = there ? (size_t)table[pg] * nkv + kvh : 0;
+            const bf16* kp = k_cache + head * PAGE * D;
+            const bf16* vp = v_cache + head * D * PAGE;
 #pragma unroll
-        for (int v = 0; v < 4; ++v) packed[v] = bf16_bits(st.o[tt][v] * inv);
-        *reinterpret_cast<short4v*>(orow + tt * 16) = packed;
+            for (int i = 0; i < CH; ++i) {
+                const int c = tid + i * 256;
+                kreg[n][i] = short4v{0, 0, 0, 0};      // pages past the end read as zeros
+                vreg[n][i] = short4v{0, 0, 0, 0};
+                if (there && (CHUNKS % 256 == 0 || c < CHUNKS)) {
+                    kreg[n][i] = *reinterpret_cast<const short4v*>(kp + c * 4);
+                    vreg[n][i] = *reinterpret_cast<const short4v*>(vp + c * 4);
+                }
+            }
+        }
+    };
+    fetch(first);
+
+    for (int pg0 = first, it = 0; pg0 <= last; pg0 += NP, ++it) {
+        const int stage = it & 1;
+#pragma unroll
+        for (int n = 0; n < NP; ++n)
+#pragma unroll
+            for (int i = 0; i < CH; ++i) {
+                const int c = tid + i * 256;
+                if (CHUNKS % 256 == 0 || c < CHUNKS) {
+                    const int key = c / (D / 4), col = (c % (D / 4)) * 4;
+                    *reinterpret_cast<short4v*>(&ks[stage][n * KPAGE + key * KLD + col]) = kreg[n][i];
+                    *reinterpret_cast<short4v*>(&vs[stage][n * VPAGE + c * 4]) = vreg[n][i];
+                }
+            }
+        if (pg0 + NP <= last) fetch(pg0 + NP);
+        __syncthreads();    // also keeps a fast wave from overwriting the stage a slow one reads
+        if (!active || pg0 > w_last || pg0 + NP - 1 < w_first) continue;
+
+        // scores of the group: sc[c][n][v] = S[key 16 (pg0 + n) + 4 kg + v][column q of tile c]
+        floatx4 sc[QT][NP];
+#pragma unroll
+        for (int n = 0; n < NP; ++n)
+#pragma unroll
+            for (int c = 0; c < QT; ++c) sc[c][n] = floatx4{0.f, 0.f, 0.f, 0.f};
+        // i outermost: QT x NP independent accumulators lie between two products into the same one
+#pragma unroll
+        for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+            for (int n = 0; n < NP; ++n) {
+                const bf16x8 ka = *reinterpret_cast<const bf16x8*>(&ks[stage][n * KPAGE + q * KLD + i * 32 + kg * 8]);
+#pragma unroll
+                for (int c = 0; c < QT; ++c)
+                    sc[c][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, bq[c][i], sc[c][n], 0, 0, 0);
+            }
+        // only groups that touch a row's own position (or the window's edge) need the mask
+        const bool masked = (pg0 + NP) * PAGE - 1 > w_min || pg0 * PAGE < w_lo_max;
+        bf16x8 pb[QT][NP / 2];
+        bool rescale = false;
+        float alpha[QT];
+#pragma unroll
+        for (int c = 0; c < QT; ++c) {
+            float mx = -INFINITY;
+            if (masked) {
+#pragma unroll
+                for (int n = 0; n < NP; ++n)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int j = (pg0 + n) * PAGE + kg * 4 + v;
+                        if (j < lo[c] || j > hi[c]) sc[c][n][v] = -INFINITY;
+                    }
+            }
+#pragma unroll
+            for (int n = 0; n < NP; ++n)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) mx = fmaxf(mx, sc[c][n][v]);
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            // maxima are kept as raw scores; p = 2^((s - m) scale_log2), one fma and one v_exp
+            const float m_new = fmaxf(st.m[c], mx);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            alpha[c] = __builtin_amdgcn_exp2f((st.m[c] - m_use) * scale_log2);   // 2^-inf = 0 at the start
+            const float neg = -m_use * scale_log2;
+            float psum = 0.f;
+#pragma unroll
+            for (int n = 0; n < NP; ++n)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float p = __builtin_amdgcn_exp2f(fmaf(sc[c][n][v], scale_log2, neg));
+                    psum += p;
+                    pb[c][n / 2][(n & 1) * 4 + v] = static_cast<bf16>(p);
+                }
+            st.l[c] = st.l[c] * alpha[c] + psum;
+            st.m[c] = m_new;
+            rescale = rescale || alpha[c] != 1.f;
+        }
+        if (__any(rescale)) {
+#pragma unroll
+            for (int c = 0; c < QT; ++c)
+#pragma unroll
+                for (int t = 0; t < D / 16; ++t) st.o[c][t] *= alpha[c];
+        }
+        // two pages per product: lane group kg supplies keys 4 kg .. 4 kg + 3 of both pages
+#pragma unroll
+        for (int n = 0; n < NP; n += 2)
+#pragma unroll
+            for (int t = 0; t < D / 16; ++t) {
+                const short4v v0 = *reinterpret_cast<const short4v*>(&vs[stage][n * VPAGE + (t * 16 + q) * PAGE + kg * 4]);
+                const short4v v1 = *reinterpret_cast<const short4v*>(&vs[stage][(n + 1) * VPAGE + (t * 16 + q) * PAGE + kg * 4]);
+                union { short4v h[2]; bf16x8 full; } va;
+                va.h[0] = v0;
+                va.h[1] = v1;
+#pragma unroll
+                for (int c = 0; c < QT; ++c)
+                    st.o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va.full, pb[c][n / 2], st.o[c][t], 0, 0, 0);
+            }
+    }
+#pragma unroll
+    for (int c = 0; c < QT; ++c) {
+        float l = st.l[c];
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
+        if (!valid[c]) continue;
+        const float inv = 1.f / l;
+        bf16* orow = out + ((size_t)(row0 + wrow + c * 16 + q) * nh + h) * D + kg * 4;
+#pragma unroll
+        for (int tt = 0; tt < D / 16; ++tt) {
+            short4v packed;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) packed[v] = bf16_bits(st.o[c][tt][v] * inv);
+            *reinterpret_cast<short4v*>(orow + tt * 16) = packed;
+        }
     }
 }
 
@@ -306,8 +469,12 @@ template <int D>
 static int launch_prefill(const bf16* qkv, int q_stride, const bf16* k, const bf16* v, bf16* out,
                           const int* tiles, const int* table, int max_blocks, int NT, int nh,
                           int nkv, float scale_log2, int window, hipStream_t s) {
-    attn_prefill_kernel<D><<<dim3(NT, nh), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
-                                                        max_blocks, nh, nkv, scale_log2, window);
+    if ((nh / nkv) % 2 == 0)
+        attn_prefill_kernel<D, 2><<<dim3(NT, nh / 2), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
+                                                                   max_blocks, nh, nkv, scale_log2, window);
+    else
+        attn_prefill_kernel<D, 1><<<dim3(NT, nh), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
+                                                               max_blocks, nh, nkv, scale_log2, window);
     LC_LAUNCH_CHECK("attn_prefill");
     return 0;
 }
