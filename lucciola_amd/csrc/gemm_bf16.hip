@@ -25,12 +25,15 @@ template <typename TO> __device__ __forceinline__ void store_out(TO* p, float v)
 template <> __device__ __forceinline__ void store_out<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void store_out<bf16>(bf16* p, float v) { *p = static_cast<bf16>(v); }
 
+// silu(g) * u with silu(g) = g / (1 + exp(-g))   (reference: src/kernels/swiglu.cu:8,31-35)
+__device__ __forceinline__ float swiglu_f(float g, float u) { return g / (1.f + expf(-g)) * u; }
+
 // ------------------------------------------------------------------------------- skinny
 constexpr int SK_KBLOCK = 128; // k elements per wave iteration
 
 // MT: tiles of 16 rows of x; NT: tiles of 16 rows of w per workgroup; the WAVES waves of a
 // workgroup take the k blocks in turn.
-template <int MT, int NT, int WAVES, int UNROLL, typename TO>
+template <int MT, int NT, int WAVES, int UNROLL, int EPI, typename TO>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __restrict__ x,
                                                                  const bf16* __restrict__ w,
                                                                  TO* __restrict__ out, int M, int N,
@@ -82,14 +85,32 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
             for (int v = 0; v < 4; ++v)
                 red[((wave * NT + nt) * MT + mt) * 256 + v * 64 + lane] = acc[nt][mt][v];
     __syncthreads();
-    for (int idx = threadIdx.x; idx < NT * MT * 256; idx += WAVES * 64) {
-        float total = 0.f;
+    if (EPI == 0) {
+        for (int idx = threadIdx.x; idx < NT * MT * 256; idx += WAVES * 64) {
+            float total = 0.f;
 #pragma unroll
-        for (int wv = 0; wv < WAVES; ++wv) total += red[wv * NT * MT * 256 + idx];
-        const int tile = idx >> 8, v = (idx >> 6) & 3, l = idx & 63;
-        const int nt = tile / MT, mt = tile % MT;
-        const int m = mt * 16 + (l & 15), n = n0 + nt * 16 + (l >> 4) * 4 + v;
-        if (m < M && n < N) store_out<TO>(out + (size_t)m * N + n, total);
+            for (int wv = 0; wv < WAVES; ++wv) total += red[wv * NT * MT * 256 + idx];
+            const int tile = idx >> 8, v = (idx >> 6) & 3, l = idx & 63;
+            const int nt = tile / MT, mt = tile % MT;
+            const int m = mt * 16 + (l & 15), n = n0 + nt * 16 + (l >> 4) * 4 + v;
+            if (m < M && n < N) store_out<TO>(out + (size_t)m * N + n, total);
+        }
+    } else {
+        // rows of w come in blocks of 16: 8 gate rows, then their 8 up rows; out has N / 2 columns
+        for (int idx = threadIdx.x; idx < NT * MT * 128; idx += WAVES * 64) {
+            const int tile = idx >> 7, v = (idx >> 5) & 3, l = idx & 31;   // l: lane of the gate half
+            const int gi = tile * 256 + v * 64 + l, ui = gi + 32;
+            float g = 0.f, u = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < WAVES; ++wv) {
+                g += red[wv * NT * MT * 256 + gi];
+                u += red[wv * NT * MT * 256 + ui];
+            }
+            const int nt = tile / MT, mt = tile % MT;
+            const int m = mt * 16 + (l & 15), n = n0 + nt * 16 + (l >> 4) * 4 + v;   // gate row, n % 16 < 8
+            const int col = (n >> 4) * 8 + (n & 7);
+            if (m < M && n < N) store_out<TO>(out + (size_t)m * (N / 2) + col, swiglu_f(g, u));
+        }
     }
 }
 
@@ -97,7 +118,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 constexpr int TB_M = 128, TB_N = 128, TB_K = 64;
 constexpr int TB_LD = TB_K + 8;   // padded row length in LDS (144 bytes)
 
-template <typename TO>
+template <int EPI, typename TO>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ x,
                                                          const bf16* __restrict__ w,
                                                          TO* __restrict__ out, int M, int N, int K,
@@ -188,30 +209,38 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int m = m0 + wm + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
-                if (m < M && n < N) store_out<TO>(out + (size_t)m * N + n, acc[i][j][v]);
+                if (EPI == 0) {
+                    if (m < M && n < N) store_out<TO>(out + (size_t)m * N + n, acc[i][j][v]);
+                } else {
+                    // columns come in blocks of 16: 8 gate, then their 8 up (8 lanes further on)
+                    const float other = __shfl_xor(acc[i][j][v], 8, 64);
+                    if ((lr & 8) == 0 && m < M && n < N)
+                        store_out<TO>(out + (size_t)m * (N / 2) + (n >> 4) * 8 + (n & 7),
+                                      swiglu_f(acc[i][j][v], other));
+                }
             }
         }
 }
 
-template <int MT, int NT, int WAVES, int UNROLL, typename TO>
+template <int MT, int NT, int WAVES, int UNROLL, int EPI, typename TO>
 static void launch_skinny(const bf16* x, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
     const int rows = 16 * NT;
-    gemm_skinny_kernel<MT, NT, WAVES, UNROLL, TO><<<(N + rows - 1) / rows, WAVES * 64, 0, s>>>(x, w, out, M, N, K);
+    gemm_skinny_kernel<MT, NT, WAVES, UNROLL, EPI, TO><<<(N + rows - 1) / rows, WAVES * 64, 0, s>>>(x, w, out, M, N, K);
 }
 
-template <typename TO>
+template <int EPI, typename TO>
 static int launch_bf16(const bf16* x, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
     if (M <= 64) {
         switch ((M + 15) / 16) {
-            case 1: launch_skinny<1, 1, 16, 2, TO>(x, w, out, M, N, K, s); break;
-            case 2: launch_skinny<2, 1, 16, 1, TO>(x, w, out, M, N, K, s); break;
-            case 3: launch_skinny<3, 2, 8, 1, TO>(x, w, out, M, N, K, s); break;
-            default: launch_skinny<4, 2, 8, 1, TO>(x, w, out, M, N, K, s); break;
+            case 1: launch_skinny<1, 1, 16, 2, EPI, TO>(x, w, out, M, N, K, s); break;
+            case 2: launch_skinny<2, 1, 16, 1, EPI, TO>(x, w, out, M, N, K, s); break;
+            case 3: launch_skinny<3, 2, 8, 1, EPI, TO>(x, w, out, M, N, K, s); break;
+            default: launch_skinny<4, 2, 8, 1, EPI, TO>(x, w, out, M, N, K, s); break;
         }
         LC_LAUNCH_CHECK("gemm_skinny");
     } else {
         const int tiles_m = (M + TB_M - 1) / TB_M, tiles_n = (N + TB_N - 1) / TB_N;
-        gemm_tiled_kernel<TO><<<tiles_m * tiles_n, 256, 0, s>>>(x, w, out, M, N, K, tiles_m, tiles_n);
+        gemm_tiled_kernel<EPI, TO><<<tiles_m * tiles_n, 256, 0, s>>>(x, w, out, M, N, K, tiles_m, tiles_n);
         LC_LAUNCH_CHECK("gemm_tiled");
     }
     return 0;
@@ -229,14 +258,24 @@ LC_API int lc_gemm_bf16_supported(int M, int N, int K) {
     return 1;
 }
 
+// epilogue 0: out[M, N] = x . w^T.  epilogue 1 (SwiGLU): the rows of w come in blocks of 16,
+// 8 gate rows followed by their 8 up rows; out[M, N / 2] = silu(gate) * up.
 LC_API int lc_gemm_bf16(const void* x, const void* w, void* out, int out_dt, int M, int N, int K,
-                        hipStream_t stream) {
+                        int epilogue, hipStream_t stream) {
     LC_CHECK(lc_gemm_bf16_supported(M, N, K), "gemm_bf16: sizes M=%d N=%d K=%d are not supported "
              "(K must be a multiple of %d)", M, N, K, SK_KBLOCK);
     LC_CHECK(x && w && out, "gemm_bf16: null pointer");
     LC_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_bf16: operands must be 16-byte aligned");
-    if (out_dt == DT_BF16) return launch_bf16<bf16>((const bf16*)x, (const bf16*)w, (bf16*)out, M, N, K, stream);
-    if (out_dt == DT_F32) return launch_bf16<float>((const bf16*)x, (const bf16*)w, (float*)out, M, N, K, stream);
+    LC_CHECK(epilogue == 0 || (epilogue == 1 && N % 16 == 0),
+             "gemm_bf16: the SwiGLU epilogue needs N (%d) to be a multiple of 16", N);
+    const bf16* xb = (const bf16*)x;
+    const bf16* wb = (const bf16*)w;
+    if (out_dt == DT_BF16)
+        return epilogue ? launch_bf16<1, bf16>(xb, wb, (bf16*)out, M, N, K, stream)
+                        : launch_bf16<0, bf16>(xb, wb, (bf16*)out, M, N, K, stream);
+    if (out_dt == DT_F32)
+        return epilogue ? launch_bf16<1, float>(xb, wb, (float*)out, M, N, K, stream)
+                        : launch_bf16<0, float>(xb, wb, (float*)out, M, N, K, stream);
     LC_CHECK(false, "gemm_bf16: unknown output dtype %d", out_dt);
     return 0;
 }

@@ -26,7 +26,7 @@ _SIGNATURES = {
     "lc_rmsnorm": "ppppfpiiiip",
     "lc_rmsnorm_act": "ppfpiiip",
     "lc_gemm_generic": "pipipiiiip",
-    "lc_gemm_bf16": "pppiiiip",
+    "lc_gemm_bf16": "pppiiiiip",
     "lc_gemm_bf16_supported": "iii",
     "lc_qk_norm_rope_write": "piiiiippfppipppip",
     "lc_attention_generic": "pipppipppiiiiiifip",
@@ -177,10 +177,37 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = No
         return out
     if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and _fast_gemm_ok(M, N, K)):
         _call("lc_gemm_bf16", _ptr(x), _ptr(w), _ptr(out), _c_int(_dt(out)), _c_int(M), _c_int(N),
-              _c_int(K), _stream())
+              _c_int(K), 0, _stream())
     else:
         _call("lc_gemm_generic", _ptr(x), _c_int(_dt(x)), _ptr(w), _c_int(_dt(w)), _ptr(out),
               _c_int(_dt(out)), _c_int(M), _c_int(N), _c_int(K), _stream())
+    return out
+
+
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """Stack gate and up weights [I, H] as blocks of 8 gate rows followed by their 8 up rows
+    (the layout ``gemm_swiglu`` wants); I must be a multiple of 8."""
+    I, H = gate.shape
+    return torch.stack([gate.view(I // 8, 8, H), up.view(I // 8, 8, H)], dim=1).reshape(2 * I, H).contiguous()
+
+
+def gemm_swiglu_supported(x_dtype, w: torch.Tensor, K: int) -> bool:
+    return (x_dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.shape[0] % 16 == 0
+            and _fast_gemm_ok(64, w.shape[0], K))
+
+
+def gemm_swiglu(x: torch.Tensor, w_interleaved: torch.Tensor) -> torch.Tensor:
+    """``silu(x . gate^T) * (x . up^T)`` in one kernel, with gate and up interleaved by
+    :func:`interleave_gate_up`; bfloat16 only.  [M, K] x [2 I, K] -> [M, I]."""
+    _need(x, "gemm_swiglu x", torch.bfloat16, 2)
+    _need(w_interleaved, "gemm_swiglu w", torch.bfloat16, 2)
+    M, K = x.shape
+    N, K2 = w_interleaved.shape
+    if K != K2 or N % 16:
+        raise KernelError(f"gemm_swiglu: x is [{M}, {K}], w is [{N}, {K2}] (rows must come in 16s)")
+    out = torch.empty((M, N // 2), dtype=torch.bfloat16, device=x.device)
+    if M:
+        _call("lc_gemm_bf16", _ptr(x), _ptr(w_interleaved), _ptr(out), DT_BF16, M, N, K, 1, _stream())
     return out
 
 

@@ -38,11 +38,21 @@ class GatedMLP(Part):
                 "down_proj": ParamDecl((self.H, self.I))}
 
     def bind(self, tensors, ctx: BuildContext) -> None:
-        self.gate_up = stack_rows([tensors["gate_proj"], tensors["up_proj"]])
+        gate, up = tensors["gate_proj"], tensors["up_proj"]
         self.down = tensors["down_proj"]
         self.dtype = ctx.dtype
+        # where the matrix-core kernel takes the sizes, gate and up rows are interleaved so that
+        # silu(gate) * up is formed in the product's epilogue and [T, 2 I] never reaches memory
+        self.fused = (ctx.device.type == "cuda" and self.I % 8 == 0 and gate.dtype == up.dtype
+                      and ops.gemm_swiglu_supported(ctx.dtype, gate.new_empty((2 * self.I, 1)), self.H))
+        if self.fused:
+            self.gate_up = ops.interleave_gate_up(gate, up)
+        else:
+            self.gate_up = stack_rows([gate, up])
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        gu = ops.gemm(x, self.gate_up, self.dtype)
-        z = ops.swiglu(gu)
+        if self.fused:
+            z = ops.gemm_swiglu(x, self.gate_up)
+        else:
+            z = ops.swiglu(ops.gemm(x, self.gate_up, self.dtype))
         return ops.gemm(z, self.down, self.dtype)

@@ -276,3 +276,19 @@ def test_attention_bf16_long_contexts(nh, nkv, d, window):
                                                    batch.block_table.cpu()),
                          kc.cpu(), vc.cpu(), nh, nkv, d, 16, d ** -0.5, window)
     close(got, want, torch.bfloat16, atol=attention_atol(torch.bfloat16, vc))
+
+
+@pytest.mark.parametrize("M,I,K", [(1, 16, 128), (8, 200, 256), (33, 1000, 128), (64, 96, 384), (65, 136, 256),
+                                   (300, 520, 128), (2048, 256, 256)])
+def test_gemm_with_swiglu_epilogue(M, I, K):
+    """gate and up interleaved in blocks of 8 rows, silu(gate) * up formed in the epilogue."""
+    x = rnd(M, K, dtype=torch.bfloat16, seed=80, scale=0.5)
+    gate = rnd(I, K, dtype=torch.bfloat16, seed=81, scale=0.2)
+    up = rnd(I, K, dtype=torch.bfloat16, seed=82, scale=0.2)
+    w = ops.interleave_gate_up(gate, up)
+    assert torch.equal(w[:8], gate[:8]) and torch.equal(w[8:16], up[:8]) and torch.equal(w[16:24], gate[8:16])
+    assert ops.gemm_swiglu_supported(torch.bfloat16, w, K)
+    got = ops.gemm_swiglu(x, w)
+    g, u = x.double() @ gate.double().T, x.double() @ up.double().T
+    want = (g / (1 + torch.exp(-g)) * u).to(torch.bfloat16)
+    close(got, want, torch.bfloat16, scale=0.5)
