@@ -270,3 +270,27 @@ def test_command_line_and_async_engine(tmp_path):
     finally:
         engine.stop()
     assert [got[0], got[1]] == want
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layers_of_the_8b_size(dtype):
+    """Two layers with the sizes of the Qwen3-8B-shaped configuration (hidden 4096, 32 query and
+    8 kv heads of 128, feed-forward 12288; the vocabulary is cut to 2048 to keep the plain
+    float64 run short): the kernels chosen for real sizes (matrix-core products, vector norms,
+    matrix-core attention in bfloat16; FMA kernels in float32) against the plain implementation,
+    whole, in portions and token by token."""
+    cfg = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 4096,
+           "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+           "intermediate_size": 12288, "vocab_size": 2048, "rope_theta": 1000000.0,
+           "rms_norm_eps": 1e-6, "tie_word_embeddings": False, "max_position_embeddings": 40960,
+           "initializer_range": 0.02}
+    weights = random_weights(cfg, 11)
+    prompts = prompts_for(cfg, [150, 37], 12)
+    refs = {n: plain_qwen3.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    for family in (traces.whole, lambda p: traces.chunked(p, sizes=(70, 2, 33, 5)),
+                   lambda p: traces.tail_decode(p, tail=8)):
+        steps = family(prompts)
+        runner = make_runner(cfg, weights, 16, traces.max_live_tokens(steps, 16) // 16, dtype, DEV)
+        got = replay(runner, steps)
+        worst = compare(got, cfg, weights, prompts, TOL[dtype], refs)
+        print(f"8B-size layers {dtype}: worst relative error {worst:.3e}")
