@@ -292,3 +292,28 @@ def test_gemm_with_swiglu_epilogue(M, I, K):
     g, u = x.double() @ gate.double().T, x.double() @ up.double().T
     want = (g / (1 + torch.exp(-g)) * u).to(torch.bfloat16)
     close(got, want, torch.bfloat16, scale=0.5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("d,page,new", [(32, 16, 1), (32, 16, 40), (48, 8, 1), (64, 16, 70)])
+def test_attention_window_edge(dtype, d, page, new):
+    """The key just outside the window gets a huge score and a value of its own: if the window
+    were one position too wide the output would be that value.  The key just inside gets the
+    same treatment and must win."""
+    nh, nkv, window, length = 2, 1, 37, 200
+    for inside in (False, True):
+        qkv, batch, kc, vc = paged_case([length], [new], nh, nkv, d, page, dtype, seed=90)
+        table = batch.block_table[0].tolist()
+        qkv.zero_()
+        q = qkv.view(new, nh + 2 * nkv, d)
+        q[:, :nh, 5] = 30.0
+        p_last = length - 1                              # the last query's position
+        j = p_last - window + (1 if inside else 0)       # first visible key is p - window + 1
+        kc[table[j // page], 0, j % page, :] = 0
+        kc[table[j // page], 0, j % page, 5] = 30.0
+        vc[table[j // page], 0, :, j % page] = 7.0
+        got = ops.attention(qkv, batch, kc, vc, nh, nkv, d, page, d ** -0.5, window)[-1].float()
+        if inside:
+            assert float((got - 7.0).abs().max()) < 0.1
+        else:
+            assert float(got.abs().max()) < 5.0          # a mix of ordinary values, not the marked one

@@ -308,3 +308,33 @@ def test_toy_architecture_with_a_stateful_mixer():
         MIXERS.unregister("toy_decay")
         FEED_FORWARDS.unregister("toy_scale")
         ARCHITECTURES.unregister("ToyForCausalLM")
+
+
+def test_block_arrangement_alone():
+    """The pre-norm residual arrangement with stand-in parts: h1 = h + mixer(norm1(h)),
+    h2 = h1 + ff(norm2(h1)); the second branch's output is still pending when the block ends."""
+    from lucciola_amd.config.registry import BLOCKS
+
+    class Scale:
+        def __init__(self, factor):
+            self.factor = factor
+
+        def forward(self, x, site=None):
+            return (x.float() * self.factor).to(x.dtype)
+
+    ctx = BuildContext(torch.float32, DEV)
+    n1 = build_part(NORMS, PartSpec("rms", {"size": 40, "eps": 1e-6}))
+    n2 = build_part(NORMS, PartSpec("rms", {"size": 40, "eps": 1e-6}))
+    w1, w2 = 1 + rnd(40, seed=1, scale=0.1), 1 + rnd(40, seed=2, scale=0.1)
+    n1.bind({"weight": w1}, ctx)
+    n2.bind({"weight": w2}, ctx)
+    block = BLOCKS.get("prenorm_residual")(Scale(2.0), Scale(-0.5), n1, n2)
+    h = rnd(6, 40, seed=3)
+    stream = ResidualStream(h.clone())
+    stream.pending = rnd(6, 40, seed=4)               # the previous block's last branch
+    h0 = h.double().cpu() + stream.pending.double().cpu()
+    block.forward(stream, None)
+    h1 = h0 + 2.0 * plain.rmsnorm(h0, w1.cpu(), 1e-6)
+    pending = -0.5 * plain.rmsnorm(h1, w2.cpu(), 1e-6)
+    torch.testing.assert_close(stream.h.double().cpu(), h1, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(stream.pending.double().cpu(), pending, rtol=1e-5, atol=1e-5)
