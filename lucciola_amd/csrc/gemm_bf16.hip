@@ -6,10 +6,10 @@
 //    rows straight from global memory into v_mfma_f32_16x16x32_bf16 operands (w is the A
 //    operand, x^T the B operand); the waves' partial sums meet in LDS.  No split-K workspace,
 //    no atomics: the order of the sums is fixed.
-//  * tiled (M > 64, prefill): 128x128x64 workgroup tiles in LDS (rows padded to 144 bytes so
-//    that operand reads are conflict free), 4 waves of 64x64 built from
-//    v_mfma_f32_32x32x16_bf16, next tile prefetched into registers while the current one is
-//    multiplied.  Workgroups are renumbered so that each XCD's L2 sees neighbouring tiles.
+//  * tiled (M > 64, prefill): 128x128x64 or 256x256x64 workgroup tiles that go from global
+//    memory straight into a ring of LDS stages, 4 waves built from v_mfma_f32_32x32x16_bf16 with
+//    hand-pipelined operand reads.  Workgroups are renumbered so that each XCD's L2 sees
+//    neighbouring tiles.
 //
 // The reference's linear kernel computes the same product with one thread per output element
 // and no matrix instruction (src/kernels/linear.cu:7-56).
@@ -115,16 +115,40 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 }
 
 // ------------------------------------------------------------------------------- tiled
-constexpr int TB_M = 128, TB_N = 128, TB_K = 64;
-constexpr int TB_LD = TB_K + 8;   // padded row length in LDS (144 bytes)
+// Workgroup tile BM x BN x 64, four waves in a 2 x 2 grid, each owning (BM/64) x (BN/64) tiles
+// of 32 x 32.  128 x 128 (two workgroups to a CU) for most shapes, 256 x 256 where the grid
+// still has two tiles per CU: it halves the bytes that cross the L2 per product.
+//
+// Operand tiles go from global memory straight into LDS (global_load_lds_dwordx4: lane l's 16
+// bytes land at the instruction's LDS base + 16 l, no registers in between) into a ring of
+// TL_STAGES stages; a stage is filled while the one before it is multiplied.  Inside a stage
+// a row's eight 16-byte chunks are stored at column (chunk ^ (row & 7)), which spreads the 32
+// rows of an operand read over all banks without padding.  The LDS reads are written by hand
+// (ds_read_b128 + explicit waits), two k-steps deep, for two reasons: the products of one
+// k-step then hide the reads of the next although a SIMD may hold a single wave, and the
+// compiler, which cannot tell the stages apart, would otherwise make every load in flight
+// land before any read.  Likewise the barrier is the bare instruction: each wave first waits
+// for its own loads of the stage, the barrier then makes all waves' loads visible.
+constexpr int TL_K = 64, TL_STAGES = 2;
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef __attribute__((address_space(1))) const void* glb_ptr_t;
 
-template <int EPI, typename TO>
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));   // other counters untouched
+}
+template <int N> __device__ __forceinline__ void wait_lgkmcnt() {
+    __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));
+}
+
+template <int BM, int BN, int EPI, typename TO>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ x,
                                                          const bf16* __restrict__ w,
                                                          TO* __restrict__ out, int M, int N, int K,
                                                          int tiles_m, int tiles_n) {
-    __shared__ __attribute__((aligned(16))) bf16 As[TB_M * TB_LD];
-    __shared__ __attribute__((aligned(16))) bf16 Bs[TB_N * TB_LD];
+    constexpr int TM = BM / 64, TN = BN / 64;
+    constexpr int LPA = BM * 8 / 256, LPB = BN * 8 / 256;   // load instructions per thread and stage
+    __shared__ __attribute__((aligned(16))) bf16 As[TL_STAGES][BM * TL_K];
+    __shared__ __attribute__((aligned(16))) bf16 Bs[TL_STAGES][BN * TL_K];
 
     // renumber: workgroups go round-robin over 8 XCDs; give each XCD a contiguous run of
     // tiles, m fastest, so that one XCD's L2 keeps the w tile that its workgroups share
@@ -136,75 +160,102 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
         id = xcd * q + min(xcd, rem) + local;   // a bijection of [0, total) for any total
     }
     const int tm = id % tiles_m, tn = id / tiles_m;
-    const int m0 = tm * TB_M, n0 = tn * TB_N;
+    const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
-    const int lr = lane & 31, lk = (lane >> 5) * 8;
+    const int wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
+    const int lr = lane & 31, kg = lane >> 5;
 
-    // global -> register staging: 4 chunks of 16 bytes per thread and operand
-    const bf16* xg[4];
-    const bf16* wg[4];
-    int soff[4];
+    // chunk p = (i * 4 + wave) * 64 + lane of a stage holds row p / 8, global column (p % 8) ^ (row & 7)
+    const bf16* xg[LPA];
+    const bf16* wg[LPB];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int c = tid + i * 256;
-        const int row = c >> 3, col = (c & 7) * 8;
-        xg[i] = x + (size_t)min(m0 + row, M - 1) * K + col;
-        wg[i] = w + (size_t)min(n0 + row, N - 1) * K + col;
-        soff[i] = row * TB_LD + col;
+    for (int i = 0; i < LPA; ++i) {
+        const int p = (i * 4 + wave) * 64 + lane, row = p >> 3, kc = (p & 7) ^ (row & 7);
+        xg[i] = x + (size_t)min(m0 + row, M - 1) * K + kc * 8;
     }
-    bf16x8 ra[4], rb[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        ra[i] = *reinterpret_cast<const bf16x8*>(xg[i]);
-        rb[i] = *reinterpret_cast<const bf16x8*>(wg[i]);
+    for (int i = 0; i < LPB; ++i) {
+        const int p = (i * 4 + wave) * 64 + lane, row = p >> 3, kc = (p & 7) ^ (row & 7);
+        wg[i] = w + (size_t)min(n0 + row, N - 1) * K + kc * 8;
     }
+    auto issue = [&](int kb, int stage) {
+#pragma unroll
+        for (int i = 0; i < LPA; ++i)
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(xg[i] + kb * TL_K),
+                                             (lds_ptr_t)(&As[stage][(i * 4 + wave) * 512]), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < LPB; ++i)
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(wg[i] + kb * TL_K),
+                                             (lds_ptr_t)(&Bs[stage][(i * 4 + wave) * 512]), 16, 0, 0);
+    };
+    const int nk = K / TL_K;
+#pragma unroll
+    for (int s = 0; s < TL_STAGES - 1; ++s)
+        if (s < nk) issue(s, s);
 
-    floatx16 acc[2][2];
+    floatx16 acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    for (int k0 = 0; k0 < K; k0 += TB_K) {
+    // byte offsets of this lane's operand rows inside a stage, and their swizzles
+    unsigned arow[TM], brow[TN];
+    int asw[TM], bsw[TN];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<bf16x8*>(As + soff[i]) = ra[i];
-            *reinterpret_cast<bf16x8*>(Bs + soff[i]) = rb[i];
-        }
-        __syncthreads();
-        if (k0 + TB_K < K) {
+    for (int i = 0; i < TM; ++i) { const int row = wm + i * 32 + lr; arow[i] = row * 128; asw[i] = row & 7; }
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                ra[i] = *reinterpret_cast<const bf16x8*>(xg[i] + k0 + TB_K);
-                rb[i] = *reinterpret_cast<const bf16x8*>(wg[i] + k0 + TB_K);
+    for (int j = 0; j < TN; ++j) { const int row = wn + j * 32 + lr; brow[j] = row * 128; bsw[j] = row & 7; }
+
+    for (int it = 0; it < nk; ++it) {
+        // block `it` has landed when at most the younger blocks' loads are still in flight
+        if (it + TL_STAGES - 2 < nk) wait_vmcnt<(TL_STAGES - 2) * (LPA + LPB)>(); else wait_vmcnt<0>();
+        __builtin_amdgcn_s_barrier();
+        if (it + TL_STAGES - 1 < nk) issue(it + TL_STAGES - 1, (it + TL_STAGES - 1) % TL_STAGES);
+        const unsigned abase = (unsigned)(uintptr_t)(lds_ptr_t)As[it % TL_STAGES];
+        const unsigned bbase = (unsigned)(uintptr_t)(lds_ptr_t)Bs[it % TL_STAGES];
+        bf16x8 a[2][TM], b[2][TN];
+        auto read = [&](int ks, int buf) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const unsigned addr = abase + arow[i] + (((ks * 2 + kg) ^ asw[i]) * 16);
+                asm volatile("ds_read_b128 %0, %1" : "=v"(a[buf][i]) : "v"(addr));
             }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const unsigned addr = bbase + brow[j] + (((ks * 2 + kg) ^ bsw[j]) * 16);
+                asm volatile("ds_read_b128 %0, %1" : "=v"(b[buf][j]) : "v"(addr));
+            }
+        };
+        read(0, 0);
+#pragma unroll
+        for (int ks = 0; ks < TL_K / 16; ++ks) {
+            if (ks + 1 < TL_K / 16) {
+                read(ks + 1, (ks + 1) & 1);
+                wait_lgkmcnt<TM + TN>();       // this k-step's operands are in; the next one's may be out
+            } else {
+                wait_lgkmcnt<0>();
+            }
+            // the products below must not be moved above the wait: tie their operands to this point
+#pragma unroll
+            for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(a[ks & 1][i]));
+#pragma unroll
+            for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(b[ks & 1][j]));
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks & 1][i], b[ks & 1][j], acc[i][j], 0, 0, 0);
         }
-#pragma unroll
-        for (int ks = 0; ks < TB_K; ks += 16) {
-            bf16x8 a[2], b[2];
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-                a[i] = *reinterpret_cast<const bf16x8*>(As + (wm + i * 32 + lr) * TB_LD + ks + lk);
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-                b[j] = *reinterpret_cast<const bf16x8*>(Bs + (wn + j * 32 + lr) * TB_LD + ks + lk);
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
-        }
-        __syncthreads();
     }
     // acc[i][j][v]: row m = (v/4)*8 + (lane/32)*4 + v%4, column n = lane%32 of the 32x32 tile
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < TN; ++j) {
             const int n = n0 + wn + j * 32 + lr;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
@@ -239,8 +290,13 @@ static int launch_bf16(const bf16* x, const bf16* w, TO* out, int M, int N, int 
         }
         LC_LAUNCH_CHECK("gemm_skinny");
     } else {
-        const int tiles_m = (M + TB_M - 1) / TB_M, tiles_n = (N + TB_N - 1) / TB_N;
-        gemm_tiled_kernel<EPI, TO><<<tiles_m * tiles_n, 256, 0, s>>>(x, w, out, M, N, K, tiles_m, tiles_n);
+        const int big_m = (M + 255) / 256, big_n = (N + 255) / 256;
+        if ((long long)big_m * big_n >= 512) {
+            gemm_tiled_kernel<256, 256, EPI, TO><<<big_m * big_n, 256, 0, s>>>(x, w, out, M, N, K, big_m, big_n);
+        } else {
+            const int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
+            gemm_tiled_kernel<128, 128, EPI, TO><<<tiles_m * tiles_n, 256, 0, s>>>(x, w, out, M, N, K, tiles_m, tiles_n);
+        }
         LC_LAUNCH_CHECK("gemm_tiled");
     }
     return 0;
@@ -254,7 +310,7 @@ using namespace lc;
 LC_API int lc_gemm_bf16_supported(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     if (K % SK_KBLOCK != 0) return 0;
-    if ((size_t)((M + TB_M - 1) / TB_M) * ((N + TB_N - 1) / TB_N) > 0x7fffffffu) return 0;
+    if ((size_t)((M + 127) / 128) * ((N + 127) / 128) > 0x7fffffffu) return 0;
     return 1;
 }
 
