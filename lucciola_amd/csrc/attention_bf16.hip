@@ -257,7 +257,7 @@ __global__ __launch_bounds__(128) void attn_decode_join_kernel(const float* __re
 // rows [32 (w % 2), +32) as two column tiles; HPW = 1: wave w works on rows [16 w, +16).
 // Key rows are padded by 16 bytes in LDS, which spreads the 16 keys of an operand read over
 // all banks.
-constexpr int PF_NP = 4;
+constexpr int PF_NP = 2;
 
 template <int D, int HPW>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(
