@@ -1,12 +1,13 @@
 // bfloat16 matrix products on the matrix cores: out[M, N] = x[M, K] . w[N, K]^T, float32
 // accumulation, output bfloat16 or float32.  Two kernels:
 //
-//  * skinny (M <= 64, decode): bound by reading w once from HBM.  A workgroup owns 16 rows of
+//  * skinny (M <= 16, decode): bound by reading w once from HBM.  A workgroup owns 16 rows of
 //    w; its waves split K in interleaved blocks of 128, each wave streaming its part of the
 //    rows straight from global memory into v_mfma_f32_16x16x32_bf16 operands (w is the A
 //    operand, x^T the B operand); the waves' partial sums meet in LDS.  No split-K workspace,
 //    no atomics: the order of the sums is fixed.
-//  * tiled (M > 64, prefill): 128x128x64 or 256x256x64 workgroup tiles that go from global
+//  * tiled (M > 16): 128x128x64 or 256x256x64 workgroup tiles (64x128x64 with K cut into shares
+//    and a reduction kernel for 16 < M <= 64, where whole-K tiles would leave CUs idle) that go from global
 //    memory straight into a ring of LDS stages, 4 waves built from v_mfma_f32_32x32x16_bf16 with
 //    hand-pipelined operand reads.  Workgroups are renumbered so that each XCD's L2 sees
 //    neighbouring tiles.
@@ -129,7 +130,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 // compiler, which cannot tell the stages apart, would otherwise make every load in flight
 // land before any read.  Likewise the barrier is the bare instruction: each wave first waits
 // for its own loads of the stage, the barrier then makes all waves' loads visible.
-constexpr int TL_K = 64, TL_STAGES = 2;
+constexpr int TL_K = 64;
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef __attribute__((address_space(1))) const void* glb_ptr_t;
 
@@ -140,11 +141,13 @@ template <int N> __device__ __forceinline__ void wait_lgkmcnt() {
     __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));
 }
 
-template <int BM, int BN, int EPI, typename TO>
+// SPLIT: blockIdx.y owns a share of the k-blocks and writes its float32 partial sums to
+// part[blockIdx.y][M][N]; splitk_reduce_kernel adds the shares in a fixed order.
+template <int BM, int BN, int TL_STAGES, int EPI, bool SPLIT, typename TO>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ x,
                                                          const bf16* __restrict__ w,
-                                                         TO* __restrict__ out, int M, int N, int K,
-                                                         int tiles_m, int tiles_n) {
+                                                         TO* __restrict__ out, float* __restrict__ part,
+                                                         int M, int N, int K, int tiles_m, int tiles_n) {
     constexpr int TM = BM / 64, TN = BN / 64;
     constexpr int LPA = BM * 8 / 256, LPB = BN * 8 / 256;   // load instructions per thread and stage
     __shared__ __attribute__((aligned(16))) bf16 As[TL_STAGES][BM * TL_K];
@@ -189,10 +192,12 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
             __builtin_amdgcn_global_load_lds((glb_ptr_t)(wg[i] + kb * TL_K),
                                              (lds_ptr_t)(&Bs[stage][(i * 4 + wave) * 512]), 16, 0, 0);
     };
-    const int nk = K / TL_K;
+    const int nk_all = K / TL_K;
+    const int kb0 = SPLIT ? (int)((long long)blockIdx.y * nk_all / gridDim.y) : 0;
+    const int nk = (SPLIT ? (int)((long long)(blockIdx.y + 1) * nk_all / gridDim.y) : nk_all) - kb0;
 #pragma unroll
     for (int s = 0; s < TL_STAGES - 1; ++s)
-        if (s < nk) issue(s, s);
+        if (s < nk) issue(kb0 + s, s);
 
     floatx16 acc[TM][TN];
 #pragma unroll
@@ -214,7 +219,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
         // block `it` has landed when at most the younger blocks' loads are still in flight
         if (it + TL_STAGES - 2 < nk) wait_vmcnt<(TL_STAGES - 2) * (LPA + LPB)>(); else wait_vmcnt<0>();
         __builtin_amdgcn_s_barrier();
-        if (it + TL_STAGES - 1 < nk) issue(it + TL_STAGES - 1, (it + TL_STAGES - 1) % TL_STAGES);
+        if (it + TL_STAGES - 1 < nk) issue(kb0 + it + TL_STAGES - 1, (it + TL_STAGES - 1) % TL_STAGES);
         const unsigned abase = (unsigned)(uintptr_t)(lds_ptr_t)As[it % TL_STAGES];
         const unsigned bbase = (unsigned)(uintptr_t)(lds_ptr_t)Bs[it % TL_STAGES];
         bf16x8 a[2][TM], b[2][TN];
@@ -260,7 +265,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int m = m0 + wm + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
-                if (EPI == 0) {
+                if (SPLIT) {
+                    if (m < M && n < N) part[((size_t)blockIdx.y * M + m) * N + n] = acc[i][j][v];
+                } else if (EPI == 0) {
                     if (m < M && n < N) store_out<TO>(out + (size_t)m * N + n, acc[i][j][v]);
                 } else {
                     // columns come in blocks of 16: 8 gate, then their 8 up (8 lanes further on)
@@ -273,6 +280,41 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
         }
 }
 
+// out = sum over the shares of part[s][M][N], added in the order of s; EPI as in the products
+template <int EPI, typename TO>
+__global__ void splitk_reduce_kernel(const float* __restrict__ part, TO* __restrict__ out, int M, int N,
+                                     int S) {
+    const size_t MN = (size_t)M * N;
+    if (EPI == 0) {
+        for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < MN;
+             idx += (size_t)gridDim.x * blockDim.x) {
+            float t = 0.f;
+            for (int s = 0; s < S; ++s) t += part[s * MN + idx];
+            store_out<TO>(out + idx, t);
+        }
+    } else {
+        const int half = N / 2;
+        for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < (size_t)M * half;
+             idx += (size_t)gridDim.x * blockDim.x) {
+            const size_t m = idx / half;
+            const int c = (int)(idx - m * half);
+            const size_t gi = m * N + (size_t)(c >> 3) * 16 + (c & 7);
+            float g = 0.f, u = 0.f;
+            for (int s = 0; s < S; ++s) { g += part[s * MN + gi]; u += part[s * MN + gi + 8]; }
+            store_out<TO>(out + idx, swiglu_f(g, u));
+        }
+    }
+}
+
+// How many shares of K the product of these sizes is cut into (1: no workspace needed).
+static int splitk_shares(int M, int N, int K) {
+    if (M <= 16 || M > 64) return 1;
+    const int tiles_n = (N + 127) / 128, nk = K / TL_K;
+    int S = (320 + tiles_n / 2) / tiles_n;
+    if (S > nk / 4) S = nk / 4;
+    return S < 1 ? 1 : S;
+}
+
 template <int MT, int NT, int WAVES, int UNROLL, int EPI, typename TO>
 static void launch_skinny(const bf16* x, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
     const int rows = 16 * NT;
@@ -280,22 +322,32 @@ static void launch_skinny(const bf16* x, const bf16* w, TO* out, int M, int N, i
 }
 
 template <int EPI, typename TO>
-static int launch_bf16(const bf16* x, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
-    if (M <= 64) {
-        switch ((M + 15) / 16) {
-            case 1: launch_skinny<1, 1, 16, 2, EPI, TO>(x, w, out, M, N, K, s); break;
-            case 2: launch_skinny<2, 1, 16, 1, EPI, TO>(x, w, out, M, N, K, s); break;
-            case 3: launch_skinny<3, 2, 8, 1, EPI, TO>(x, w, out, M, N, K, s); break;
-            default: launch_skinny<4, 2, 8, 1, EPI, TO>(x, w, out, M, N, K, s); break;
-        }
+static int launch_bf16(const bf16* x, const bf16* w, TO* out, float* workspace, int M, int N, int K,
+                       hipStream_t s) {
+    if (M <= 16) {
+        launch_skinny<1, 1, 16, 2, EPI, TO>(x, w, out, M, N, K, s);
         LC_LAUNCH_CHECK("gemm_skinny");
+    } else if (M <= 64) {
+        // 64 x 128 tiles, K cut into shares so that every CU has a workgroup
+        const int S = splitk_shares(M, N, K), tiles_n = (N + 127) / 128;
+        if (S == 1) {
+            gemm_tiled_kernel<64, 128, 4, EPI, false, TO><<<tiles_n, 256, 0, s>>>(x, w, out, nullptr, M, N, K, 1, tiles_n);
+            LC_LAUNCH_CHECK("gemm_tiled");
+        } else {
+            LC_CHECK(workspace, "gemm_bf16: M=%d N=%d K=%d needs a workspace", M, N, K);
+            gemm_tiled_kernel<64, 128, 4, 0, true, TO><<<dim3(tiles_n, S), 256, 0, s>>>(x, w, out, workspace, M, N, K, 1, tiles_n);
+            LC_LAUNCH_CHECK("gemm_tiled");
+            const size_t work = EPI ? (size_t)M * N / 2 : (size_t)M * N;
+            splitk_reduce_kernel<EPI, TO><<<(int)((work + 255) / 256), 256, 0, s>>>(workspace, out, M, N, S);
+            LC_LAUNCH_CHECK("splitk_reduce");
+        }
     } else {
         const int big_m = (M + 255) / 256, big_n = (N + 255) / 256;
         if ((long long)big_m * big_n >= 512) {
-            gemm_tiled_kernel<256, 256, EPI, TO><<<big_m * big_n, 256, 0, s>>>(x, w, out, M, N, K, big_m, big_n);
+            gemm_tiled_kernel<256, 256, 2, EPI, false, TO><<<big_m * big_n, 256, 0, s>>>(x, w, out, nullptr, M, N, K, big_m, big_n);
         } else {
             const int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
-            gemm_tiled_kernel<128, 128, EPI, TO><<<tiles_m * tiles_n, 256, 0, s>>>(x, w, out, M, N, K, tiles_m, tiles_n);
+            gemm_tiled_kernel<128, 128, 2, EPI, false, TO><<<tiles_m * tiles_n, 256, 0, s>>>(x, w, out, nullptr, M, N, K, tiles_m, tiles_n);
         }
         LC_LAUNCH_CHECK("gemm_tiled");
     }
@@ -314,10 +366,18 @@ LC_API int lc_gemm_bf16_supported(int M, int N, int K) {
     return 1;
 }
 
+// float32 words of workspace that lc_gemm_bf16 needs for these sizes (0: none).
+LC_API long long lc_gemm_bf16_workspace(int M, int N, int K) {
+    if (!lc_gemm_bf16_supported(M, N, K)) return 0;
+    const int S = splitk_shares(M, N, K);
+    return S > 1 ? (long long)S * M * N : 0;
+}
+
 // epilogue 0: out[M, N] = x . w^T.  epilogue 1 (SwiGLU): the rows of w come in blocks of 16,
 // 8 gate rows followed by their 8 up rows; out[M, N / 2] = silu(gate) * up.
+// workspace: lc_gemm_bf16_workspace(M, N, K) float32 words (may be null when that is 0).
 LC_API int lc_gemm_bf16(const void* x, const void* w, void* out, int out_dt, int M, int N, int K,
-                        int epilogue, hipStream_t stream) {
+                        int epilogue, float* workspace, hipStream_t stream) {
     LC_CHECK(lc_gemm_bf16_supported(M, N, K), "gemm_bf16: sizes M=%d N=%d K=%d are not supported "
              "(K must be a multiple of %d)", M, N, K, SK_KBLOCK);
     LC_CHECK(x && w && out, "gemm_bf16: null pointer");
@@ -327,11 +387,11 @@ LC_API int lc_gemm_bf16(const void* x, const void* w, void* out, int out_dt, int
     const bf16* xb = (const bf16*)x;
     const bf16* wb = (const bf16*)w;
     if (out_dt == DT_BF16)
-        return epilogue ? launch_bf16<1, bf16>(xb, wb, (bf16*)out, M, N, K, stream)
-                        : launch_bf16<0, bf16>(xb, wb, (bf16*)out, M, N, K, stream);
+        return epilogue ? launch_bf16<1, bf16>(xb, wb, (bf16*)out, workspace, M, N, K, stream)
+                        : launch_bf16<0, bf16>(xb, wb, (bf16*)out, workspace, M, N, K, stream);
     if (out_dt == DT_F32)
-        return epilogue ? launch_bf16<1, float>(xb, wb, (float*)out, M, N, K, stream)
-                        : launch_bf16<0, float>(xb, wb, (float*)out, M, N, K, stream);
+        return epilogue ? launch_bf16<1, float>(xb, wb, (float*)out, workspace, M, N, K, stream)
+                        : launch_bf16<0, float>(xb, wb, (float*)out, workspace, M, N, K, stream);
     LC_CHECK(false, "gemm_bf16: unknown output dtype %d", out_dt);
     return 0;
 }

@@ -26,7 +26,7 @@ _SIGNATURES = {
     "lc_rmsnorm": "ppppfpiiiip",
     "lc_rmsnorm_act": "ppfpiiip",
     "lc_gemm_generic": "pipipiiiip",
-    "lc_gemm_bf16": "pppiiiiip",
+    "lc_gemm_bf16": "pppiiiiipp",
     "lc_gemm_bf16_supported": "iii",
     "lc_qk_norm_rope_write": "piiiiippfppipppip",
     "lc_attention_generic": "pipppipppiiiiiifip",
@@ -62,6 +62,8 @@ def library():
         except OSError as exc:
             raise KernelError(f"cannot load the kernel library {path}: {exc}") from exc
         lib.lc_last_error.restype = ctypes.c_char_p
+        lib.lc_gemm_bf16_workspace.restype = ctypes.c_longlong
+        lib.lc_gemm_bf16_workspace.argtypes = [ctypes.c_int] * 3
         for name, sig in _SIGNATURES.items():
             fn = getattr(lib, name, None)
             if fn is None:
@@ -177,7 +179,7 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = No
         return out
     if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and _fast_gemm_ok(M, N, K)):
         _call("lc_gemm_bf16", _ptr(x), _ptr(w), _ptr(out), _c_int(_dt(out)), _c_int(M), _c_int(N),
-              _c_int(K), 0, _stream())
+              _c_int(K), 0, _ptr(_gemm_workspace(M, N, K, x.device)), _stream())
     else:
         _call("lc_gemm_generic", _ptr(x), _c_int(_dt(x)), _ptr(w), _c_int(_dt(w)), _ptr(out),
               _c_int(_dt(out)), _c_int(M), _c_int(N), _c_int(K), _stream())
@@ -207,8 +209,15 @@ def gemm_swiglu(x: torch.Tensor, w_interleaved: torch.Tensor) -> torch.Tensor:
         raise KernelError(f"gemm_swiglu: x is [{M}, {K}], w is [{N}, {K2}] (rows must come in 16s)")
     out = torch.empty((M, N // 2), dtype=torch.bfloat16, device=x.device)
     if M:
-        _call("lc_gemm_bf16", _ptr(x), _ptr(w_interleaved), _ptr(out), DT_BF16, M, N, K, 1, _stream())
+        _call("lc_gemm_bf16", _ptr(x), _ptr(w_interleaved), _ptr(out), DT_BF16, M, N, K, 1,
+              _ptr(_gemm_workspace(M, N, K, x.device)), _stream())
     return out
+
+
+def _gemm_workspace(M: int, N: int, K: int, device) -> Optional[torch.Tensor]:
+    """Float32 scratch for the products that cut K into shares (None when none is needed)."""
+    words = library().lc_gemm_bf16_workspace(M, N, K)
+    return torch.empty((words,), dtype=torch.float32, device=device) if words else None
 
 
 def _fast_gemm_ok(M: int, N: int, K: int) -> bool:
