@@ -306,11 +306,14 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ part, TO* __restr
     }
 }
 
-// How many shares of K the product of these sizes is cut into (1: no workspace needed).
+// How many shares of K the product of these sizes is cut into (1: no workspace needed): as
+// many as it takes to give every CU a workgroup when whole-K tiles would be too few.
 static int splitk_shares(int M, int N, int K) {
-    if (M <= 16 || M > 64) return 1;
-    const int tiles_n = (N + 127) / 128, nk = K / TL_K;
-    int S = (320 + tiles_n / 2) / tiles_n;
+    if (M <= 16) return 1;
+    const int tiles = M <= 64 ? (N + 127) / 128 : ((M + 127) / 128) * ((N + 127) / 128);
+    if (tiles >= 200) return 1;
+    const int nk = K / TL_K;
+    int S = (320 + tiles / 2) / tiles;
     if (S > nk / 4) S = nk / 4;
     return S < 1 ? 1 : S;
 }
@@ -343,10 +346,21 @@ static int launch_bf16(const bf16* x, const bf16* w, TO* out, float* workspace, 
         }
     } else {
         const int big_m = (M + 255) / 256, big_n = (N + 255) / 256;
+        const int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
+        const int S = splitk_shares(M, N, K);
+        if (S > 1) {
+            LC_CHECK(workspace, "gemm_bf16: M=%d N=%d K=%d needs a workspace", M, N, K);
+            gemm_tiled_kernel<128, 128, 2, 0, true, TO><<<dim3(tiles_m * tiles_n, S), 256, 0, s>>>(
+                x, w, out, workspace, M, N, K, tiles_m, tiles_n);
+            LC_LAUNCH_CHECK("gemm_tiled");
+            const size_t work = EPI ? (size_t)M * N / 2 : (size_t)M * N;
+            splitk_reduce_kernel<EPI, TO><<<(int)((work + 255) / 256), 256, 0, s>>>(workspace, out, M, N, S);
+            LC_LAUNCH_CHECK("splitk_reduce");
+            return 0;
+        }
         if ((long long)big_m * big_n >= 512) {
             gemm_tiled_kernel<256, 256, 2, EPI, false, TO><<<big_m * big_n, 256, 0, s>>>(x, w, out, nullptr, M, N, K, big_m, big_n);
         } else {
-            const int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
             gemm_tiled_kernel<128, 128, 2, EPI, false, TO><<<tiles_m * tiles_n, 256, 0, s>>>(x, w, out, nullptr, M, N, K, tiles_m, tiles_n);
         }
         LC_LAUNCH_CHECK("gemm_tiled");
