@@ -116,9 +116,7 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
     the same make-up have the same layout; ``into``: the buffer of such an earlier batch."""
     bs = cache.block_size
     requests, q_start, first_pos, slot_list = [], [0], [], []
-    token_ids: List[int] = []
-    positions: List[int] = []
-    tok_req: List[int] = []
+    token_parts, position_parts, req_parts = [], [], []
     want_rows: List[int] = []
     for r, e in enumerate(entries):
         n = len(e.tokens)
@@ -130,11 +128,14 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
             if not 0 <= int(w) < n:
                 raise ValueError(f"request {e.request!r}: wanted place {w} is outside its {n} tokens")
             want_rows.append(q_start[-1] + int(w))
-        token_ids.extend(int(t) for t in e.tokens)
-        positions.extend(range(base, base + n))
-        tok_req.extend([r] * n)
+        token_parts.append(np.asarray(e.tokens, dtype=np.int32))
+        position_parts.append(np.arange(base, base + n, dtype=np.int32))
+        req_parts.append(np.full(n, r, dtype=np.int32))
         q_start.append(q_start[-1] + n)
     T, R = q_start[-1], len(entries)
+    token_ids = np.concatenate(token_parts) if token_parts else np.zeros(0, np.int32)
+    positions = np.concatenate(position_parts) if position_parts else np.zeros(0, np.int32)
+    tok_req = np.concatenate(req_parts) if req_parts else np.zeros(0, np.int32)
 
     pk = _Packer()
     h_tok = pk.add(token_ids)
@@ -166,15 +167,12 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
                 raise ValueError(f"pad_blocks {pad_blocks} is below the longest block table {mb}")
             mb = pad_blocks
         flat = np.full((R, mb), -1, dtype=np.int32)
+        slots = np.empty(T, dtype=np.int32)
         for r, t in enumerate(tables):
             flat[r, :len(t)] = t
-        slots = np.empty(T, dtype=np.int32)
-        for r in range(R):
-            tab = tables[r]
-            for i in range(q_start[r], q_start[r + 1]):
-                p = positions[i]
-                page = tab[p // bs]
-                slots[i] = page * bs + p % bs if page >= 0 else -1
+            pos = position_parts[r]
+            pages = flat[r, pos // bs]
+            slots[q_start[r]:q_start[r + 1]] = np.where(pages >= 0, pages * bs + pos % bs, -1)
         group_handles.append((pk.add(flat), mb, pk.add(slots)))
 
     buffer = pk.upload(device, into)
@@ -192,7 +190,7 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
     return StepBatch(
         num_tokens=T, num_requests=R, requests=requests, q_start=q_start,
         first_position=first_pos, slot_list=slot_list,
-        max_position=max(positions, default=0),
+        max_position=int(positions.max()) if T else 0,
         token_ids=pk.view(h_tok), positions=pk.view(h_pos), tok_req=pk.view(h_req),
         want_rows=pk.view(h_want), slot_ids=pk.view(h_slot), groups=groups,
         num_wanted=len(want_rows), buffer=buffer)

@@ -10,6 +10,7 @@ from __future__ import annotations
 
 from typing import Dict, Hashable, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
@@ -89,10 +90,13 @@ class ModelRunner:
             if e.request in seen:
                 raise ValueError(f"request {e.request!r} appears twice in one step")
             seen.add(e.request)
-            for t in e.tokens:
-                if not 0 <= int(t) < V:
-                    raise ValueError(f"request {e.request!r}: token id {t} is outside the "
-                                     f"vocabulary of {V}")
+            ids = np.asarray(e.tokens)
+            if ids.dtype.kind not in "iu":
+                raise ValueError(f"request {e.request!r}: token ids must be integers")
+            if int(ids.min()) < 0 or int(ids.max()) >= V:
+                bad = int(ids[(ids < 0) | (ids >= V)][0])
+                raise ValueError(f"request {e.request!r}: token id {bad} is outside the "
+                                 f"vocabulary of {V}")
             have = self.cache.length(e.request) if self.cache.has(e.request) else 0
             if limit and have + len(e.tokens) > limit:
                 raise ValueError(f"request {e.request!r}: {have + len(e.tokens)} tokens exceed "
