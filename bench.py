@@ -41,6 +41,11 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--points", default="1,64", help="further decode batch sizes (comma list, '' for none)")
     ap.add_argument("--block-size", type=int, default=16)
+    ap.add_argument("--workload", default="decode", choices=["decode", "mixed"],
+                    help="decode: the default line; mixed: 64 requests with prompts of 16 to 2,048 "
+                         "tokens through the scheduler (Qwen3-0.6B-shaped), chunked prefill beside decode")
+    ap.add_argument("--new-tokens", type=int, default=128, help="mixed: tokens generated per request")
+    ap.add_argument("--max-tokens-per-step", type=int, default=2048, help="mixed: the scheduler's budget")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -56,6 +61,8 @@ def main() -> int:
     dev = "cuda:0"
     torch.cuda.set_device(0)
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    if args.workload == "mixed":
+        return mixed_workload(args, dtype, dev)
     cfg = dict(SIZES_8B, architectures=["Qwen3ForCausalLM"], num_hidden_layers=args.layers)
     points = [int(p) for p in args.points.split(",") if p]
     max_batch = max([args.batch] + points)
@@ -155,6 +162,57 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
         "points": point_values,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+SIZES_06B = dict(num_hidden_layers=28, hidden_size=1024, num_attention_heads=16,
+                 num_key_value_heads=8, head_dim=128, intermediate_size=3072, vocab_size=151936,
+                 rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
+                 max_position_embeddings=40960, initializer_range=0.02)
+
+
+def mixed_workload(args, dtype, dev) -> int:
+    """64 requests with random prompts of 16 to 2,048 tokens, all submitted at once; the
+    scheduler cuts the prompts into portions under its token budget beside the decode tokens of
+    the requests that are already running."""
+    import random
+    import torch
+    from lucciola_amd.config.engine_config import EngineConfig
+    from lucciola_amd.engine.llm_engine import LLMEngine
+    from lucciola_amd.sampling.sampler import SamplingParams
+
+    cfg = dict(SIZES_06B, architectures=["Qwen3ForCausalLM"])
+    rng = random.Random(0)
+    prompts = [[rng.randrange(cfg["vocab_size"]) for _ in range(rng.randint(16, 2048))] for _ in range(64)]
+    total_tokens = sum(len(p) for p in prompts) + 64 * args.new_tokens
+    blocks = -(-total_tokens // args.block_size) + 64
+    engine = LLMEngine.from_random(cfg, 0, EngineConfig(
+        dtype=dtype, block_size=args.block_size, max_blocks=blocks, max_seqs=64,
+        max_tokens_per_step=args.max_tokens_per_step, device=dev))
+    params = SamplingParams(max_new_tokens=args.new_tokens, ignore_eos=True)
+    engine.generate(prompts[:4], SamplingParams(max_new_tokens=4, ignore_eos=True))   # warm-up
+    torch.cuda.synchronize()
+    steps0 = engine.runner.steps
+    t = time.perf_counter()
+    outputs = engine.generate(prompts, params)
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - t
+    generated = sum(len(o) for o in outputs)
+    prompt_tokens = sum(len(p) for p in prompts)
+    line = {
+        "metric": "tokens/s, 64 requests with prompts of 16..2048 tokens (Qwen3-0.6B-shaped), chunked prefill beside decode",
+        "value": round((prompt_tokens + generated) / seconds, 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": engine.runner.steps - steps0, "warmup": 1,
+        "ms_per_step": round(seconds * 1e3 / max(1, engine.runner.steps - steps0), 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
+        "data": "synthetic: random weights, random token ids",
+        "config": {"model": "Qwen3-0.6B-shaped", "layers": cfg["num_hidden_layers"], "requests": 64,
+                   "prompt_tokens": prompt_tokens, "generated_tokens": generated,
+                   "max_tokens_per_step": args.max_tokens_per_step, "page_size": args.block_size,
+                   "preemptions": engine.scheduler.num_preemptions, "seconds": round(seconds, 3),
+                   "generated_tokens_per_s": round(generated / seconds, 1)},
     }
     print(json.dumps(line), flush=True)
     return 0

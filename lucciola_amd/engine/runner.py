@@ -137,11 +137,17 @@ class ModelRunner:
         widest = max((len(g.tables[e.request]) for g in self.cache.groups for e in entries),
                      default=1)
         pad = max(64, -(-widest // 64) * 64)
+        # batches of 5 or more requests are filled up to a multiple of 8 with copies of the
+        # first entry (same token, same position, same cache slot: the copies compute and write
+        # what the original does), so that a batch that shrinks by one does not need a new graph
+        real = len(entries)
+        rows = real if real <= 4 else -(-real // 8) * 8
+        entries = list(entries) + [entries[0]] * (rows - real)
         epoch = self.model.position_epoch()
         if epoch != self._graph_epoch:      # a position table was made anew: addresses changed
             self._graphs.clear()
             self._graph_epoch = epoch
-        key = (len(entries), pad)
+        key = (rows, pad)
         captured = self._graphs.get(key)
         next_position = max(self.cache.length(e.request) for e in entries)
         if captured is None or not self.model.positions_ready(next_position):
@@ -158,11 +164,11 @@ class ModelRunner:
             with torch.cuda.graph(graph):
                 static_logits = self.model.forward(batch, sites)
             self._graphs[key] = _CapturedStep(graph, batch, sites, static_logits)
-            return logits
+            return logits[:real]
         build_batch(entries, self.cache, self.device, pad_blocks=pad, into=captured.batch.buffer)
         captured.graph.replay()
         self.graph_replays += 1
-        return captured.logits.clone()      # the next replay overwrites the graph's own output
+        return captured.logits[:real].clone()      # the next replay overwrites the graph's own output
 
     def _sites(self, batch: StepBatch) -> List[SiteView]:
         sites = []
