@@ -36,7 +36,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=8192)
-    ap.add_argument("--layers", type=int, default=SIZES_8B["num_hidden_layers"])
+    ap.add_argument("--model", default="8b", choices=["8b", "32b", "0.6b"],
+                    help="layer sizes: Qwen3-8B-shaped (the default line), 32B- or 0.6B-shaped")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the model has (0: all)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--points", default="1,64", help="further decode batch sizes (comma list, '' for none)")
@@ -63,7 +65,10 @@ def main() -> int:
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     if args.workload == "mixed":
         return mixed_workload(args, dtype, dev)
-    cfg = dict(SIZES_8B, architectures=["Qwen3ForCausalLM"], num_hidden_layers=args.layers)
+    sizes = {"8b": SIZES_8B, "32b": SIZES_32B, "0.6b": SIZES_06B}[args.model]
+    layers_full = sizes["num_hidden_layers"]
+    args.layers = args.layers or layers_full
+    cfg = dict(sizes, architectures=["Qwen3ForCausalLM"], num_hidden_layers=args.layers)
     points = [int(p) for p in args.points.split(",") if p]
     max_batch = max([args.batch] + points)
     steps_total = args.steps + args.warmup + 8
@@ -148,12 +153,12 @@ def main() -> int:
         print(f"[bench] decode batch {b}: {pm:.3f} ms/step", file=sys.stderr, flush=True)
 
     line = {
-        "metric": "decode tok/s (Qwen3-8B-shaped, batch 8, context 8192)",
+        "metric": f"decode tok/s (Qwen3-{args.model.upper()}-shaped, batch {args.batch}, context {args.context})",
         "value": round(tps, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
         "data": "synthetic: random weights, random token ids, cache of the live requests filled with random keys/values",
-        "config": {"model": "Qwen3-8B-shaped", "layers": L, "layers_full": SIZES_8B["num_hidden_layers"],
+        "config": {"model": f"Qwen3-{args.model.upper()}-shaped", "layers": L, "layers_full": layers_full,
                    "hidden": H, "heads": nh, "kv_heads": nkv, "head_dim": d, "intermediate": I,
                    "vocab": V, "global_batch": args.batch, "seq_len": args.context,
                    "page_size": bs, "prefill_tokens": args.prefill_tokens, "parallelism": "single GPU"},
@@ -166,6 +171,11 @@ def main() -> int:
     print(json.dumps(line), flush=True)
     return 0
 
+
+SIZES_32B = dict(num_hidden_layers=64, hidden_size=5120, num_attention_heads=64,
+                 num_key_value_heads=8, head_dim=128, intermediate_size=25600, vocab_size=151936,
+                 rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
+                 max_position_embeddings=40960, initializer_range=0.02)
 
 SIZES_06B = dict(num_hidden_layers=28, hidden_size=1024, num_attention_heads=16,
                  num_key_value_heads=8, head_dim=128, intermediate_size=3072, vocab_size=151936,
