@@ -29,12 +29,17 @@ def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="lucciola_amd", description=__doc__,
                                  formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--model", help="folder with config.json and model.safetensors")
-    ap.add_argument("--max-blocks", type=int, default=0,
+    ap.add_argument("--max-blocks", "--num-pages", dest="max_blocks", type=int, default=0,
                     help="pages of the cache; 0 sizes it from free memory (the reference's default)")
-    ap.add_argument("--block-size", type=int, default=16, help="tokens in a page")
+    ap.add_argument("--block-size", "--page-size", dest="block_size", type=int, default=16,
+                    help="tokens in a page")
+    ap.add_argument("--mem-fraction", type=float, default=0.90,
+                    help="with --max-blocks 0: share of the free memory the cache may take "
+                         "(the reference's 0.90, src/async_engine.cc:13)")
     ap.add_argument("--max-new-tokens", type=int, default=100)
     ap.add_argument("--temperature", type=float, default=0.0, help="0 is greedy")
-    ap.add_argument("--seed", type=int, default=0, help="of the sampler, or of --random-config")
+    ap.add_argument("--seed", "--sample-seed", dest="seed", type=int, default=0,
+                    help="of the sampler, or of --random-config")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--max-tokens-per-step", type=int, default=576)
     ap.add_argument("--max-seqs", type=int, default=256)
@@ -42,6 +47,7 @@ def main(argv=None) -> int:
     ap.add_argument("--prompt-ids", action="append", default=[],
                     help="a request as comma-separated token ids (may be given several times)")
     ap.add_argument("--prompt-ids-file", help="a file with one request of token ids per line")
+    ap.add_argument("--random-prompts", help="comma-separated lengths: one request of random ids for each")
     ap.add_argument("--random-config", help="a config.json to make random weights for")
     ap.add_argument("--write-model", help="with --random-config: the model folder to write")
     ap.add_argument("--device", default="cuda:0")
@@ -66,7 +72,8 @@ def main(argv=None) -> int:
 
     engine = LLMEngine.from_folder(args.model, EngineConfig(
         dtype=args.dtype, block_size=args.block_size, max_blocks=args.max_blocks,
-        max_tokens_per_step=args.max_tokens_per_step, max_seqs=args.max_seqs, device=args.device))
+        max_tokens_per_step=args.max_tokens_per_step, max_seqs=args.max_seqs, device=args.device,
+        memory_fraction=args.mem_fraction))
     print(f"model ready: {len(engine.model.layers)} layers, {engine.runner.cache.num_blocks} pages "
           f"of {args.block_size} tokens", file=sys.stderr, flush=True)
 
@@ -78,6 +85,11 @@ def main(argv=None) -> int:
     if args.prompt_ids_file:
         with open(args.prompt_ids_file, "r", encoding="utf-8") as fh:
             prompts += [_ids(line) for line in fh if line.strip()]
+    if args.random_prompts:
+        import random
+        rng = random.Random(args.seed)
+        prompts += [[rng.randrange(engine.model.vocab_size) for _ in range(n)]
+                    for n in _ids(args.random_prompts)]
     if prompts:
         outputs = engine.generate(prompts, [params(i) for i in range(len(prompts))])
         for out in outputs:

@@ -89,6 +89,18 @@ class LLMEngine:
                 outputs.append(StepOutput(seq.seq_id, token, finished))
         return outputs
 
+    def stats(self) -> Dict[str, int]:
+        """Counters: steps and tokens run, graph replays, preemptions, pages and slots in use."""
+        cache = self.runner.cache
+        return {
+            "steps": self.runner.steps, "tokens": self.runner.tokens,
+            "graph_replays": self.runner.graph_replays,
+            "preemptions": self.scheduler.num_preemptions,
+            "waiting": len(self.scheduler.waiting), "running": len(self.scheduler.running),
+            "pages_total": cache.num_blocks, "pages_free": cache.num_free_blocks(),
+            "slots_free": cache.slots.num_free(),
+        }
+
     # ------------------------------------------------------------------ whole requests
     def generate(self, prompts: Seq[Seq[int]], params=None,
                  on_token: Optional[Callable[[int, int, bool], None]] = None) -> List[List[int]]:

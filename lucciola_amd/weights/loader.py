@@ -12,6 +12,7 @@ float32 (norm weights) are widened to float32, which changes no value.
 """
 from __future__ import annotations
 
+import json
 import os
 from dataclasses import dataclass
 from typing import Callable, Dict, Iterable, List, Mapping, Optional, Tuple
@@ -80,24 +81,48 @@ class WeightSource:
 
 
 class FolderSource(WeightSource):
-    """``model.safetensors`` of a model folder (src/qwen.cc:69: a single file of that name)."""
+    """The weights of a model folder: ``model.safetensors`` (src/qwen.cc:69: a single file of
+    that name), or, for checkpoints that are cut into shards, the files that
+    ``model.safetensors.index.json`` names under ``weight_map``."""
 
     def __init__(self, folder: str):
-        self.where = os.path.join(folder, "model.safetensors")
-        self._file = SafetensorsFile(self.where)
+        single = os.path.join(folder, "model.safetensors")
+        index = os.path.join(folder, "model.safetensors.index.json")
+        self._files: Dict[str, SafetensorsFile] = {}
+        self._where_is: Dict[str, str] = {}
+        if os.path.isfile(single) or not os.path.isfile(index):
+            self.where = single
+            self._files[single] = SafetensorsFile(single)      # raises if there is none
+            for name in self._files[single].names():
+                self._where_is[name] = single
+            return
+        self.where = index
+        with open(index, "r", encoding="utf-8") as fh:
+            try:
+                weight_map = json.load(fh)["weight_map"]
+            except (json.JSONDecodeError, KeyError, TypeError) as exc:
+                raise WeightsError(index, [], [], [], [("weight_map", f"unreadable index ({exc})")]) from exc
+        for name, shard in weight_map.items():
+            path = os.path.join(folder, shard)
+            if path not in self._files:
+                self._files[path] = SafetensorsFile(path)
+            if name not in self._files[path].entries:
+                raise WeightsError(index, [name], [], [])
+            self._where_is[name] = path
 
     def names(self) -> List[str]:
-        return self._file.names()
+        return list(self._where_is)
 
     def shape_dtype(self, name):
-        e = self._file.entries[name]
+        e = self._files[self._where_is[name]].entries[name]
         return e.shape, e.dtype
 
     def get(self, name: str) -> torch.Tensor:
-        return self._file.get(name)
+        return self._files[self._where_is[name]].get(name)
 
     def close(self) -> None:
-        self._file.close()
+        for f in self._files.values():
+            f.close()
 
 
 class DictSource(WeightSource):

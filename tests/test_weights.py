@@ -181,3 +181,33 @@ def test_head_follows_the_checkpoint_as_in_the_reference(tmp_path):
     write_safetensors(os.path.join(folder_a, "model.safetensors"), tensors.items())
     model, _ = load_model(folder_a, "float32", "cpu")
     assert model.head is model.embedding
+
+
+def test_sharded_checkpoint(tmp_path):
+    """model.safetensors.index.json names the shard that holds each tensor."""
+    cfg, _, seed = configs.ALL["B"]
+    folder = write_model_folder(str(tmp_path / "m"), cfg, seed)
+    with SafetensorsFile(os.path.join(folder, "model.safetensors")) as f:
+        tensors = {n: f.get(n).clone() for n in f.names()}
+    os.remove(os.path.join(folder, "model.safetensors"))
+    names = sorted(tensors)
+    shards = {"model-00001-of-00002.safetensors": names[::2], "model-00002-of-00002.safetensors": names[1::2]}
+    weight_map = {}
+    for shard, members in shards.items():
+        write_safetensors(os.path.join(folder, shard), [(n, tensors[n]) for n in members])
+        weight_map.update({n: shard for n in members})
+    with open(os.path.join(folder, "model.safetensors.index.json"), "w") as fh:
+        json.dump({"metadata": {}, "weight_map": weight_map}, fh)
+    source = FolderSource(folder)
+    assert sorted(source.names()) == names
+    assert all(torch.equal(source.get(n), tensors[n]) for n in names)
+    source.close()
+    model, _ = load_model(folder, "float32", "cpu")
+    assert len(model.layers) == cfg["num_hidden_layers"]
+    # an index that names a tensor its shard does not hold
+    weight_map[names[0]] = "model-00002-of-00002.safetensors"
+    with open(os.path.join(folder, "model.safetensors.index.json"), "w") as fh:
+        json.dump({"weight_map": weight_map}, fh)
+    with pytest.raises(WeightsError) as info:
+        FolderSource(folder)
+    assert info.value.missing == [names[0]]
