@@ -8,8 +8,6 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Callable, Dict, List, Optional, Sequence as Seq
 
-import torch
-
 from ..config.engine_config import EngineConfig
 from ..sampling.sampler import Sampler, SamplingParams
 from .loading import load_model, random_model

@@ -21,7 +21,7 @@ from typing import Any, Dict, Optional
 
 import torch
 
-from ..config.registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Registry)
+from ..config.registry import Registry
 from ..config.specs import PartSpec
 from ..weights.loader import ParamDecl
 
@@ -45,7 +45,7 @@ class ResidualStream:
 
 
 class Part:
-    """Base of all parts.  Subclasses set ``self.p`` from keyword parameters in ``__init__``."""
+    """Base of all parts.  A part is built from keyword parameters (its sizes and constants)."""
 
     # True if ``forward`` only launches kernels on tensors whose addresses and shapes depend
     # on nothing but the batch layout (no host-side reads of batch values, no loops over

@@ -13,7 +13,7 @@ import os
 import struct
 import warnings
 from dataclasses import dataclass
-from typing import Dict, Iterable, Iterator, List, Tuple
+from typing import Dict, Iterable, List, Tuple
 
 import numpy as np
 import torch
