@@ -6,11 +6,11 @@
 //    rows straight from global memory into v_mfma_f32_16x16x32_bf16 operands (w is the A
 //    operand, x^T the B operand); the waves' partial sums meet in LDS.  No split-K workspace,
 //    no atomics: the order of the sums is fixed.
-//  * tiled (M > 16): 128x128x64 or 256x256x64 workgroup tiles (64x128x64 with K cut into shares
-//    and a reduction kernel for 16 < M <= 64, where whole-K tiles would leave CUs idle) that go from global
-//    memory straight into a ring of LDS stages, 4 waves built from v_mfma_f32_32x32x16_bf16 with
-//    hand-pipelined operand reads.  Workgroups are renumbered so that each XCD's L2 sees
-//    neighbouring tiles.
+//  * tiled (M > 16): workgroup tiles of 64x128 to 256x256 by 64 (the small ones with K cut into
+//    shares and a reduction kernel where whole-K tiles would leave CUs idle) that go from global
+//    memory straight into a ring of LDS stages, 4 waves built from v_mfma_f32_32x32x16_bf16 in
+//    a hand-scheduled loop.  Workgroups are renumbered so that each XCD's L2 sees neighbouring
+//    tiles.
 //
 // The reference's linear kernel computes the same product with one thread per output element
 // and no matrix instruction (src/kernels/linear.cu:7-56).
@@ -117,19 +117,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 
 // ------------------------------------------------------------------------------- tiled
 // Workgroup tile BM x BN x 64, four waves in a 2 x 2 grid, each owning (BM/64) x (BN/64) tiles
-// of 32 x 32.  128 x 128 (two workgroups to a CU) for most shapes, 256 x 256 where the grid
-// still has two tiles per CU: it halves the bytes that cross the L2 per product.
+// of 32 x 32.
 //
 // Operand tiles go from global memory straight into LDS (global_load_lds_dwordx4: lane l's 16
 // bytes land at the instruction's LDS base + 16 l, no registers in between) into a ring of
-// TL_STAGES stages; a stage is filled while the one before it is multiplied.  Inside a stage
-// a row's eight 16-byte chunks are stored at column (chunk ^ (row & 7)), which spreads the 32
-// rows of an operand read over all banks without padding.  The LDS reads are written by hand
-// (ds_read_b128 + explicit waits), two k-steps deep, for two reasons: the products of one
-// k-step then hide the reads of the next although a SIMD may hold a single wave, and the
-// compiler, which cannot tell the stages apart, would otherwise make every load in flight
-// land before any read.  Likewise the barrier is the bare instruction: each wave first waits
-// for its own loads of the stage, the barrier then makes all waves' loads visible.
+// TL_STAGES stages.  Inside a stage a row's eight 16-byte chunks are stored at column
+// (chunk ^ ((row >> 1) & 7)): the 16 lanes that the LDS serves per cycle for a 128-bit read
+// (16 consecutive rows, one chunk) then cover all 64 banks.
+//
+// The loop is scheduled by hand, because a SIMD holds a single wave of this kernel and nothing
+// else hides a stall.  Per k-step of 16 the wave issues its (BM/64)*(BN/64) products; between
+// them, one at a time, go the LDS reads of the NEXT k-step's operands (ds_read_b128 in inline
+// assembly with explicit waits: the compiler cannot tell the stages apart and would make every
+// load in flight land before any read) and, in a block's first k-step, the global loads of the
+// block TL_STAGES-1 ahead.  In a block's last k-step the wave waits for its own loads of the
+// next block, meets the others at a bare barrier (all waves' loads are then visible, and all
+// have finished reading the stage that the next loads overwrite) and reads the next block's
+// first operands while the rest of its products run.  sched_barrier pins that order.
 constexpr int TL_K = 64;
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef __attribute__((address_space(1))) const void* glb_ptr_t;
@@ -148,10 +152,15 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
                                                          const bf16* __restrict__ w,
                                                          TO* __restrict__ out, float* __restrict__ part,
                                                          int M, int N, int K, int tiles_m, int tiles_n) {
+    constexpr int S = TL_STAGES;
     constexpr int TM = BM / 64, TN = BN / 64;
-    constexpr int LPA = BM * 8 / 256, LPB = BN * 8 / 256;   // load instructions per thread and stage
-    __shared__ __attribute__((aligned(16))) bf16 As[TL_STAGES][BM * TL_K];
-    __shared__ __attribute__((aligned(16))) bf16 Bs[TL_STAGES][BN * TL_K];
+    constexpr int KS = TL_K / 16;                             // k-steps per block
+    constexpr int LPA = BM * 8 / 256, LPB = BN * 8 / 256, LP = LPA + LPB;   // load instructions per thread and stage
+    constexpr int NM = TM * TN, NR = TM + TN;                 // products and operand reads per k-step
+    constexpr int A_STAGE = BM * TL_K * 2, B_STAGE = BN * TL_K * 2;          // bytes
+    static_assert(S >= 2 && (S - 1) * LP <= 63, "the load counter holds 63");
+    static_assert(S * (A_STAGE + B_STAGE) <= 160 * 1024, "LDS");
+    __shared__ __attribute__((aligned(1024))) char lds[S * (A_STAGE + B_STAGE)];   // A stages, then B stages
 
     // renumber: workgroups go round-robin over 8 XCDs; give each XCD a contiguous run of
     // tiles, m fastest, so that one XCD's L2 keeps the w tile that its workgroups share
@@ -165,39 +174,44 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
     const int tm = id % tiles_m, tn = id / tiles_m;
     const int m0 = tm * BM, n0 = tn * BN;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
     const int lr = lane & 31, kg = lane >> 5;
+    auto swz = [](int row) { return (row >> 1) & 7; };
 
-    // chunk p = (i * 4 + wave) * 64 + lane of a stage holds row p / 8, global column (p % 8) ^ (row & 7)
+    const int nk_all = K / TL_K;
+    const int kb0 = SPLIT ? (int)((long long)blockIdx.y * nk_all / gridDim.y) : 0;
+    const int nk = (SPLIT ? (int)((long long)(blockIdx.y + 1) * nk_all / gridDim.y) : nk_all) - kb0;
+
+    // chunk p = (i * 4 + wave) * 64 + lane of a stage holds row p / 8, global chunk (p % 8) ^ swz(row)
     const bf16* xg[LPA];
     const bf16* wg[LPB];
 #pragma unroll
     for (int i = 0; i < LPA; ++i) {
-        const int p = (i * 4 + wave) * 64 + lane, row = p >> 3, kc = (p & 7) ^ (row & 7);
-        xg[i] = x + (size_t)min(m0 + row, M - 1) * K + kc * 8;
+        const int p = (i * 4 + wave) * 64 + lane, row = p >> 3, kc = (p & 7) ^ swz(row);
+        xg[i] = x + (size_t)min(m0 + row, M - 1) * K + (size_t)kb0 * TL_K + kc * 8;
     }
 #pragma unroll
     for (int i = 0; i < LPB; ++i) {
-        const int p = (i * 4 + wave) * 64 + lane, row = p >> 3, kc = (p & 7) ^ (row & 7);
-        wg[i] = w + (size_t)min(n0 + row, N - 1) * K + kc * 8;
+        const int p = (i * 4 + wave) * 64 + lane, row = p >> 3, kc = (p & 7) ^ swz(row);
+        wg[i] = w + (size_t)min(n0 + row, N - 1) * K + (size_t)kb0 * TL_K + kc * 8;
     }
-    auto issue = [&](int kb, int stage) {
-#pragma unroll
-        for (int i = 0; i < LPA; ++i)
-            __builtin_amdgcn_global_load_lds((glb_ptr_t)(xg[i] + kb * TL_K),
-                                             (lds_ptr_t)(&As[stage][(i * 4 + wave) * 512]), 16, 0, 0);
-#pragma unroll
-        for (int i = 0; i < LPB; ++i)
-            __builtin_amdgcn_global_load_lds((glb_ptr_t)(wg[i] + kb * TL_K),
-                                             (lds_ptr_t)(&Bs[stage][(i * 4 + wave) * 512]), 16, 0, 0);
+    // load instruction idx (x first, then w) of block kb into a stage
+    auto issue_one = [&](int idx, int kb, int stage) {
+        if (idx < LPA)
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(xg[idx] + kb * TL_K),
+                (lds_ptr_t)(lds + stage * A_STAGE + (idx * 4 + wave) * 1024), 16, 0, 0);
+        else
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(wg[idx - LPA] + kb * TL_K),
+                (lds_ptr_t)(lds + S * A_STAGE + stage * B_STAGE + ((idx - LPA) * 4 + wave) * 1024), 16, 0, 0);
     };
-    const int nk_all = K / TL_K;
-    const int kb0 = SPLIT ? (int)((long long)blockIdx.y * nk_all / gridDim.y) : 0;
-    const int nk = (SPLIT ? (int)((long long)(blockIdx.y + 1) * nk_all / gridDim.y) : nk_all) - kb0;
 #pragma unroll
-    for (int s = 0; s < TL_STAGES - 1; ++s)
-        if (s < nk) issue(kb0 + s, s);
+    for (int s = 0; s < S - 1; ++s)
+        if (s < nk) {
+#pragma unroll
+            for (int i = 0; i < LP; ++i) issue_one(i, s, s);
+        }
 
     floatx16 acc[TM][TN];
 #pragma unroll
@@ -207,55 +221,116 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    // byte offsets of this lane's operand rows inside a stage, and their swizzles
-    unsigned arow[TM], brow[TN];
-    int asw[TM], bsw[TN];
+    // LDS address of this lane's operand rows in stage 0, with the lane's part of the swizzle;
+    // k-step ks flips chunk bits: ((2 ks + kg) ^ swz) * 16 = ((kg ^ swz) * 16) ^ (ks * 32)
+    const unsigned lds0 = (unsigned)(uintptr_t)(lds_ptr_t)lds;
+    unsigned pa[TM], pb[TN];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) { const int row = wm + i * 32 + lr; arow[i] = row * 128; asw[i] = row & 7; }
-#pragma unroll
-    for (int j = 0; j < TN; ++j) { const int row = wn + j * 32 + lr; brow[j] = row * 128; bsw[j] = row & 7; }
-
-    for (int it = 0; it < nk; ++it) {
-        // block `it` has landed when at most the younger blocks' loads are still in flight
-        if (it + TL_STAGES - 2 < nk) wait_vmcnt<(TL_STAGES - 2) * (LPA + LPB)>(); else wait_vmcnt<0>();
-        __builtin_amdgcn_s_barrier();
-        if (it + TL_STAGES - 1 < nk) issue(kb0 + it + TL_STAGES - 1, (it + TL_STAGES - 1) % TL_STAGES);
-        const unsigned abase = (unsigned)(uintptr_t)(lds_ptr_t)As[it % TL_STAGES];
-        const unsigned bbase = (unsigned)(uintptr_t)(lds_ptr_t)Bs[it % TL_STAGES];
-        bf16x8 a[2][TM], b[2][TN];
-        auto read = [&](int ks, int buf) {
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const unsigned addr = abase + arow[i] + (((ks * 2 + kg) ^ asw[i]) * 16);
-                asm volatile("ds_read_b128 %0, %1" : "=v"(a[buf][i]) : "v"(addr));
-            }
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const unsigned addr = bbase + brow[j] + (((ks * 2 + kg) ^ bsw[j]) * 16);
-                asm volatile("ds_read_b128 %0, %1" : "=v"(b[buf][j]) : "v"(addr));
-            }
-        };
-        read(0, 0);
-#pragma unroll
-        for (int ks = 0; ks < TL_K / 16; ++ks) {
-            if (ks + 1 < TL_K / 16) {
-                read(ks + 1, (ks + 1) & 1);
-                wait_lgkmcnt<TM + TN>();       // this k-step's operands are in; the next one's may be out
-            } else {
-                wait_lgkmcnt<0>();
-            }
-            // the products below must not be moved above the wait: tie their operands to this point
-#pragma unroll
-            for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(a[ks & 1][i]));
-#pragma unroll
-            for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(b[ks & 1][j]));
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks & 1][i], b[ks & 1][j], acc[i][j], 0, 0, 0);
-        }
+    for (int i = 0; i < TM; ++i) {
+        const int row = wm + i * 32 + lr;
+        pa[i] = lds0 + row * 128 + ((kg ^ swz(row)) * 16);
     }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int row = wn + j * 32 + lr;
+        pb[j] = lds0 + S * A_STAGE + row * 128 + ((kg ^ swz(row)) * 16);
+    }
+
+    bf16x8 a[2][TM], b[2][TN];
+    auto read_one = [&](int r, int stage, int ks, int buf) {
+        if (r < TM) {
+            const unsigned addr = (pa[r] ^ (ks * 32)) + stage * A_STAGE;
+            asm volatile("ds_read_b128 %0, %1" : "=v"(a[buf][r]) : "v"(addr));
+        } else {
+            const unsigned addr = (pb[r - TM] ^ (ks * 32)) + stage * B_STAGE;
+            asm volatile("ds_read_b128 %0, %1" : "=v"(b[buf][r - TM]) : "v"(addr));
+        }
+    };
+    // the products that follow a wait must not be moved above it: tie their operands to that point
+    auto tie = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(a[buf][i]));
+#pragma unroll
+        for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(b[buf][j]));
+    };
+    auto product = [&](int k, int buf) {
+        const int i = k / TN, j = k % TN;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[buf][i], b[buf][j], acc[i][j], 0, 0, 0);
+    };
+
+    // where the reads and loads sit among the NM products of a k-step
+    constexpr int QR = (2 * NR + NM - 1) / NM;                 // reads after each product, from the first on
+    constexpr int RS = (NR + QR - 1) / QR;                     // products that the reads take
+    constexpr int QL = NM > RS ? (LP + (NM - RS) - 1) / (NM - RS) : LP;   // loads after each later product
+    constexpr int BAR = NM / 4;                                // the product after which a block's last k-step syncs
+    constexpr int QT = NM - BAR - 1 > 0 ? (NR + (NM - BAR - 1) - 1) / (NM - BAR - 1) : NR;
+
+    // block 0 has landed when at most the S-2 younger blocks are still in flight
+    if (nk >= S - 1) wait_vmcnt<(S - 2) * LP>(); else wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int r = 0; r < NR; ++r) read_one(r, 0, 0, 0);
+
+    int stage = 0, lstage = S - 1;   // the stage of block `it`; the stage that block it+S-1 goes to
+    auto block = [&](int it, auto load_tag) {
+        constexpr bool LOAD = decltype(load_tag)::value;       // block it+S-1 exists and is loaded here
+        const int nstage = stage + 1 == S ? 0 : stage + 1;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int cur = ks & 1, nxt = cur ^ 1;
+            wait_lgkmcnt<0>();
+            tie(cur);
+            __builtin_amdgcn_sched_barrier(0);
+            if (ks < KS - 1) {
+#pragma unroll
+                for (int k = 0; k < NM; ++k) {
+                    product(k, cur);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int r = k * QR; r < (k + 1) * QR; ++r)
+                        if (r < NR) read_one(r, stage, ks + 1, nxt);
+                    if (LOAD && ks == 0 && (k >= RS || NM == RS)) {
+                        const int first = NM == RS ? k * QL : (k - RS) * QL;
+#pragma unroll
+                        for (int l = first; l < first + QL; ++l)
+                            if (l < LP) issue_one(l, it + S - 1, lstage);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < NM; ++k) {
+                    product(k, cur);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (LOAD) {
+                        if (k == BAR) { wait_vmcnt<(S - 2) * LP>(); __builtin_amdgcn_s_barrier(); }
+                        if (NM - BAR - 1 > 0) {
+#pragma unroll
+                            for (int r = (k - BAR - 1) * QT; r < (k - BAR) * QT; ++r)
+                                if (k > BAR && r < NR) read_one(r, nstage, 0, nxt);
+                        } else if (k == BAR) {
+#pragma unroll
+                            for (int r = 0; r < NR; ++r) read_one(r, nstage, 0, nxt);
+                        }
+                    } else if (k == BAR) {
+                        if (it + 1 < nk) {
+                            wait_vmcnt<0>();
+                            __builtin_amdgcn_s_barrier();
+#pragma unroll
+                            for (int r = 0; r < NR; ++r) read_one(r, nstage, 0, nxt);
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        stage = nstage;
+        lstage = lstage + 1 == S ? 0 : lstage + 1;
+    };
+    int it = 0;
+    for (; it + S - 1 < nk; ++it) block(it, std::true_type{});
+    for (; it < nk; ++it) block(it, std::false_type{});
+
     // acc[i][j][v]: row m = (v/4)*8 + (lane/32)*4 + v%4, column n = lane%32 of the 32x32 tile
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -306,14 +381,46 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ part, TO* __restr
     }
 }
 
+// The tile shapes of the tiled kernel.  TILE_AUTO picks by size; the others are forced through
+// lc_gemm_bf16_force_tile (tests and tuning).
+enum : int { TILE_AUTO = -1, TILE_64x128 = 0, TILE_128x128 = 1, TILE_256x128 = 2, TILE_256x256 = 3, TILE_COUNT = 4 };
+static int g_force_tile = TILE_AUTO;
+constexpr int kCUs = 256;
+
+static int tile_bm(int t) { return t == TILE_64x128 ? 64 : t == TILE_128x128 ? 128 : 256; }
+static int tile_bn(int t) { return t == TILE_256x256 ? 256 : 128; }
+static long long tile_count(int t, int M, int N) {
+    return (long long)((M + tile_bm(t) - 1) / tile_bm(t)) * ((N + tile_bn(t) - 1) / tile_bn(t));
+}
+
+// The tile for a product with M > 16.  Up to 64 rows: the 64-row tile.  Beyond: the shape with
+// the least estimated time, (tiles a CU works through) x (tile area) / (measured relative rate
+// of the shape: larger tiles move fewer bytes per product).
+static int pick_tile(int M, int N) {
+    if (g_force_tile != TILE_AUTO) return g_force_tile;
+    if (M <= 64) return TILE_64x128;
+    const double rate[TILE_COUNT] = {0.0, 0.87, 1.0, 1.2};
+    int best = TILE_128x128;
+    double best_cost = 0.0;
+    for (int t = TILE_128x128; t < TILE_COUNT; ++t) {
+        const long long per_cu = (tile_count(t, M, N) + kCUs - 1) / kCUs;
+        const double cost = (double)per_cu * tile_bm(t) * tile_bn(t) / rate[t];
+        if (t == TILE_128x128 || cost < best_cost) { best = t; best_cost = cost; }
+    }
+    return best;
+}
+
 // How many shares of K the product of these sizes is cut into (1: no workspace needed): as
-// many as it takes to give every CU a workgroup when whole-K tiles would be too few.
+// many as it takes to give every CU a workgroup when whole-K tiles would be too few.  Only the
+// two small tiles are cut.
 static int splitk_shares(int M, int N, int K) {
     if (M <= 16) return 1;
-    const int tiles = M <= 64 ? (N + 127) / 128 : ((M + 127) / 128) * ((N + 127) / 128);
+    const int t = pick_tile(M, N);
+    if (t != TILE_64x128 && t != TILE_128x128) return 1;
+    const long long tiles = tile_count(t, M, N);
     if (tiles >= 200) return 1;
     const int nk = K / TL_K;
-    int S = (320 + tiles / 2) / tiles;
+    int S = (int)((320 + tiles / 2) / tiles);
     if (S > nk / 4) S = nk / 4;
     return S < 1 ? 1 : S;
 }
@@ -324,48 +431,45 @@ static void launch_skinny(const bf16* x, const bf16* w, TO* out, int M, int N, i
     gemm_skinny_kernel<MT, NT, WAVES, UNROLL, EPI, TO><<<(N + rows - 1) / rows, WAVES * 64, 0, s>>>(x, w, out, M, N, K);
 }
 
+template <int BM, int BN, int STAGES, int EPI, typename TO>
+static int launch_tiled(const bf16* x, const bf16* w, TO* out, float* workspace, int M, int N, int K,
+                        int shares, hipStream_t s) {
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    if (shares == 1) {
+        gemm_tiled_kernel<BM, BN, STAGES, EPI, false, TO><<<tiles_m * tiles_n, 256, 0, s>>>(
+            x, w, out, nullptr, M, N, K, tiles_m, tiles_n);
+        LC_LAUNCH_CHECK("gemm_tiled");
+        return 0;
+    }
+    if constexpr (BM <= 128 && BN == 128) {
+        LC_CHECK(workspace, "gemm_bf16: M=%d N=%d K=%d needs a workspace", M, N, K);
+        gemm_tiled_kernel<BM, BN, STAGES, 0, true, TO><<<dim3(tiles_m * tiles_n, shares), 256, 0, s>>>(
+            x, w, out, workspace, M, N, K, tiles_m, tiles_n);
+        LC_LAUNCH_CHECK("gemm_tiled");
+        const size_t work = EPI ? (size_t)M * N / 2 : (size_t)M * N;
+        splitk_reduce_kernel<EPI, TO><<<(int)((work + 255) / 256), 256, 0, s>>>(workspace, out, M, N, shares);
+        LC_LAUNCH_CHECK("splitk_reduce");
+        return 0;
+    }
+    LC_CHECK(false, "gemm_bf16: tile %dx%d is not cut along K", BM, BN);
+    return 0;
+}
+
 template <int EPI, typename TO>
 static int launch_bf16(const bf16* x, const bf16* w, TO* out, float* workspace, int M, int N, int K,
                        hipStream_t s) {
-    if (M <= 16) {
+    if (M <= 16 && g_force_tile == TILE_AUTO) {
         launch_skinny<1, 1, 16, 2, EPI, TO>(x, w, out, M, N, K, s);
         LC_LAUNCH_CHECK("gemm_skinny");
-    } else if (M <= 64) {
-        // 64 x 128 tiles, K cut into shares so that every CU has a workgroup
-        const int S = splitk_shares(M, N, K), tiles_n = (N + 127) / 128;
-        if (S == 1) {
-            gemm_tiled_kernel<64, 128, 4, EPI, false, TO><<<tiles_n, 256, 0, s>>>(x, w, out, nullptr, M, N, K, 1, tiles_n);
-            LC_LAUNCH_CHECK("gemm_tiled");
-        } else {
-            LC_CHECK(workspace, "gemm_bf16: M=%d N=%d K=%d needs a workspace", M, N, K);
-            gemm_tiled_kernel<64, 128, 4, 0, true, TO><<<dim3(tiles_n, S), 256, 0, s>>>(x, w, out, workspace, M, N, K, 1, tiles_n);
-            LC_LAUNCH_CHECK("gemm_tiled");
-            const size_t work = EPI ? (size_t)M * N / 2 : (size_t)M * N;
-            splitk_reduce_kernel<EPI, TO><<<(int)((work + 255) / 256), 256, 0, s>>>(workspace, out, M, N, S);
-            LC_LAUNCH_CHECK("splitk_reduce");
-        }
-    } else {
-        const int big_m = (M + 255) / 256, big_n = (N + 255) / 256;
-        const int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
-        const int S = splitk_shares(M, N, K);
-        if (S > 1) {
-            LC_CHECK(workspace, "gemm_bf16: M=%d N=%d K=%d needs a workspace", M, N, K);
-            gemm_tiled_kernel<128, 128, 2, 0, true, TO><<<dim3(tiles_m * tiles_n, S), 256, 0, s>>>(
-                x, w, out, workspace, M, N, K, tiles_m, tiles_n);
-            LC_LAUNCH_CHECK("gemm_tiled");
-            const size_t work = EPI ? (size_t)M * N / 2 : (size_t)M * N;
-            splitk_reduce_kernel<EPI, TO><<<(int)((work + 255) / 256), 256, 0, s>>>(workspace, out, M, N, S);
-            LC_LAUNCH_CHECK("splitk_reduce");
-            return 0;
-        }
-        if ((long long)big_m * big_n >= 512) {
-            gemm_tiled_kernel<256, 256, 2, EPI, false, TO><<<big_m * big_n, 256, 0, s>>>(x, w, out, nullptr, M, N, K, big_m, big_n);
-        } else {
-            gemm_tiled_kernel<128, 128, 2, EPI, false, TO><<<tiles_m * tiles_n, 256, 0, s>>>(x, w, out, nullptr, M, N, K, tiles_m, tiles_n);
-        }
-        LC_LAUNCH_CHECK("gemm_tiled");
+        return 0;
     }
-    return 0;
+    const int shares = splitk_shares(M, N, K);
+    switch (pick_tile(M, N)) {
+    case TILE_64x128:  return launch_tiled<64, 128, 4, EPI, TO>(x, w, out, workspace, M, N, K, shares, s);
+    case TILE_128x128: return launch_tiled<128, 128, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, s);
+    case TILE_256x128: return launch_tiled<256, 128, 3, EPI, TO>(x, w, out, workspace, M, N, K, shares, s);
+    default:           return launch_tiled<256, 256, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, s);
+    }
 }
 
 }  // namespace lc
@@ -376,8 +480,16 @@ using namespace lc;
 LC_API int lc_gemm_bf16_supported(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     if (K % SK_KBLOCK != 0) return 0;
-    if ((size_t)((M + 127) / 128) * ((N + 127) / 128) > 0x7fffffffu) return 0;
+    if ((size_t)((M + 63) / 64) * ((N + 127) / 128) > 0x7fffffffu) return 0;
     return 1;
+}
+
+// Forces the tile shape of the tiled kernel for every later product of any M (-1: choose by
+// size again).  For tests and tuning; not for use while other threads launch products.
+LC_API int lc_gemm_bf16_force_tile(int tile) {
+    LC_CHECK(tile >= TILE_AUTO && tile < TILE_COUNT, "gemm_bf16: no tile shape %d", tile);
+    g_force_tile = tile;
+    return 0;
 }
 
 // float32 words of workspace that lc_gemm_bf16 needs for these sizes (0: none).

@@ -28,6 +28,7 @@ _SIGNATURES = {
     "lc_gemm_generic": "pipipiiiip",
     "lc_gemm_bf16": "pppiiiiipp",
     "lc_gemm_bf16_supported": "iii",
+    "lc_gemm_bf16_force_tile": "i",
     "lc_qk_norm_rope_write": "piiiiippfppipppip",
     "lc_attention_generic": "pipppipppiiiiiifip",
     "lc_attn_bf16_supported": "iiii",
@@ -218,6 +219,12 @@ def _gemm_workspace(M: int, N: int, K: int, device) -> Optional[torch.Tensor]:
     """Float32 scratch for the products that cut K into shares (None when none is needed)."""
     words = library().lc_gemm_bf16_workspace(M, N, K)
     return torch.empty((words,), dtype=torch.float32, device=device) if words else None
+
+
+def force_gemm_tile(tile: int) -> None:
+    """Make the tiled bfloat16 product use one tile shape for every size (0: 64x128, 1: 128x128,
+    2: 256x128, 3: 256x256; -1: choose by size again).  For tests and tuning."""
+    _call("lc_gemm_bf16_force_tile", _c_int(tile))
 
 
 def _fast_gemm_ok(M: int, N: int, K: int) -> bool:

@@ -245,6 +245,32 @@ def test_gemm_bf16_matrix_cores(out_dtype, M, N, K):
     close(got, want, out_dtype, scale=K ** 0.5)
 
 
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("M,N,K", [(1, 16, 128), (70, 130, 128), (257, 300, 256), (300, 1000, 640),
+                                   (513, 257, 384), (64, 128, 1024), (1000, 520, 2048)])
+def test_gemm_bf16_every_tile_shape(tile, M, N, K):
+    """Each tile shape of the tiled kernel at sizes that leave ragged edges in both directions,
+    from two k-blocks (fewer than the ring of stages holds) to many; with and without the SwiGLU
+    epilogue, bfloat16 and float32 output."""
+    x = rnd(M, K, dtype=torch.bfloat16, seed=63)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=64)
+    assert ops._fast_gemm_ok(M, N, K)
+    ops.force_gemm_tile(tile)
+    try:
+        got16 = ops.gemm(x, w, torch.bfloat16)
+        got32 = ops.gemm(x, w, torch.float32)
+        fused = ops.gemm_swiglu(x, w[:N // 16 * 16]) if N >= 16 else None
+    finally:
+        ops.force_gemm_tile(-1)
+    close(got16, ref.gemm(x, w, torch.bfloat16), torch.bfloat16, scale=K ** 0.5)
+    close(got32, ref.gemm(x, w, torch.float32), torch.float32, scale=K ** 0.5)
+    if fused is not None:
+        full = x.double() @ w[:N // 16 * 16].double().T
+        blocks = full.view(M, -1, 2, 8)
+        g, u = blocks[:, :, 0, :].reshape(M, -1), blocks[:, :, 1, :].reshape(M, -1)
+        close(fused, (g / (1 + torch.exp(-g)) * u).to(torch.bfloat16), torch.bfloat16, scale=K ** 0.5)
+
+
 def test_gemm_bf16_one_hot_rows_and_columns():
     """x picks single columns of w: the product must return exactly those entries, so a wrong
     operand layout (rows, k order) shows as a wrong element, not as a small error."""
