@@ -26,8 +26,31 @@ template <typename TO> __device__ __forceinline__ void store_out(TO* p, float v)
 template <> __device__ __forceinline__ void store_out<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void store_out<bf16>(bf16* p, float v) { *p = static_cast<bf16>(v); }
 
-// silu(g) * u with silu(g) = g / (1 + exp(-g))   (reference: src/kernels/swiglu.cu:8,31-35)
-__device__ __forceinline__ float swiglu_f(float g, float u) { return g / (1.f + expf(-g)) * u; }
+// two adjacent elements in one store; p is aligned to the pair
+template <typename TO> __device__ __forceinline__ void store_pair(TO* p, float a, float b);
+template <> __device__ __forceinline__ void store_pair<float>(float* p, float a, float b) {
+    *reinterpret_cast<float2*>(p) = make_float2(a, b);
+}
+template <> __device__ __forceinline__ void store_pair<bf16>(bf16* p, float a, float b) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    bf16x2 v;
+    v[0] = static_cast<bf16>(a);
+    v[1] = static_cast<bf16>(b);
+    *reinterpret_cast<bf16x2*>(p) = v;
+}
+
+// the value of another lane of the same row of 16 lanes, by a DPP move: CTRL 0xB1 swaps
+// neighbours (lane ^ 1), 0x128 rotates the row by 8 (lane ^ 8).  All lanes must be active.
+template <int CTRL> __device__ __forceinline__ float lane_swap(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+// silu(g) * u with silu(g) = g / (1 + exp(-g))   (reference: src/kernels/swiglu.cu:8,31-35).
+// exp and the reciprocal are the hardware's single instructions (about one unit in the last
+// place each); the results of these products are rounded to bfloat16 afterwards.
+__device__ __forceinline__ float swiglu_f(float g, float u) {
+    return g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u;
+}
 
 // ------------------------------------------------------------------------------- skinny
 constexpr int SK_KBLOCK = 128; // k elements per wave iteration
@@ -331,28 +354,64 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
     for (; it + S - 1 < nk; ++it) block(it, std::true_type{});
     for (; it < nk; ++it) block(it, std::false_type{});
 
-    // acc[i][j][v]: row m = (v/4)*8 + (lane/32)*4 + v%4, column n = lane%32 of the 32x32 tile
+    // acc[i][j][v]: row m = (v/4)*8 + (lane/32)*4 + v%4, column n = lane%32 of the 32x32 tile.
+    const int mrow = m0 + wm + (lane >> 5) * 4;     // + i * 32 + (v / 4) * 8 + v % 4
+    const int ncol = n0 + wn + lr;                  // + j * 32
+    if (EPI == 1 && !SPLIT) {
+        // columns come in blocks of 16: 8 gate, then their 8 up (8 lanes further on).  Of two
+        // consecutive rows the gate lane finishes the first and the up lane the second.
+        const bool up = lr & 8;
+        const int ng = up ? ncol - 8 : ncol;
+        TO* dst = out + (size_t)(mrow + (up ? 1 : 0)) * (N / 2) + (size_t)(ng >> 4) * 8 + (ng & 7);
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int n = n0 + wn + j * 32 + lr;
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int m = m0 + wm + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
-                if (SPLIT) {
-                    if (m < M && n < N) part[((size_t)blockIdx.y * M + m) * N + n] = acc[i][j][v];
-                } else if (EPI == 0) {
-                    if (m < M && n < N) store_out<TO>(out + (size_t)m * N + n, acc[i][j][v]);
-                } else {
-                    // columns come in blocks of 16: 8 gate, then their 8 up (8 lanes further on)
-                    const float other = __shfl_xor(acc[i][j][v], 8, 64);
-                    if ((lr & 8) == 0 && m < M && n < N)
-                        store_out<TO>(out + (size_t)m * (N / 2) + (n >> 4) * 8 + (n & 7),
-                                      swiglu_f(acc[i][j][v], other));
+                for (int v = 0; v < 16; v += 2) {
+                    float first = acc[i][j][v], second = acc[i][j][v + 1];
+                    asm volatile("" : "+v"(first), "+v"(second));   // two values, not one indexed by `up`
+                    const float got = lane_swap<0x128>(up ? first : second);   // lane ^ 8
+                    const float r = swiglu_f(up ? got : first, up ? second : got);
+                    const int dm = i * 32 + (v >> 2) * 8 + (v & 3);
+                    if (mrow + (up ? 1 : 0) + dm < M && ng + j * 32 < N)
+                        store_out<TO>(dst + (size_t)dm * (N / 2) + j * 16, r);
                 }
-            }
+    } else {
+        using TS = typename std::conditional<SPLIT, float, TO>::type;
+        TS* base = SPLIT ? (TS*)(part + (size_t)blockIdx.y * M * N) : (TS*)out;
+        if ((N & 1) == 0) {
+            // neighbouring lanes swap every other value, so that a lane holds two adjacent
+            // columns of one row and stores them together: even lanes the even v, odd lanes the odd
+            const bool odd = lane & 1;
+            TS* dst = base + (size_t)(mrow + (odd ? 1 : 0)) * N + (ncol & ~1);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; v += 2) {
+                        float first = acc[i][j][v], second = acc[i][j][v + 1];
+                        asm volatile("" : "+v"(first), "+v"(second));   // two values, not one indexed by `odd`
+                        const float got = lane_swap<0xB1>(odd ? first : second);   // lane ^ 1
+                        const int dm = i * 32 + (v >> 2) * 8 + (v & 3);
+                        if (mrow + (odd ? 1 : 0) + dm < M && (ncol & ~1) + j * 32 < N)
+                            store_pair<TS>(dst + (size_t)dm * N + j * 32, odd ? got : first, odd ? second : got);
+                    }
+        } else {
+            TS* dst = base + (size_t)mrow * N + ncol;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int dm = i * 32 + (v >> 2) * 8 + (v & 3);
+                        if (mrow + dm < M && ncol + j * 32 < N)
+                            store_out<TS>(dst + (size_t)dm * N + j * 32, acc[i][j][v]);
+                    }
         }
+    }
 }
 
 // out = sum over the shares of part[s][M][N], added in the order of s; EPI as in the products
@@ -383,12 +442,12 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ part, TO* __restr
 
 // The tile shapes of the tiled kernel.  TILE_AUTO picks by size; the others are forced through
 // lc_gemm_bf16_force_tile (tests and tuning).
-enum : int { TILE_AUTO = -1, TILE_64x128 = 0, TILE_128x128 = 1, TILE_256x128 = 2, TILE_256x256 = 3, TILE_COUNT = 4 };
+enum : int { TILE_AUTO = -1, TILE_64x128 = 0, TILE_128x128 = 1, TILE_256x128 = 2, TILE_256x192 = 3, TILE_256x256 = 4, TILE_COUNT = 5 };
 static int g_force_tile = TILE_AUTO;
 constexpr int kCUs = 256;
 
 static int tile_bm(int t) { return t == TILE_64x128 ? 64 : t == TILE_128x128 ? 128 : 256; }
-static int tile_bn(int t) { return t == TILE_256x256 ? 256 : 128; }
+static int tile_bn(int t) { return t == TILE_256x256 ? 256 : t == TILE_256x192 ? 192 : 128; }
 static long long tile_count(int t, int M, int N) {
     return (long long)((M + tile_bm(t) - 1) / tile_bm(t)) * ((N + tile_bn(t) - 1) / tile_bn(t));
 }
@@ -399,7 +458,7 @@ static long long tile_count(int t, int M, int N) {
 static int pick_tile(int M, int N) {
     if (g_force_tile != TILE_AUTO) return g_force_tile;
     if (M <= 64) return TILE_64x128;
-    const double rate[TILE_COUNT] = {0.0, 0.87, 1.0, 1.2};
+    const double rate[TILE_COUNT] = {0.0, 0.87, 1.0, 1.1, 1.2};
     int best = TILE_128x128;
     double best_cost = 0.0;
     for (int t = TILE_128x128; t < TILE_COUNT; ++t) {
@@ -418,9 +477,9 @@ static int splitk_shares(int M, int N, int K) {
     const int t = pick_tile(M, N);
     if (t != TILE_64x128 && t != TILE_128x128) return 1;
     const long long tiles = tile_count(t, M, N);
-    if (tiles >= 200) return 1;
+    if (tiles >= 400) return 1;
     const int nk = K / TL_K;
-    int S = (int)((320 + tiles / 2) / tiles);
+    int S = (int)((480 + tiles / 2) / tiles);
     if (S > nk / 4) S = nk / 4;
     return S < 1 ? 1 : S;
 }
@@ -468,6 +527,7 @@ static int launch_bf16(const bf16* x, const bf16* w, TO* out, float* workspace, 
     case TILE_64x128:  return launch_tiled<64, 128, 4, EPI, TO>(x, w, out, workspace, M, N, K, shares, s);
     case TILE_128x128: return launch_tiled<128, 128, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, s);
     case TILE_256x128: return launch_tiled<256, 128, 3, EPI, TO>(x, w, out, workspace, M, N, K, shares, s);
+    case TILE_256x192: return launch_tiled<256, 192, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, s);
     default:           return launch_tiled<256, 256, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, s);
     }
 }
@@ -508,6 +568,7 @@ LC_API int lc_gemm_bf16(const void* x, const void* w, void* out, int out_dt, int
              "(K must be a multiple of %d)", M, N, K, SK_KBLOCK);
     LC_CHECK(x && w && out, "gemm_bf16: null pointer");
     LC_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_bf16: operands must be 16-byte aligned");
+    LC_CHECK((uintptr_t)out % 8 == 0 && (uintptr_t)workspace % 8 == 0, "gemm_bf16: out and workspace must be 8-byte aligned");
     LC_CHECK(epilogue == 0 || (epilogue == 1 && N % 16 == 0),
              "gemm_bf16: the SwiGLU epilogue needs N (%d) to be a multiple of 16", N);
     const bf16* xb = (const bf16*)x;
