@@ -518,7 +518,12 @@ template <int EPI, typename TO>
 static int launch_bf16(const bf16* x, const bf16* w, TO* out, float* workspace, int M, int N, int K,
                        hipStream_t s) {
     if (M <= 16 && g_force_tile == TILE_AUTO) {
-        launch_skinny<1, 1, 16, 2, EPI, TO>(x, w, out, M, N, K, s);
+        // measured: with one or two rows of x a deeper unroll keeps more of w in flight; from
+        // about 12 rows on, x costs as much to fetch as w, and two row tiles per workgroup
+        // share it (only where that still leaves every CU two workgroups)
+        if (M <= 2) launch_skinny<1, 1, 16, 4, EPI, TO>(x, w, out, M, N, K, s);
+        else if (M >= 12 && N >= 32 * 2 * kCUs) launch_skinny<1, 2, 16, 2, EPI, TO>(x, w, out, M, N, K, s);
+        else launch_skinny<1, 1, 16, 2, EPI, TO>(x, w, out, M, N, K, s);
         LC_LAUNCH_CHECK("gemm_skinny");
         return 0;
     }

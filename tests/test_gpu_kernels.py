@@ -235,7 +235,8 @@ def test_sampling_follows_the_distribution():
 @pytest.mark.parametrize("M,N,K", [(1, 16, 128), (8, 100, 256), (17, 4096, 1024), (64, 331, 384),
                                    (65, 128, 128), (128, 257, 512), (300, 1000, 640), (2048, 512, 1024),
                                    (3, 151936 // 8, 256), (33, 4096, 4096), (64, 6144, 1024), (48, 100, 128),
-                                   (20, 24576, 256), (600, 3000, 256)])
+                                   (20, 24576, 256), (600, 3000, 256), (2, 331, 512), (13, 16400, 256),
+                                   (16, 24576, 128), (12, 16384, 2048)])
 def test_gemm_bf16_matrix_cores(out_dtype, M, N, K):
     x = rnd(M, K, dtype=torch.bfloat16, seed=60)
     w = rnd(N, K, dtype=torch.bfloat16, seed=61)
@@ -306,7 +307,8 @@ def test_attention_bf16_long_contexts(nh, nkv, d, window):
 
 
 @pytest.mark.parametrize("M,I,K", [(1, 16, 128), (8, 200, 256), (33, 1000, 128), (64, 96, 384), (65, 136, 256),
-                                   (300, 520, 128), (2048, 256, 256), (40, 2048, 1024), (64, 12288, 512)])
+                                   (300, 520, 128), (2048, 256, 256), (40, 2048, 1024), (64, 12288, 512),
+                                   (2, 72, 640), (14, 8200, 256), (16, 8192, 128)])
 def test_gemm_with_swiglu_epilogue(M, I, K):
     """gate and up interleaved in blocks of 8 rows, silu(gate) * up formed in the epilogue."""
     x = rnd(M, K, dtype=torch.bfloat16, seed=80, scale=0.5)
