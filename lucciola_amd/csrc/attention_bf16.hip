@@ -257,10 +257,10 @@ __global__ __launch_bounds__(128) void attn_decode_join_kernel(const float* __re
 // rows [32 (w % 2), +32) as two column tiles; HPW = 1: wave w works on rows [16 w, +16).
 // Key rows are padded by 16 bytes in LDS, which spreads the 16 keys of an operand read over
 // all banks.
-constexpr int PF_NP = 2;
+constexpr int PF_NP = 4;
 
 template <int D, int HPW>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
+__global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     const bf16* __restrict__ qkv, int q_stride, const bf16* __restrict__ k_cache,
     const bf16* __restrict__ v_cache, bf16* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ block_table, int max_blocks, int nh, int nkv, float scale_log2,
@@ -390,10 +390,15 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                 for (int v = 0; v < 4; ++v) mx = fmaxf(mx, sc[c][n][v]);
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            // maxima are kept as raw scores; p = 2^((s - m) scale_log2), one fma and one v_exp
-            const float m_new = fmaxf(st.m[c], mx);
+            // Maxima are kept as raw scores; p = 2^((s - m) scale_log2), one fma and one v_exp.
+            // m is a reference point, not necessarily the maximum: it moves (and the sums are
+            // rescaled) only when a score would exceed it by more than 2^8, which keeps every p
+            // in range and makes rescaling rare.  The result sum p v / sum p is the same for
+            // any reference; the choice is made per query row from that row's scores alone.
+            const bool move = mx * scale_log2 > st.m[c] * scale_log2 + 8.f;   // true while m is -inf
+            const float m_new = move ? mx : st.m[c];
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            alpha[c] = __builtin_amdgcn_exp2f((st.m[c] - m_use) * scale_log2);   // 2^-inf = 0 at the start
+            alpha[c] = move ? __builtin_amdgcn_exp2f((st.m[c] - m_use) * scale_log2) : 1.f;   // 2^-inf = 0 at the start
             const float neg = -m_use * scale_log2;
             float psum = 0.f;
 #pragma unroll
@@ -406,7 +411,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                 }
             st.l[c] = st.l[c] * alpha[c] + psum;
             st.m[c] = m_new;
-            rescale = rescale || alpha[c] != 1.f;
+            rescale = rescale || move;
         }
         if (__any(rescale)) {
 #pragma unroll

@@ -149,13 +149,17 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
     h_ctx = pk.add(ctx_len)
     decode_tokens = [q_start[r] for r in range(R) if q_start[r + 1] - q_start[r] == 1]
     h_dec = pk.add(decode_tokens)
-    tiles: List[int] = []
+    tile_list: List[Tuple[int, int, int, int]] = []
     for r in range(R):
         n = q_start[r + 1] - q_start[r]
         if n == 1:
             continue
         for t0 in range(0, n, PREFILL_TILE):
-            tiles.extend((r, q_start[r] + t0, min(PREFILL_TILE, n - t0), first_pos[r] + t0))
+            tile_list.append((r, q_start[r] + t0, min(PREFILL_TILE, n - t0), first_pos[r] + t0))
+    # the tiles that see the most keys first: workgroups start in this order, and the longest
+    # ones set the kernel's time (the order changes no tile's result)
+    tile_list.sort(key=lambda t: -(t[3] + t[2]))
+    tiles: List[int] = [v for t in tile_list for v in t]
     h_tiles = pk.add(tiles)
 
     group_handles = []
