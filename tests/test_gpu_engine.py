@@ -60,6 +60,60 @@ def test_replay_families(dtype, key, family):
         assert g.pool.num_free() == blocks
 
 
+def random_configuration(seed):
+    """A configuration drawn at random from what config.json allows: any number of heads and
+    groups, head sizes in steps of 16, widths, feed-forward sizes and vocabularies that are odd
+    or not, windows on some layers, any page size."""
+    import random
+    rng = random.Random(1000 + seed)
+    layers = rng.randint(1, 4)
+    kv = rng.choice([1, 2, 3, 4])
+    group = rng.choice([1, 2, 3, 4, 5, 6, 8])
+    cfg = {
+        "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+        "num_hidden_layers": layers, "hidden_size": rng.choice([24, 40, 75, 100, 136, 200]),
+        "num_attention_heads": kv * group, "num_key_value_heads": kv,
+        "head_dim": rng.choice([16, 32, 48, 64, 80, 96, 112, 128]),
+        "intermediate_size": rng.choice([16, 57, 88, 130, 256, 301]),
+        "vocab_size": rng.randint(50, 700),
+        "rope_theta": rng.choice([10000.0, 50000.0, 1000000.0]),
+        "rms_norm_eps": rng.choice([1e-6, 3e-6, 1e-5]),
+        "tie_word_embeddings": rng.random() < 0.5, "max_position_embeddings": 4096,
+        "initializer_range": rng.choice([0.02, 0.05]), "hidden_act": "silu",
+    }
+    if rng.random() < 0.5:
+        cfg["sliding_window"] = rng.randint(5, 40)
+        cfg["use_sliding_window"] = True
+        cfg["layer_types"] = [rng.choice(["full_attention", "sliding_attention"]) for _ in range(layers)]
+        if "sliding_attention" not in cfg["layer_types"]:
+            cfg["layer_types"][rng.randrange(layers)] = "sliding_attention"
+    page = rng.choice([4, 8, 16, 32])
+    lengths = [rng.randint(1, 150) for _ in range(5)]
+    return cfg, page, lengths
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(8))
+def test_random_configurations(seed, dtype):
+    """Configurations drawn at random, replayed mixed (pages used again) and with a decoded
+    tail: sizes that no fixed test names must give right results too, through whichever kernel
+    takes them."""
+    cfg, page, lengths = random_configuration(seed)
+    weights = random_weights(cfg, seed)
+    prompts = prompts_for(cfg, lengths, seed)
+    refs = {n: plain_qwen3.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    for family in (traces.mixed, traces.tail_decode):
+        steps = family(prompts)
+        blocks = traces.max_live_tokens(steps, page) // page
+        runner = make_runner(cfg, weights, page, blocks, dtype, DEV)
+        got = replay(runner, steps)
+        assert len(got) == sum(len(p) for p in prompts.values())
+        worst = compare(got, cfg, weights, prompts, TOL[dtype], refs)
+        print(f"seed {seed} {family.__name__} {dtype}: {cfg['num_attention_heads']} heads of "
+              f"{cfg['head_dim']} in {cfg['num_key_value_heads']} groups, width {cfg['hidden_size']}, "
+              f"page {page}: worst relative error {worst:.3e}")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_pages_reused_with_stale_contents(dtype):
     """Requests run one after the other in a pool that holds only one of them, after the pool
