@@ -143,16 +143,35 @@ __device__ __forceinline__ void attend_range(AttnState<D, QT>& st, const bf16x8 
 }
 
 // ------------------------------------------------------------------------------- decode
+// What the decode kernel does to the raw q, k, v of its token before it attends, when the
+// step has no separate kernel for it: RMSNorm over the head (weights optional), rotary
+// embedding of the first `rot` entries (table optional: row p holds rot/2 cosines, then rot/2
+// sines), and, if write_kv, the token's k and v into their place in the cache.  The formulas
+// and their order are those of the separate kernel (elementwise.hip, qk_norm_rope_write).
+struct DecodePrologue {
+    const float* q_w;
+    const float* k_w;
+    const float* rope;
+    float eps;
+    int rot;
+    int write_kv;
+    int enabled;
+};
+
+// Every workgroup prepares the q heads of its group itself (into LDS); the one whose share of
+// the pages holds the token's own position also prepares k and v and writes them to the
+// cache before anyone in the workgroup reads that page.
 template <int D>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
-    const bf16* __restrict__ qkv, int q_stride, const bf16* __restrict__ k_cache,
-    const bf16* __restrict__ v_cache, bf16* __restrict__ out, float* __restrict__ part_o,
+    const bf16* __restrict__ qkv, int q_stride, bf16* k_cache, bf16* v_cache,
+    bf16* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const int* __restrict__ decode_tokens,
     const int* __restrict__ tok_req, const int* __restrict__ positions,
     const int* __restrict__ block_table, int max_blocks, int nh, int nkv, float scale_log2,
-    int window, int splits) {
+    int window, int splits, DecodePrologue pro) {
     __shared__ float sm_o[4][D * 16];
     __shared__ float sm_m[4][16], sm_l[4][16];
+    __shared__ __attribute__((aligned(16))) bf16 sm_q[16 * D];
 
     const int split = blockIdx.x, kvh = blockIdx.y, di = blockIdx.z;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -168,7 +187,53 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const int* table = block_table + (size_t)req * max_blocks;
 
     bf16x8 bq[1][D / 32];
-    {
+    if (pro.enabled) {
+        const bool owner = pro.write_kv && begin <= last_page && last_page < end;
+        const int ntask = G + (owner ? 2 : 0);            // the q heads, then k, then v
+        const int half = pro.rot / 2;
+        const float* cs = pro.rope ? pro.rope + (size_t)p * pro.rot : nullptr;
+        const bf16* row = qkv + (size_t)t * q_stride;
+        for (int task = wave; task < ntask; task += 4) {
+            if (task == G + 1) {                          // v: copied, transposed into the page
+                const bf16* x = row + (size_t)(nh + nkv + kvh) * D;
+                bf16* col = v_cache + ((size_t)table[last_page] * nkv + kvh) * D * PAGE + (p % PAGE);
+                for (int i = lane; i < D; i += 64) col[(size_t)i * PAGE] = x[i];
+                continue;
+            }
+            const bool is_k = task == G;
+            const bf16* x = row + (size_t)(is_k ? nh + kvh : kvh * G + task) * D;
+            const float* w = is_k ? pro.k_w : pro.q_w;
+            bf16* dst = is_k ? k_cache + (((size_t)table[last_page] * nkv + kvh) * PAGE + (p % PAGE)) * D
+                             : sm_q + task * D;
+            float inv = 1.f;
+            if (w) {
+                float ss = 0.f;
+                for (int i = lane; i < D; i += 64) {
+                    const float v = static_cast<float>(x[i]);
+                    ss += v * v;
+                }
+                ss = wave_sum(ss);
+                inv = rsqrtf(ss / (float)D + pro.eps);
+            }
+            for (int i = lane; i < half; i += 64) {
+                float a = static_cast<float>(x[i]) * inv, b = static_cast<float>(x[i + half]) * inv;
+                if (w) { a *= w[i]; b *= w[i + half]; }
+                float c = 1.f, sn = 0.f;
+                if (cs) { c = cs[i]; sn = cs[half + i]; }
+                dst[i] = static_cast<bf16>(a * c - b * sn);
+                dst[i + half] = static_cast<bf16>(a * sn + b * c);
+            }
+            for (int i = pro.rot + lane; i < D; i += 64) {
+                float a = static_cast<float>(x[i]) * inv;
+                if (w) a *= w[i];
+                dst[i] = static_cast<bf16>(a);
+            }
+        }
+        __syncthreads();      // q is in LDS; the owner's k and v have reached memory
+        const bf16* qrow = sm_q + min(q, G - 1) * D + kg * 8;
+#pragma unroll
+        for (int i = 0; i < D / 32; ++i) bq[0][i] = *reinterpret_cast<const bf16x8*>(qrow + i * 32);
+    } else {
         const bf16* qrow = qkv + (size_t)t * q_stride + (size_t)(kvh * G + min(q, G - 1)) * D + kg * 8;
 #pragma unroll
         for (int i = 0; i < D / 32; ++i) bq[0][i] = *reinterpret_cast<const bf16x8*>(qrow + i * 32);
@@ -453,14 +518,15 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
 }
 
 template <int D>
-static int launch_decode(const bf16* qkv, int q_stride, const bf16* k, const bf16* v, bf16* out,
+static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* out,
                          float* part_o, float* part_ml, const int* decode_tokens, const int* tok_req,
                          const int* positions, const int* table, int max_blocks, int ND, int nh,
-                         int nkv, float scale_log2, int window, int splits, hipStream_t s) {
+                         int nkv, float scale_log2, int window, int splits, DecodePrologue pro,
+                         hipStream_t s) {
     dim3 grid(splits, nkv, ND);
     attn_decode_kernel<D><<<grid, 256, 0, s>>>(qkv, q_stride, k, v, out, part_o, part_ml,
                                                decode_tokens, tok_req, positions, table, max_blocks,
-                                               nh, nkv, scale_log2, window, splits);
+                                               nh, nkv, scale_log2, window, splits, pro);
     LC_LAUNCH_CHECK("attn_decode");
     if (splits > 1) {
         attn_decode_join_kernel<D><<<dim3(ND, nh), 128, 0, s>>>(
@@ -517,12 +583,20 @@ LC_API int lc_attn_decode_splits(int num_decode, int nkv, int max_ctx) {
         default: LC_CHECK(false, "attention_bf16: head size %d has no matrix-core kernel", d); \
     }
 
-LC_API int lc_attn_decode_bf16(const void* qkv, int q_stride, const void* k_cache, const void* v_cache,
+// prologue != 0: qkv holds the raw projections; the kernel norms and rotates q and k itself
+// (q_w, k_w, rope_table may be null; rot entries of a head rotate) and, if write_kv != 0, writes
+// the tokens' k and v to the cache.  Otherwise qkv is ready and the cache holds the tokens.
+LC_API int lc_attn_decode_bf16(const void* qkv, int q_stride, void* k_cache, void* v_cache,
                                void* out, float* part_o, float* part_ml, const int* decode_tokens,
                                const int* tok_req, const int* positions, const int* block_table,
                                int max_blocks, int num_decode, int nh, int nkv, int d, int page_size,
-                               float scale, int window, int splits, hipStream_t stream) {
+                               float scale, int window, int splits, int prologue, const float* q_w,
+                               const float* k_w, float eps, const float* rope_table, int rot,
+                               int write_kv, hipStream_t stream) {
     if (num_decode == 0) return 0;
+    LC_CHECK(!prologue || (rot >= 0 && rot <= d && rot % 2 == 0 && (q_w == nullptr) == (k_w == nullptr)),
+             "attn_decode_bf16: bad prologue (rot=%d of %d)", rot, d);
+    DecodePrologue pro = {q_w, k_w, rope_table, eps, rope_table ? rot : 0, write_kv, prologue};
     LC_CHECK(lc_attn_bf16_supported(nh, nkv, d, page_size),
              "attn_decode_bf16: unsupported sizes nh=%d nkv=%d d=%d page=%d", nh, nkv, d, page_size);
     LC_CHECK(qkv && k_cache && v_cache && out && decode_tokens && tok_req && positions && block_table,
@@ -531,9 +605,9 @@ LC_API int lc_attn_decode_bf16(const void* qkv, int q_stride, const void* k_cach
              "attn_decode_bf16: %d shares need a workspace", splits);
     LC_CHECK(q_stride % 8 == 0 && (uintptr_t)qkv % 16 == 0, "attn_decode_bf16: q must be 16-byte aligned");
     const float sl2 = scale * 1.4426950408889634f;
-#define CALL(DD) launch_decode<DD>((const bf16*)qkv, q_stride, (const bf16*)k_cache, (const bf16*)v_cache, \
+#define CALL(DD) launch_decode<DD>((const bf16*)qkv, q_stride, (bf16*)k_cache, (bf16*)v_cache,             \
         (bf16*)out, part_o, part_ml, decode_tokens, tok_req, positions, block_table, max_blocks,           \
-        num_decode, nh, nkv, sl2, window, splits, stream)
+        num_decode, nh, nkv, sl2, window, splits, pro, stream)
     LC_DISPATCH_D(d, CALL)
 #undef CALL
     return 0;

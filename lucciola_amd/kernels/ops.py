@@ -33,7 +33,7 @@ _SIGNATURES = {
     "lc_attention_generic": "pipppipppiiiiiifip",
     "lc_attn_bf16_supported": "iiii",
     "lc_attn_decode_splits": "iii",
-    "lc_attn_decode_bf16": "pippppppppp" + "iiiiii" + "f" + "ii" + "p",
+    "lc_attn_decode_bf16": "pippppppppp" + "iiiiii" + "f" + "ii" + "ippfpii" + "p",
     "lc_attn_prefill_bf16": "pippppp" + "iiiiii" + "f" + "i" + "p",
     "lc_swiglu": "ppiiip",
     "lc_sample": "pppppiip",
@@ -308,11 +308,26 @@ class AttentionBatch:
     all_decode: bool = False
 
 
+@dataclass
+class QKPrologue:
+    """What has to happen to the raw q, k, v of a step before attention: RMSNorm of every q and
+    k head (weights may be None), rotary embedding (table may be None), and the write of k and
+    v to the cache slots (``slots`` None: no write, another site owns the cache)."""
+
+    q_weight: Optional[torch.Tensor]
+    k_weight: Optional[torch.Tensor]
+    eps: float
+    rope_table: Optional[torch.Tensor]
+    slots: Optional[torch.Tensor]
+
+
 def attention(qkv: torch.Tensor, batch: AttentionBatch, k_cache: torch.Tensor,
               v_cache: torch.Tensor, nh: int, nkv: int, d: int, page_size: int, scale: float,
-              window: int = 0) -> torch.Tensor:
+              window: int = 0, prologue: Optional[QKPrologue] = None) -> torch.Tensor:
     """Causal attention of the q heads in ``qkv`` [T, (nh + 2 nkv) d] over the cached keys and
-    values (the step's own have been written already) -> [T, nh d]."""
+    values -> [T, nh d].  Without ``prologue`` the step's own keys and values have been written
+    already and q is ready; with it, ``qkv`` is raw: a step of single tokens does the prologue
+    inside the decode kernel, any other step runs :func:`qk_norm_rope_write` first."""
     _need(qkv, "qkv", None, 2)
     _need(k_cache, "k cache", qkv.dtype, 4)
     _need(v_cache, "v cache", qkv.dtype, 4)
@@ -325,9 +340,14 @@ def attention(qkv: torch.Tensor, batch: AttentionBatch, k_cache: torch.Tensor,
     _need(batch.block_table, "block table", torch.int32, 2)
     _check_caches(k_cache, v_cache, nkv, page_size, d)
     lib = library()
-    if qkv.dtype == torch.bfloat16 and batch.decode_tokens is not None \
-            and batch.prefill_tiles is not None \
-            and lib.lc_attn_bf16_supported(nh, nkv, d, page_size):
+    fast = (qkv.dtype == torch.bfloat16 and batch.decode_tokens is not None
+            and batch.prefill_tiles is not None and lib.lc_attn_bf16_supported(nh, nkv, d, page_size))
+    in_kernel = fast and prologue is not None and batch.num_decode == T
+    if prologue is not None and not in_kernel:
+        qk_norm_rope_write(qkv, nh, nkv, d, prologue.q_weight, prologue.k_weight, prologue.eps,
+                           batch.positions, prologue.rope_table, k_cache, v_cache, prologue.slots,
+                           page_size)
+    if fast:
         mb = batch.block_table.shape[1]
         nd = batch.num_decode
         if nd > 0:
@@ -336,10 +356,19 @@ def attention(qkv: torch.Tensor, batch: AttentionBatch, k_cache: torch.Tensor,
             if splits > 1:
                 part_o = torch.empty((nd * nh * splits * d,), dtype=torch.float32, device=qkv.device)
                 part_ml = torch.empty((nd * nh * splits * 2,), dtype=torch.float32, device=qkv.device)
+            rope = prologue.rope_table if in_kernel else None
+            if rope is not None:
+                _need(rope, "rotary table", torch.float32, 2)
             _call("lc_attn_decode_bf16", _ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
                   _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(batch.decode_tokens),
                   _ptr(batch.tok_req), _ptr(batch.positions), _ptr(batch.block_table), mb, nd, nh,
-                  nkv, d, page_size, scale, window, splits, _stream())
+                  nkv, d, page_size, scale, window, splits,
+                  1 if in_kernel else 0,
+                  _ptr(prologue.q_weight if in_kernel else None),
+                  _ptr(prologue.k_weight if in_kernel else None),
+                  _c_float(prologue.eps if in_kernel else 0.0), _ptr(rope),
+                  rope.shape[1] if rope is not None else 0,
+                  1 if in_kernel and prologue.slots is not None else 0, _stream())
         nt = batch.prefill_tiles.shape[0]
         if nt > 0:
             _call("lc_attn_prefill_bf16", _ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),

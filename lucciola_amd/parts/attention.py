@@ -83,9 +83,7 @@ class Attention(Part):
             if table is None:
                 self.position.apply(qkv, self.nh, self.nkv, self.d, attn.positions)
         k_cache, v_cache = site.kv
-        ops.qk_norm_rope_write(qkv, self.nh, self.nkv, self.d, q_w, k_w, eps, attn.positions, table,
-                               k_cache, v_cache, attn.slots if site.writes_cache else None,
-                               site.page_size)
+        prologue = ops.QKPrologue(q_w, k_w, eps, table, attn.slots if site.writes_cache else None)
         o = ops.attention(qkv, attn, k_cache, v_cache, self.nh, self.nkv, self.d, site.page_size,
-                          self.scale, self.window or 0)
+                          self.scale, self.window or 0, prologue)
         return ops.gemm(o, self.o, self.dtype)

@@ -67,7 +67,11 @@ def qk_norm_rope_write(qkv, nh, nkv, d, q_weight, k_weight, eps, positions, rope
             v_cache[page, :, :, off] = v[t]
 
 
-def attention(qkv, batch, k_cache, v_cache, nh, nkv, d, page_size, scale, window=0):
+def attention(qkv, batch, k_cache, v_cache, nh, nkv, d, page_size, scale, window=0, prologue=None):
+    if prologue is not None:
+        qk_norm_rope_write(qkv, nh, nkv, d, prologue.q_weight, prologue.k_weight, prologue.eps,
+                           batch.positions, prologue.rope_table, k_cache, v_cache, prologue.slots,
+                           page_size)
     T = qkv.shape[0]
     q = qkv.view(T, nh + 2 * nkv, d)[:, :nh].to(F64)
     out = torch.zeros(T, nh, d, dtype=F64, device=qkv.device)

@@ -306,6 +306,45 @@ def test_attention_bf16_long_contexts(nh, nkv, d, window):
     close(got, want, torch.bfloat16, atol=attention_atol(torch.bfloat16, vc))
 
 
+@pytest.mark.parametrize("nh,nkv,d,window,rot,normed", [(32, 8, 128, 0, 128, True), (6, 2, 96, 24, 96, True),
+                                                        (8, 1, 64, 0, 32, False), (4, 4, 32, 0, 0, True),
+                                                        (16, 1, 32, 0, 32, True)])
+def test_attention_decode_with_prologue_in_the_kernel(nh, nkv, d, window, rot, normed):
+    """A step of single tokens with raw q, k, v: the decode kernel norms, rotates and writes
+    the cache itself.  Output and cache must equal those of the separate kernel followed by
+    the plain decode kernel, for short and long contexts (one or many shares of the pages),
+    a token at a page's first and last place, part of the head rotated or none."""
+    lengths = [1, 16, 17, 300, 2049, 5000, 33]
+    qkv, batch, kc, vc = paged_case(lengths, [1] * len(lengths), nh, nkv, d, 16, torch.bfloat16, seed=90)
+    assert ops.library().lc_attn_bf16_supported(nh, nkv, d, 16)
+    qw = (1 + 0.1 * rnd(d, seed=91)) if normed else None
+    kw = (1 + 0.1 * rnd(d, seed=92)) if normed else None
+    table = None
+    if rot:
+        ang = torch.arange(6000, dtype=torch.float64)[:, None] * (10000.0 ** (-torch.arange(rot // 2, dtype=torch.float64) * 2 / rot))
+        table = torch.cat([ang.cos(), ang.sin()], 1).float().to(DEV)
+    slots = torch.tensor([int(batch.block_table[r, (n - 1) // 16]) * 16 + (n - 1) % 16
+                          for r, n in enumerate(lengths)], dtype=torch.int32, device=DEV)
+    # separately
+    qkv1, kc1, vc1 = qkv.clone(), kc.clone(), vc.clone()
+    ops.qk_norm_rope_write(qkv1, nh, nkv, d, qw, kw, 1e-6, batch.positions, table, kc1, vc1, slots, 16)
+    want = ops.attention(qkv1, batch, kc1, vc1, nh, nkv, d, 16, d ** -0.5, window)
+    # in the kernel
+    qkv2, kc2, vc2 = qkv.clone(), kc.clone(), vc.clone()
+    got = ops.attention(qkv2, batch, kc2, vc2, nh, nkv, d, 16, d ** -0.5, window,
+                        ops.QKPrologue(qw, kw, 1e-6, table, slots))
+    assert torch.equal(qkv2, qkv)                       # raw input untouched
+    assert torch.equal(kc2, kc1) and torch.equal(vc2, vc1)
+    close(got, want, torch.bfloat16, atol=attention_atol(torch.bfloat16, vc1))
+    assert float((got.float() - want.float()).abs().max()) <= 2.0 ** -7 * float(want.float().abs().max())
+    # no cache write asked for: the cache stays as it was, q is still prepared
+    kc3, vc3 = kc1.clone(), vc1.clone()
+    got3 = ops.attention(qkv.clone(), batch, kc3, vc3, nh, nkv, d, 16, d ** -0.5, window,
+                         ops.QKPrologue(qw, kw, 1e-6, table, None))
+    assert torch.equal(kc3, kc1) and torch.equal(vc3, vc1)
+    close(got3, want, torch.bfloat16, atol=attention_atol(torch.bfloat16, vc1))
+
+
 @pytest.mark.parametrize("M,I,K", [(1, 16, 128), (8, 200, 256), (33, 1000, 128), (64, 96, 384), (65, 136, 256),
                                    (300, 520, 128), (2048, 256, 256), (40, 2048, 1024), (64, 12288, 512),
                                    (2, 72, 640), (14, 8200, 256), (16, 8192, 128)])
