@@ -14,6 +14,7 @@ code only; the tensors are made by :meth:`CacheManager.allocate_tensors`.
 """
 from __future__ import annotations
 
+from array import array
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
@@ -32,7 +33,8 @@ class PageGroup:
     spec: PagedKV
     sites: List[int]
     pool: PagePool
-    tables: Dict[Hashable, List[int]] = field(default_factory=dict)  # -1: given back
+    # a request's page ids in order, as a typed array (numpy views it without a copy); -1: given back
+    tables: Dict[Hashable, array] = field(default_factory=dict)
 
 
 @dataclass
@@ -113,7 +115,7 @@ class CacheManager:
         slot = self.slots.allocate()
         self.requests[request] = RequestState(slot)
         for g in self.groups:
-            g.tables[request] = []
+            g.tables[request] = array("i")
         return slot
 
     def can_admit(self) -> bool:
@@ -184,7 +186,7 @@ class CacheManager:
 
     # ------------------------------------------------------------------ views for a step
     def block_table(self, group_index: int, request: Hashable) -> List[int]:
-        return self.groups[group_index].tables[request]
+        return list(self.groups[group_index].tables[request])
 
     def slot_of_token(self, group_index: int, request: Hashable, position: int) -> int:
         page = self.groups[group_index].tables[request][position // self.block_size]

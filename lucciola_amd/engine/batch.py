@@ -109,33 +109,62 @@ class _Packer:
 
 
 def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
-                pad_blocks: Optional[int] = None, into: Optional[torch.Tensor] = None) -> StepBatch:
+                pad_blocks: Optional[int] = None, into: Optional[torch.Tensor] = None,
+                refresh_only: bool = False) -> Optional[StepBatch]:
     """Lay the entries out as one flat batch.  Pages for the new tokens must be reserved.
 
     ``pad_blocks``: width of the block tables (at least the longest table), so that batches of
-    the same make-up have the same layout; ``into``: the buffer of such an earlier batch."""
+    the same make-up have the same layout; ``into``: the buffer of such an earlier batch;
+    ``refresh_only``: only bring that buffer up to date (its views exist already), return None."""
     bs = cache.block_size
-    requests, q_start, first_pos, slot_list = [], [0], [], []
-    token_parts, position_parts, req_parts = [], [], []
-    want_rows: List[int] = []
-    for r, e in enumerate(entries):
-        n = len(e.tokens)
-        base = cache.length(e.request)
-        requests.append(e.request)
-        first_pos.append(base)
-        slot_list.append(cache.slot(e.request))
-        for w in e.want:
-            if not 0 <= int(w) < n:
-                raise ValueError(f"request {e.request!r}: wanted place {w} is outside its {n} tokens")
-            want_rows.append(q_start[-1] + int(w))
-        token_parts.append(np.asarray(e.tokens, dtype=np.int32))
-        position_parts.append(np.arange(base, base + n, dtype=np.int32))
-        req_parts.append(np.full(n, r, dtype=np.int32))
-        q_start.append(q_start[-1] + n)
-    T, R = q_start[-1], len(entries)
-    token_ids = np.concatenate(token_parts) if token_parts else np.zeros(0, np.int32)
-    positions = np.concatenate(position_parts) if position_parts else np.zeros(0, np.int32)
-    tok_req = np.concatenate(req_parts) if req_parts else np.zeros(0, np.int32)
+    R = len(entries)
+    requests = [e.request for e in entries]
+    first_pos = [cache.length(req) for req in requests]
+    slot_list = [cache.slot(req) for req in requests]
+    single = all(len(e.tokens) == 1 and len(e.want) == 1 and int(e.want[0]) == 0 for e in entries)
+    if single:
+        # a step of single tokens, each wanting its logits: everything is one array operation
+        T = R
+        q_start = list(range(R + 1))
+        token_ids = np.fromiter((e.tokens[0] for e in entries), dtype=np.int32, count=R)
+        positions = np.asarray(first_pos, dtype=np.int32)
+        tok_req = np.arange(R, dtype=np.int32)
+        want_rows = tok_req
+        ctx_len = positions + 1
+        decode_tokens = tok_req
+        tiles: List[int] = []
+    else:
+        q_start = [0]
+        token_parts, position_parts, req_parts = [], [], []
+        want_rows = []
+        for r, e in enumerate(entries):
+            n = len(e.tokens)
+            base = first_pos[r]
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise ValueError(f"request {e.request!r}: wanted place {w} is outside its {n} tokens")
+                want_rows.append(q_start[-1] + int(w))
+            token_parts.append(np.asarray(e.tokens, dtype=np.int32))
+            position_parts.append(np.arange(base, base + n, dtype=np.int32))
+            req_parts.append(np.full(n, r, dtype=np.int32))
+            q_start.append(q_start[-1] + n)
+        T = q_start[-1]
+        token_ids = np.concatenate(token_parts) if token_parts else np.zeros(0, np.int32)
+        positions = np.concatenate(position_parts) if position_parts else np.zeros(0, np.int32)
+        tok_req = np.concatenate(req_parts) if req_parts else np.zeros(0, np.int32)
+        ctx_len = [first_pos[r] + (q_start[r + 1] - q_start[r]) for r in range(R)]
+        decode_tokens = [q_start[r] for r in range(R) if q_start[r + 1] - q_start[r] == 1]
+        tile_list: List[Tuple[int, int, int, int]] = []
+        for r in range(R):
+            n = q_start[r + 1] - q_start[r]
+            if n == 1:
+                continue
+            for t0 in range(0, n, PREFILL_TILE):
+                tile_list.append((r, q_start[r] + t0, min(PREFILL_TILE, n - t0), first_pos[r] + t0))
+        # the tiles that see the most keys first: workgroups start in this order, and the
+        # longest ones set the kernel's time (the order changes no tile's result)
+        tile_list.sort(key=lambda t: -(t[3] + t[2]))
+        tiles = [v for t in tile_list for v in t]
 
     pk = _Packer()
     h_tok = pk.add(token_ids)
@@ -144,25 +173,13 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
     h_want = pk.add(want_rows)
     h_slot = pk.add(slot_list)
     h_qs = pk.add(q_start)
-
-    ctx_len = [first_pos[r] + (q_start[r + 1] - q_start[r]) for r in range(R)]
     h_ctx = pk.add(ctx_len)
-    decode_tokens = [q_start[r] for r in range(R) if q_start[r + 1] - q_start[r] == 1]
     h_dec = pk.add(decode_tokens)
-    tile_list: List[Tuple[int, int, int, int]] = []
-    for r in range(R):
-        n = q_start[r + 1] - q_start[r]
-        if n == 1:
-            continue
-        for t0 in range(0, n, PREFILL_TILE):
-            tile_list.append((r, q_start[r] + t0, min(PREFILL_TILE, n - t0), first_pos[r] + t0))
-    # the tiles that see the most keys first: workgroups start in this order, and the longest
-    # ones set the kernel's time (the order changes no tile's result)
-    tile_list.sort(key=lambda t: -(t[3] + t[2]))
-    tiles: List[int] = [v for t in tile_list for v in t]
     h_tiles = pk.add(tiles)
+    num_wanted, num_decode = len(want_rows), len(decode_tokens)
 
     group_handles = []
+    rows = np.arange(R)
     for gi, g in enumerate(cache.groups):
         tables = [g.tables[req] for req in requests]
         mb = max((len(t) for t in tables), default=1) or 1
@@ -171,16 +188,17 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
                 raise ValueError(f"pad_blocks {pad_blocks} is below the longest block table {mb}")
             mb = pad_blocks
         flat = np.full((R, mb), -1, dtype=np.int32)
-        slots = np.empty(T, dtype=np.int32)
         for r, t in enumerate(tables):
-            flat[r, :len(t)] = t
-            pos = position_parts[r]
-            pages = flat[r, pos // bs]
-            slots[q_start[r]:q_start[r + 1]] = np.where(pages >= 0, pages * bs + pos % bs, -1)
+            if len(t):
+                flat[r, :len(t)] = np.frombuffer(t, dtype=np.int32)
+        pages = flat[tok_req, positions // bs] if T else np.zeros(0, np.int32)
+        slots = np.where(pages >= 0, pages * bs + positions % bs, -1).astype(np.int32)
         group_handles.append((pk.add(flat), mb, pk.add(slots)))
 
     buffer = pk.upload(device, into)
-    max_ctx = max(ctx_len, default=0)
+    if refresh_only:
+        return None
+    max_ctx = int(max(ctx_len)) if R else 0
     if pad_blocks is not None:
         max_ctx = pad_blocks * bs      # what the layout allows, not what this batch holds
     groups = []
@@ -188,13 +206,13 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
         groups.append(AttentionBatch(
             tok_req=pk.view(h_req), positions=pk.view(h_pos),
             block_table=pk.view(h_bt, (R, mb)), q_start=pk.view(h_qs), ctx_len=pk.view(h_ctx),
-            slots=pk.view(h_sl), num_decode=len(decode_tokens),
+            slots=pk.view(h_sl), num_decode=num_decode,
             decode_tokens=pk.view(h_dec), prefill_tiles=pk.view(h_tiles, (len(tiles) // 4, 4)),
-            max_ctx=max_ctx, all_decode=len(decode_tokens) == R))
+            max_ctx=max_ctx, all_decode=num_decode == R))
     return StepBatch(
         num_tokens=T, num_requests=R, requests=requests, q_start=q_start,
         first_position=first_pos, slot_list=slot_list,
         max_position=int(positions.max()) if T else 0,
         token_ids=pk.view(h_tok), positions=pk.view(h_pos), tok_req=pk.view(h_req),
         want_rows=pk.view(h_want), slot_ids=pk.view(h_slot), groups=groups,
-        num_wanted=len(want_rows), buffer=buffer)
+        num_wanted=num_wanted, buffer=buffer)

@@ -84,23 +84,22 @@ class ModelRunner:
         V = self.model.vocab_size
         if not entries:
             return torch.empty((0, V), dtype=torch.float32, device=self.device)
-        seen = set()
+        names = [e.request for e in entries]
+        if len(set(names)) != len(names):
+            twice = next(n for n in names if names.count(n) > 1)
+            raise ValueError(f"request {twice!r} appears twice in one step")
         limit = self.model.spec.max_positions
-        for e in entries:
-            if e.request in seen:
-                raise ValueError(f"request {e.request!r} appears twice in one step")
-            seen.add(e.request)
-            ids = np.asarray(e.tokens)
-            if ids.dtype.kind not in "iu":
-                raise ValueError(f"request {e.request!r}: token ids must be integers")
-            if int(ids.min()) < 0 or int(ids.max()) >= V:
-                bad = int(ids[(ids < 0) | (ids >= V)][0])
-                raise ValueError(f"request {e.request!r}: token id {bad} is outside the "
-                                 f"vocabulary of {V}")
-            have = self.cache.length(e.request) if self.cache.has(e.request) else 0
-            if limit and have + len(e.tokens) > limit:
-                raise ValueError(f"request {e.request!r}: {have + len(e.tokens)} tokens exceed "
-                                 f"the model's {limit} positions")
+        if all(len(e.tokens) == 1 for e in entries):      # one check for a step of single tokens
+            self._check_ids(np.asarray([e.tokens[0] for e in entries]), entries)
+        else:
+            for e in entries:
+                self._check_ids(np.asarray(e.tokens), [e])
+        if limit:
+            for e in entries:
+                have = self.cache.length(e.request) if self.cache.has(e.request) else 0
+                if have + len(e.tokens) > limit:
+                    raise ValueError(f"request {e.request!r}: {have + len(e.tokens)} tokens exceed "
+                                     f"the model's {limit} positions")
         if not self.can_run(entries):
             raise OutOfPages(f"the cache cannot take this step ({sum(len(e.tokens) for e in entries)}"
                              f" tokens of {len(entries)} requests; "
@@ -127,6 +126,15 @@ class ModelRunner:
         self.steps += 1
         self.tokens += num_tokens
         return logits
+
+    def _check_ids(self, ids: np.ndarray, entries: Sequence[StepEntry]) -> None:
+        V = self.model.vocab_size
+        who = entries[0].request if len(entries) == 1 else [e.request for e in entries]
+        if ids.dtype.kind not in "iu":
+            raise ValueError(f"request {who!r}: token ids must be integers")
+        if int(ids.min()) < 0 or int(ids.max()) >= V:
+            bad = int(ids[(ids < 0) | (ids >= V)][0])
+            raise ValueError(f"request {who!r}: token id {bad} is outside the vocabulary of {V}")
 
     # ------------------------------------------------------------------ graph replay
     def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
@@ -165,7 +173,8 @@ class ModelRunner:
                 static_logits = self.model.forward(batch, sites)
             self._graphs[key] = _CapturedStep(graph, batch, sites, static_logits)
             return logits[:real]
-        build_batch(entries, self.cache, self.device, pad_blocks=pad, into=captured.batch.buffer)
+        build_batch(entries, self.cache, self.device, pad_blocks=pad, into=captured.batch.buffer,
+                    refresh_only=True)
         captured.graph.replay()
         self.graph_replays += 1
         return captured.logits[:real].clone()      # the next replay overwrites the graph's own output

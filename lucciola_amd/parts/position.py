@@ -8,12 +8,24 @@ float32) and the kernel looks them up; the table grows when a longer position sh
 """
 from __future__ import annotations
 
-from typing import Optional
+from typing import Dict, Optional, Tuple
 
 import torch
 
 from ..config.registry import POSITION_ENCODINGS
 from .base import BuildContext, Part
+
+
+class _SharedTable:
+    """One table for all parts with the same rotated size, base and device (the layers of a
+    model, usually): ``generation`` counts how often it has been made anew."""
+
+    def __init__(self) -> None:
+        self.table: Optional[torch.Tensor] = None
+        self.generation = 0
+
+
+_TABLES: Dict[Tuple[int, float, str], _SharedTable] = {}
 
 
 @POSITION_ENCODINGS.register("rotary")
@@ -24,12 +36,21 @@ class Rotary(Part):
             raise ValueError(f"rotary: the rotated size {rotary_dim} must be even")
         self.rotary_dim, self.theta = int(rotary_dim), float(theta)
         self.initial = int(max_positions)
-        self._table: Optional[torch.Tensor] = None
+        self._shared = _SharedTable()
         self._device = None
-        self.generation = 0      # counts how often the table has been made anew
 
     def bind(self, tensors, ctx: BuildContext) -> None:
         self._device = ctx.device
+        self._shared = _TABLES.setdefault((self.rotary_dim, self.theta, str(torch.device(ctx.device))),
+                                          _SharedTable())
+
+    @property
+    def generation(self) -> int:
+        return self._shared.generation
+
+    @property
+    def _table(self) -> Optional[torch.Tensor]:
+        return self._shared.table
 
     def _make(self, count: int) -> torch.Tensor:
         half = self.rotary_dim // 2
@@ -47,8 +68,8 @@ class Rotary(Part):
             count = max(need, min(self.initial, 16384), 256)
             if self._table is not None:
                 count = max(count, 2 * self._table.shape[0])
-            self._table = self._make(count)
-            self.generation += 1
+            self._shared.table = self._make(count)
+            self._shared.generation += 1
         return self._table
 
     def capacity(self) -> int:
