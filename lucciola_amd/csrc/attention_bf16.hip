@@ -321,8 +321,8 @@ __global__ __launch_bounds__(128) void attn_decode_join_kernel(const float* __re
 // HPW = 2 (an even number of heads per kv head): wave w works on head w / 2 of the pair and on
 // rows [32 (w % 2), +32) as two column tiles; HPW = 1: wave w works on rows [16 w, +16).
 // Key rows are padded by 16 bytes in LDS, which spreads the 16 keys of an operand read over
-// all banks.
-constexpr int PF_NP = 4;
+// all banks; value pages are interleaved in pairs and rotated for the same reason.
+constexpr int PF_NP = 4;   // even: value pages go to LDS in pairs
 
 template <int D, int HPW>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
@@ -409,7 +409,17 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
                 if (CHUNKS % 256 == 0 || c < CHUNKS) {
                     const int key = c / (D / 4), col = (c % (D / 4)) * 4;
                     *reinterpret_cast<short4v*>(&ks[stage][n * KPAGE + key * KLD + col]) = kreg[n][i];
-                    *reinterpret_cast<short4v*>(&vs[stage][n * VPAGE + c * 4]) = vreg[n][i];
+                    // values: the pages of a pair (n, n + 1) are interleaved, [dim][4 keys of n | the same
+                    // 4 keys of n + 1] in 16-byte pieces, so that a product's operand is one 128-bit
+                    // read; the pieces of a row rotate with the row, which spreads the 16 rows of
+                    // a read (and the 16 pieces of a write) over all banks
+                    if ((n & 1) == 0) {
+                        const int dim = c >> 2, piece = (c & 3) ^ ((dim >> 2) & 3);
+                        union { short4v h[2]; bf16x8 full; } both;
+                        both.h[0] = vreg[n][i];
+                        both.h[1] = vreg[n + 1][i];
+                        *reinterpret_cast<bf16x8*>(&vs[stage][(n >> 1) * 2 * VPAGE + dim * 32 + piece * 8]) = both.full;
+                    }
                 }
             }
         if (pg0 + NP <= last) fetch(pg0 + NP);
@@ -489,14 +499,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
         for (int n = 0; n < NP; n += 2)
 #pragma unroll
             for (int t = 0; t < D / 16; ++t) {
-                const short4v v0 = *reinterpret_cast<const short4v*>(&vs[stage][n * VPAGE + (t * 16 + q) * PAGE + kg * 4]);
-                const short4v v1 = *reinterpret_cast<const short4v*>(&vs[stage][(n + 1) * VPAGE + (t * 16 + q) * PAGE + kg * 4]);
-                union { short4v h[2]; bf16x8 full; } va;
-                va.h[0] = v0;
-                va.h[1] = v1;
+                const bf16x8 va = *reinterpret_cast<const bf16x8*>(
+                    &vs[stage][(n >> 1) * 2 * VPAGE + (t * 16 + q) * 32 + ((kg ^ ((q >> 2) & 3)) * 8)]);
 #pragma unroll
                 for (int c = 0; c < QT; ++c)
-                    st.o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va.full, pb[c][n / 2], st.o[c][t], 0, 0, 0);
+                    st.o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[c][n / 2], st.o[c][t], 0, 0, 0);
             }
     }
 #pragma unroll
