@@ -310,6 +310,134 @@ def test_toy_architecture_with_a_stateful_mixer():
         ARCHITECTURES.unregister("ToyForCausalLM")
 
 
+# ------------------------------------------------------------------ routing and another position encoding
+class ToyRouted(Part):
+    """A feed-forward with routing: a float32 router picks the top 2 of E one-matrix experts per
+    token; their outputs are mixed with the softmax of the two router logits."""
+
+    def __init__(self, hidden_size, experts):
+        super().__init__(hidden_size=hidden_size, experts=experts)
+        self.H, self.E = hidden_size, experts
+
+    def declare(self):
+        out = {"router": ParamDecl((self.E, self.H))}
+        for e in range(self.E):
+            out[f"expert{e}"] = ParamDecl((self.H, self.H))
+        return out
+
+    def bind(self, tensors, ctx):
+        self.router = tensors["router"]
+        self.experts = [tensors[f"expert{e}"] for e in range(self.E)]
+        self.dtype = ctx.dtype
+
+    def forward(self, x):
+        logits = ops.gemm(x, self.router, torch.float32)           # routing in float32
+        top, idx = logits.topk(2, dim=1)
+        mix = torch.softmax(top, dim=1)
+        out = torch.zeros(x.shape[0], self.H, dtype=torch.float32, device=x.device)
+        for e, w in enumerate(self.experts):
+            rows = (idx == e).any(dim=1).nonzero().flatten()
+            if rows.numel() == 0:
+                continue
+            y = ops.gemm(x[rows].contiguous(), w, torch.float32)
+            weight = (mix[rows] * (idx[rows] == e)).sum(dim=1, keepdim=True)
+            out[rows] += weight * y
+        return out.to(self.dtype)
+
+
+class ToyOffset(Part):
+    """A position encoding that is no rotation: q and k get sin(position * rate_j) added to
+    entry j of every head (in place, before the cache write)."""
+
+    def __init__(self, rate):
+        super().__init__(rate=rate)
+        self.rate = rate
+
+    def bind(self, tensors, ctx):
+        pass
+
+    def rotary_table(self, max_position):
+        return None                                    # not a table the fused kernel can use
+
+    def apply(self, qkv, nh, nkv, d, positions):
+        j = torch.arange(d, device=qkv.device, dtype=torch.float32)
+        add = torch.sin(positions.float()[:, None] * self.rate * (j + 1))     # [T, d]
+        heads = qkv.view(qkv.shape[0], nh + 2 * nkv, d)
+        heads[:, :nh + nkv] += add[:, None, :].to(qkv.dtype)
+
+
+TOY2 = {"architectures": ["Toy2ForCausalLM"], "hidden_size": 40, "vocab_size": 61, "experts": 5,
+        "eps": 1e-6, "heads": 3, "head_dim": 16, "rate": 0.37}
+
+
+def toy2_spec(c):
+    norm = PartSpec("rms", {"size": c["hidden_size"], "eps": c["eps"]})
+    attn = PartSpec("attention", {"hidden_size": c["hidden_size"], "num_heads": c["heads"],
+                                  "num_kv_heads": 1, "head_dim": c["head_dim"],
+                                  "position": PartSpec("toy_offset", {"rate": c["rate"]})})
+    ff = PartSpec("toy_routed", {"hidden_size": c["hidden_size"], "experts": c["experts"]})
+    layers = []
+    for i in range(2):
+        names = {"mixer_norm.weight": f"l{i}.n1", "feed_forward_norm.weight": f"l{i}.n2",
+                 "feed_forward.router": f"l{i}.router"}
+        names.update({f"feed_forward.expert{e}": f"l{i}.e{e}" for e in range(c["experts"])})
+        names.update({f"mixer.{k}_proj": f"l{i}.{k}" for k in "qkvo"})
+        layers.append(LayerSpec("prenorm_residual", attn, ff, norm, norm, names))
+    return ModelSpec(hidden_size=c["hidden_size"], vocab_size=c["vocab_size"], embedding_name="emb",
+                     layers=layers, run_order=[RunEntry(0), RunEntry(1)],
+                     final_norm=norm, final_norm_names={"weight": "final"}, head_name="head", init_std=0.3)
+
+
+def toy2_plain(c, w, ids):
+    w = {k: v.double() for k, v in w.items()}
+    T, d = len(ids), c["head_dim"]
+    h = w["emb"][torch.tensor(ids)]
+    add = torch.sin(torch.arange(T, dtype=F64)[:, None] * c["rate"] * (torch.arange(d, dtype=F64) + 1))
+    for i in range(2):
+        x = plain.rmsnorm(h, w[f"l{i}.n1"], c["eps"])
+        q = (x @ w[f"l{i}.q"].T).view(T, c["heads"], d) + add[:, None, :]
+        k = (x @ w[f"l{i}.k"].T).view(T, 1, d) + add[:, None, :]
+        v = (x @ w[f"l{i}.v"].T).view(T, 1, d)
+        h = h + plain.attention(q, k, v, list(range(T))).reshape(T, -1) @ w[f"l{i}.o"].T
+        x = plain.rmsnorm(h, w[f"l{i}.n2"], c["eps"])
+        logits = x @ w[f"l{i}.router"].T
+        top, idx = logits.topk(2, dim=1)
+        mix = torch.softmax(top, dim=1)
+        y = torch.zeros_like(h)
+        for t in range(T):
+            for slot in range(2):
+                y[t] += mix[t, slot] * (w[f"l{i}.e{int(idx[t, slot])}"] @ x[t])
+        h = h + y
+    return plain.rmsnorm(h, w["final"], c["eps"]) @ w["head"].T
+
+
+def test_toy_routed_feed_forward_and_another_position_encoding():
+    """A feed-forward with routing and a position encoding that is no rotation, both defined
+    here, registered, built and stepped without a change to the package: the cache, the step
+    function and the scheduler know nothing of either."""
+    from lucciola_amd.config.registry import POSITION_ENCODINGS
+    FEED_FORWARDS.register("toy_routed", ToyRouted, replace=True)
+    POSITION_ENCODINGS.register("toy_offset", ToyOffset, replace=True)
+    ARCHITECTURES.register("Toy2ForCausalLM", Architecture("Toy2ForCausalLM", read_config=dict,
+                                                           model_spec=toy2_spec), replace=True)
+    try:
+        spec = toy2_spec(TOY2)
+        weights = dict(random_tensors(declared_tensors(spec), 9, spec.init_std, torch.float32))
+        model = _build(spec, DictSource(weights), "float32", "cuda:0")
+        prompts = prompts_for({"vocab_size": TOY2["vocab_size"]}, [19, 5, 44, 30], 4)
+        refs = {n: toy2_plain(TOY2, weights, ids) for n, ids in prompts.items()}
+        for family in (traces.whole, traces.tail_decode, traces.mixed):
+            steps = family(prompts)
+            runner = ModelRunner(model, EngineConfig(dtype="float32", block_size=8, max_seqs=4, device="cuda:0",
+                                                     max_blocks=traces.max_live_tokens(steps, 8) // 8))
+            got = replay(runner, steps)
+            compare(got, TOY2, weights, prompts, 2e-5, refs)
+    finally:
+        FEED_FORWARDS.unregister("toy_routed")
+        POSITION_ENCODINGS.unregister("toy_offset")
+        ARCHITECTURES.unregister("Toy2ForCausalLM")
+
+
 def test_block_arrangement_alone():
     """The pre-norm residual arrangement with stand-in parts: h1 = h + mixer(norm1(h)),
     h2 = h1 + ff(norm2(h1)); the second branch's output is still pending when the block ends."""
