@@ -58,6 +58,33 @@ __device__ __forceinline__ void load_page(PageRegs<D>& r, const bf16* __restrict
     for (int i = 0; i < D / 16; ++i) r.v[i] = *reinterpret_cast<const short4v*>(vb + i * 16 * PAGE);
 }
 
+// Maximum and sum over the four lanes q, q + 16, q + 32, q + 48 that hold one column of a
+// matrix-core tile: two lane swaps of gfx950 (v_permlane32_swap exchanges the upper half of one
+// register with the lower half of another, v_permlane16_swap the odd rows of 16 lanes with the
+// even ones), no trip through LDS.  Written in assembly because the compiler's builtin loses
+// the second result when both operands hold the same value; the s_nops cover the hazards
+// that the compiler would otherwise handle.
+__device__ __forceinline__ void swap_halves(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap_rows(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float column_max(float x) {
+    float a = x, b = x;
+    swap_halves(a, b);
+    a = b = fmaxf(a, b);
+    swap_rows(a, b);
+    return fmaxf(a, b);
+}
+__device__ __forceinline__ float column_sum(float x) {
+    float a = x, b = x;
+    swap_halves(a, b);
+    a = b = a + b;
+    swap_rows(a, b);
+    return a + b;
+}
+
 __device__ __forceinline__ short bf16_bits(float f) {
     const bf16 b = static_cast<bf16>(f);
     return *reinterpret_cast<const short*>(&b);
@@ -84,8 +111,7 @@ __device__ __forceinline__ void attend_page(AttnState<D, QT>& st, const PageRegs
             s[v] = (j >= lo[c] && j <= hi[c]) ? s[v] * scale_log2 : -INFINITY;
             mx = fmaxf(mx, s[v]);
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = column_max(mx);
         const float m_new = fmaxf(st.m[c], mx);
         const float alpha = (st.m[c] == -INFINITY) ? 0.f : exp2f(st.m[c] - m_new);
         float p[4], psum = 0.f;
@@ -246,8 +272,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 
     // the waves' results meet in LDS
     float l = st.l[0];
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
+    l = column_sum(l);
     if (kg == 0) { sm_m[wave][q] = st.m[0]; sm_l[wave][q] = l; }
 #pragma unroll
     for (int tt = 0; tt < D / 16; ++tt)
@@ -463,8 +488,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
             for (int n = 0; n < NP; ++n)
 #pragma unroll
                 for (int v = 0; v < 4; ++v) mx = fmaxf(mx, sc[c][n][v]);
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            mx = column_max(mx);
             // Maxima are kept as raw scores; p = 2^((s - m) scale_log2), one fma and one v_exp.
             // m is a reference point, not necessarily the maximum: it moves (and the sums are
             // rescaled) only when a score would exceed it by more than 2^8, which keeps every p
@@ -509,8 +533,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
 #pragma unroll
     for (int c = 0; c < QT; ++c) {
         float l = st.l[c];
-        l += __shfl_xor(l, 16, 64);
-        l += __shfl_xor(l, 32, 64);
+        l = column_sum(l);
         if (!valid[c]) continue;
         const float inv = 1.f / l;
         bf16* orow = out + ((size_t)(row0 + wrow + c * 16 + q) * nh + h) * D + kg * 4;
