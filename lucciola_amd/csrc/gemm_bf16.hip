@@ -168,13 +168,18 @@ template <int N> __device__ __forceinline__ void wait_lgkmcnt() {
     __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));
 }
 
-// SPLIT: blockIdx.y owns a share of the k-blocks and writes its float32 partial sums to
-// part[blockIdx.y][M][N]; splitk_reduce_kernel adds the shares in a fixed order.
+// The grid's workgroups take the tiles [tile_base, tile_base + tile_count) of the tiles_m x
+// tiles_n tiles of the product.
+// SPLIT: blockIdx.y owns a share of the k-blocks and writes its float32 partial sums for a
+// reduction kernel to add in a fixed order: to part[blockIdx.y][M][N] (splitk_reduce_kernel),
+// or, if `compact`, tile by tile to part[blockIdx.y][tile - tile_base][BM][BN]
+// (tail_reduce_kernel).
 template <int BM, int BN, int TL_STAGES, int EPI, bool SPLIT, typename TO>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ x,
                                                          const bf16* __restrict__ w,
                                                          TO* __restrict__ out, float* __restrict__ part,
-                                                         int M, int N, int K, int tiles_m, int tiles_n) {
+                                                         int M, int N, int K, int tiles_m, int tile_base,
+                                                         int tile_count, int compact) {
     constexpr int S = TL_STAGES;
     constexpr int TM = BM / 64, TN = BN / 64;
     constexpr int KS = TL_K / 16;                             // k-steps per block
@@ -187,13 +192,15 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 
     // renumber: workgroups go round-robin over 8 XCDs; give each XCD a contiguous run of
     // tiles, m fastest, so that one XCD's L2 keeps the w tile that its workgroups share
-    const int total = tiles_m * tiles_n;
+    const int total = tile_count;
     int id = blockIdx.x;
     {
         const int q = total >> 3, rem = total & 7;
         const int xcd = id & 7, local = id >> 3;
         id = xcd * q + min(xcd, rem) + local;   // a bijection of [0, total) for any total
     }
+    const int local_tile = id;
+    id += tile_base;
     const int tm = id % tiles_m, tn = id / tiles_m;
     const int m0 = tm * BM, n0 = tn * BN;
 
@@ -379,12 +386,17 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
                 }
     } else {
         using TS = typename std::conditional<SPLIT, float, TO>::type;
-        TS* base = SPLIT ? (TS*)(part + (size_t)blockIdx.y * M * N) : (TS*)out;
-        if ((N & 1) == 0) {
+        const bool tilewise = SPLIT && compact;    // addresses inside the tile's own [BM][BN] block
+        TS* base = !SPLIT ? (TS*)out
+                 : tilewise ? (TS*)(part + ((size_t)blockIdx.y * tile_count + local_tile) * BM * BN)
+                            : (TS*)(part + (size_t)blockIdx.y * M * N);
+        const size_t ld = tilewise ? BN : N;
+        const int r0 = tilewise ? m0 : 0, c0 = tilewise ? n0 : 0;
+        if ((ld & 1) == 0) {
             // neighbouring lanes swap every other value, so that a lane holds two adjacent
             // columns of one row and stores them together: even lanes the even v, odd lanes the odd
             const bool odd = lane & 1;
-            TS* dst = base + (size_t)(mrow + (odd ? 1 : 0)) * N + (ncol & ~1);
+            TS* dst = base + (size_t)(mrow - r0 + (odd ? 1 : 0)) * ld + ((ncol & ~1) - c0);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -396,10 +408,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
                         const float got = lane_swap<0xB1>(odd ? first : second);   // lane ^ 1
                         const int dm = i * 32 + (v >> 2) * 8 + (v & 3);
                         if (mrow + (odd ? 1 : 0) + dm < M && (ncol & ~1) + j * 32 < N)
-                            store_pair<TS>(dst + (size_t)dm * N + j * 32, odd ? got : first, odd ? second : got);
+                            store_pair<TS>(dst + (size_t)dm * ld + j * 32, odd ? got : first, odd ? second : got);
                     }
         } else {
-            TS* dst = base + (size_t)mrow * N + ncol;
+            TS* dst = base + (size_t)(mrow - r0) * ld + (ncol - c0);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -408,7 +420,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
                     for (int v = 0; v < 16; ++v) {
                         const int dm = i * 32 + (v >> 2) * 8 + (v & 3);
                         if (mrow + dm < M && ncol + j * 32 < N)
-                            store_out<TS>(dst + (size_t)dm * N + j * 32, acc[i][j][v]);
+                            store_out<TS>(dst + (size_t)dm * ld + j * 32, acc[i][j][v]);
                     }
         }
     }
@@ -440,6 +452,36 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ part, TO* __restr
     }
 }
 
+// out = sum over the shares of the tiles [tile_base, tile_base + count) that were written tile by
+// tile, part[s][tile - tile_base][BM][BN], added in the order of s; EPI as in the products.
+// One workgroup per tile and 2048 of its elements.
+template <int EPI, typename TO>
+__global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restrict__ part, TO* __restrict__ out,
+                                                          int M, int N, int BM, int BN, int tiles_m,
+                                                          int tile_base, int count, int S) {
+    const int local = blockIdx.x, tile = tile_base + local;
+    const int m0 = (tile % tiles_m) * BM, n0 = (tile / tiles_m) * BN;
+    const size_t area = (size_t)BM * BN;
+    const float* src = part + (size_t)local * area;
+    for (int e = blockIdx.y * 2048 + threadIdx.x; e < min((int)area, (blockIdx.y + 1) * 2048); e += 256) {
+        const int row = e / BN, col = e - row * BN;
+        const int m = m0 + row, n = n0 + col;
+        if (m >= M || n >= N) continue;
+        if (EPI == 0) {
+            float t = 0.f;
+            for (int s = 0; s < S; ++s) t += src[(size_t)s * count * area + e];
+            store_out<TO>(out + (size_t)m * N + n, t);
+        } else if ((n & 15) < 8) {                     // a gate column; its up column lies 8 further on
+            float g = 0.f, u = 0.f;
+            for (int s = 0; s < S; ++s) {
+                g += src[(size_t)s * count * area + e];
+                u += src[(size_t)s * count * area + e + 8];
+            }
+            store_out<TO>(out + (size_t)m * (N / 2) + (size_t)(n >> 4) * 8 + (n & 7), swiglu_f(g, u));
+        }
+    }
+}
+
 // The tile shapes of the tiled kernel.  TILE_AUTO picks by size; the others are forced through
 // lc_gemm_bf16_force_tile (tests and tuning).
 enum : int { TILE_AUTO = -1, TILE_64x128 = 0, TILE_128x128 = 1, TILE_256x128 = 2, TILE_256x192 = 3, TILE_256x256 = 4, TILE_COUNT = 5 };
@@ -452,18 +494,41 @@ static long long tile_count(int t, int M, int N) {
     return (long long)((M + tile_bm(t) - 1) / tile_bm(t)) * ((N + tile_bn(t) - 1) / tile_bn(t));
 }
 
+// The shapes with 256 rows run one workgroup to a CU, so their tiles go through the CUs in
+// rounds of kCUs.  When the last round would be less than half full, its tiles are cut along K
+// into `shares` parts each (written tile by tile, summed by tail_reduce_kernel), which fills
+// that round's CUs with shorter pieces: rest tiles, shares parts (0, 1: no such tail).
+struct TailPlan {
+    int rest, shares;
+};
+static TailPlan tail_plan(int t, int M, int N, int K) {
+    TailPlan none = {0, 1};
+    if (tile_bm(t) != 256) return none;
+    const long long tiles = tile_count(t, M, N);
+    const int rest = (int)(tiles % kCUs), nk = K / TL_K;
+    if (tiles < kCUs || rest == 0 || rest > kCUs / 2 || nk < 16) return none;
+    int shares = kCUs / rest;
+    if (shares > nk / 8) shares = nk / 8;
+    if (shares < 2) return none;
+    TailPlan plan = {rest, shares};
+    return plan;
+}
+
 // The tile for a product with M > 16.  Up to 64 rows: the 64-row tile.  Beyond: the shape with
-// the least estimated time, (tiles a CU works through) x (tile area) / (measured relative rate
-// of the shape: larger tiles move fewer bytes per product).
-static int pick_tile(int M, int N) {
+// the least estimated time, (rounds of tiles a CU works through) x (tile area) / (measured
+// relative rate of the shape: larger tiles move fewer bytes per product).
+static int pick_tile(int M, int N, int K) {
     if (g_force_tile != TILE_AUTO) return g_force_tile;
     if (M <= 64) return TILE_64x128;
     const double rate[TILE_COUNT] = {0.0, 0.87, 1.0, 1.1, 1.2};
     int best = TILE_128x128;
     double best_cost = 0.0;
     for (int t = TILE_128x128; t < TILE_COUNT; ++t) {
-        const long long per_cu = (tile_count(t, M, N) + kCUs - 1) / kCUs;
-        const double cost = (double)per_cu * tile_bm(t) * tile_bn(t) / rate[t];
+        const long long tiles = tile_count(t, M, N);
+        double rounds = (double)((tiles + kCUs - 1) / kCUs);
+        const TailPlan tail = tail_plan(t, M, N, K);
+        if (tail.shares > 1) rounds = (double)(tiles / kCUs) + 1.0 / tail.shares + 0.1;
+        const double cost = rounds * tile_bm(t) * tile_bn(t) / rate[t];
         if (t == TILE_128x128 || cost < best_cost) { best = t; best_cost = cost; }
     }
     return best;
@@ -471,10 +536,10 @@ static int pick_tile(int M, int N) {
 
 // How many shares of K the product of these sizes is cut into (1: no workspace needed): as
 // many as it takes to give every CU a workgroup when whole-K tiles would be too few.  Only the
-// two small tiles are cut.
+// two small tiles are cut as a whole.
 static int splitk_shares(int M, int N, int K) {
     if (M <= 16) return 1;
-    const int t = pick_tile(M, N);
+    const int t = pick_tile(M, N, K);
     if (t != TILE_64x128 && t != TILE_128x128) return 1;
     const long long tiles = tile_count(t, M, N);
     if (tiles >= 400) return 1;
@@ -482,6 +547,17 @@ static int splitk_shares(int M, int N, int K) {
     int S = (int)((480 + tiles / 2) / tiles);
     if (S > nk / 4) S = nk / 4;
     return S < 1 ? 1 : S;
+}
+
+// float32 words of workspace that the product needs (0: none)
+static long long workspace_words(int M, int N, int K) {
+    if (M <= 16 && g_force_tile == TILE_AUTO) return 0;
+    const int t = pick_tile(M, N, K);
+    const int S = splitk_shares(M, N, K);
+    if (S > 1) return (long long)S * M * N;
+    const TailPlan tail = tail_plan(t, M, N, K);
+    if (tail.shares > 1) return (long long)tail.shares * tail.rest * tile_bm(t) * tile_bn(t);
+    return 0;
 }
 
 template <int MT, int NT, int WAVES, int UNROLL, int EPI, typename TO>
@@ -492,26 +568,39 @@ static void launch_skinny(const bf16* x, const bf16* w, TO* out, int M, int N, i
 
 template <int BM, int BN, int STAGES, int EPI, typename TO>
 static int launch_tiled(const bf16* x, const bf16* w, TO* out, float* workspace, int M, int N, int K,
-                        int shares, hipStream_t s) {
+                        int shares, TailPlan tail, hipStream_t s) {
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-    if (shares == 1) {
-        gemm_tiled_kernel<BM, BN, STAGES, EPI, false, TO><<<tiles_m * tiles_n, 256, 0, s>>>(
-            x, w, out, nullptr, M, N, K, tiles_m, tiles_n);
+    const int tiles = tiles_m * tiles_n;
+    if (shares == 1 && tail.shares <= 1) {
+        gemm_tiled_kernel<BM, BN, STAGES, EPI, false, TO><<<tiles, 256, 0, s>>>(
+            x, w, out, nullptr, M, N, K, tiles_m, 0, tiles, 0);
         LC_LAUNCH_CHECK("gemm_tiled");
         return 0;
     }
-    if constexpr (BM <= 128 && BN == 128) {
-        LC_CHECK(workspace, "gemm_bf16: M=%d N=%d K=%d needs a workspace", M, N, K);
-        gemm_tiled_kernel<BM, BN, STAGES, 0, true, TO><<<dim3(tiles_m * tiles_n, shares), 256, 0, s>>>(
-            x, w, out, workspace, M, N, K, tiles_m, tiles_n);
+    LC_CHECK(workspace, "gemm_bf16: M=%d N=%d K=%d needs a workspace", M, N, K);
+    if constexpr (BM == 256) {
+        LC_CHECK(shares == 1 && tail.rest > 0 && tail.rest < tiles, "gemm_bf16: bad tail for tile %dx%d", BM, BN);
+        const int whole = tiles - tail.rest;
+        gemm_tiled_kernel<BM, BN, STAGES, EPI, false, TO><<<whole, 256, 0, s>>>(
+            x, w, out, nullptr, M, N, K, tiles_m, 0, whole, 0);
+        LC_LAUNCH_CHECK("gemm_tiled");
+        gemm_tiled_kernel<BM, BN, STAGES, 0, true, TO><<<dim3(tail.rest, tail.shares), 256, 0, s>>>(
+            x, w, out, workspace, M, N, K, tiles_m, whole, tail.rest, 1);
+        LC_LAUNCH_CHECK("gemm_tiled");
+        tail_reduce_kernel<EPI, TO><<<dim3(tail.rest, (BM * BN + 2047) / 2048), 256, 0, s>>>(
+            workspace, out, M, N, BM, BN, tiles_m, whole, tail.rest, tail.shares);
+        LC_LAUNCH_CHECK("tail_reduce");
+        return 0;
+    } else {
+        LC_CHECK(tail.shares <= 1, "gemm_bf16: tile %dx%d has no tail", BM, BN);
+        gemm_tiled_kernel<BM, BN, STAGES, 0, true, TO><<<dim3(tiles, shares), 256, 0, s>>>(
+            x, w, out, workspace, M, N, K, tiles_m, 0, tiles, 0);
         LC_LAUNCH_CHECK("gemm_tiled");
         const size_t work = EPI ? (size_t)M * N / 2 : (size_t)M * N;
         splitk_reduce_kernel<EPI, TO><<<(int)((work + 255) / 256), 256, 0, s>>>(workspace, out, M, N, shares);
         LC_LAUNCH_CHECK("splitk_reduce");
         return 0;
     }
-    LC_CHECK(false, "gemm_bf16: tile %dx%d is not cut along K", BM, BN);
-    return 0;
 }
 
 template <int EPI, typename TO>
@@ -528,12 +617,14 @@ static int launch_bf16(const bf16* x, const bf16* w, TO* out, float* workspace, 
         return 0;
     }
     const int shares = splitk_shares(M, N, K);
-    switch (pick_tile(M, N)) {
-    case TILE_64x128:  return launch_tiled<64, 128, 4, EPI, TO>(x, w, out, workspace, M, N, K, shares, s);
-    case TILE_128x128: return launch_tiled<128, 128, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, s);
-    case TILE_256x128: return launch_tiled<256, 128, 3, EPI, TO>(x, w, out, workspace, M, N, K, shares, s);
-    case TILE_256x192: return launch_tiled<256, 192, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, s);
-    default:           return launch_tiled<256, 256, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, s);
+    const int tile = pick_tile(M, N, K);
+    const TailPlan tail = tail_plan(tile, M, N, K);
+    switch (tile) {
+    case TILE_64x128:  return launch_tiled<64, 128, 4, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
+    case TILE_128x128: return launch_tiled<128, 128, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
+    case TILE_256x128: return launch_tiled<256, 128, 3, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
+    case TILE_256x192: return launch_tiled<256, 192, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
+    default:           return launch_tiled<256, 256, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     }
 }
 
@@ -560,8 +651,7 @@ LC_API int lc_gemm_bf16_force_tile(int tile) {
 // float32 words of workspace that lc_gemm_bf16 needs for these sizes (0: none).
 LC_API long long lc_gemm_bf16_workspace(int M, int N, int K) {
     if (!lc_gemm_bf16_supported(M, N, K)) return 0;
-    const int S = splitk_shares(M, N, K);
-    return S > 1 ? (long long)S * M * N : 0;
+    return workspace_words(M, N, K);
 }
 
 // epilogue 0: out[M, N] = x . w^T.  epilogue 1 (SwiGLU): the rows of w come in blocks of 16,

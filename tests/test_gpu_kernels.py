@@ -272,6 +272,30 @@ def test_gemm_bf16_every_tile_shape(tile, M, N, K):
         close(fused, (g / (1 + torch.exp(-g)) * u).to(torch.bfloat16), torch.bfloat16, scale=K ** 0.5)
 
 
+@pytest.mark.parametrize("tile,M,N,K", [(4, 2000, 10200, 1024), (2, 2048, 10240, 1024), (3, 1990, 6520, 2048),
+                                        (-1, 2048, 10240, 5120)])
+def test_gemm_bf16_last_round_cut_along_k(tile, M, N, K):
+    """Sizes whose tiles fill the CUs once or twice and leave a small rest: the rest's tiles
+    are cut along K and summed by a second kernel.  Plain and with the SwiGLU epilogue,
+    bfloat16 and float32 output, ragged edges."""
+    x = rnd(M, K, dtype=torch.bfloat16, seed=65, scale=0.5)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=66, scale=0.5)
+    ops.force_gemm_tile(tile)
+    try:
+        assert ops.library().lc_gemm_bf16_workspace(M, N, K) > 0      # the cut is really taken
+        got16 = ops.gemm(x, w, torch.bfloat16)
+        got32 = ops.gemm(x, w, torch.float32)
+        fused = ops.gemm_swiglu(x, w[:N // 16 * 16])
+    finally:
+        ops.force_gemm_tile(-1)
+    want = x.float() @ w.float().T
+    close(got32, want, torch.float32, scale=K ** 0.5)
+    close(got16, want.to(torch.bfloat16), torch.bfloat16, scale=K ** 0.5)
+    blocks = want[:, :N // 16 * 16].double().view(M, -1, 2, 8)
+    g, u = blocks[:, :, 0, :].reshape(M, -1), blocks[:, :, 1, :].reshape(M, -1)
+    close(fused, (g / (1 + torch.exp(-g)) * u).to(torch.bfloat16), torch.bfloat16, scale=K ** 0.5)
+
+
 def test_gemm_bf16_one_hot_rows_and_columns():
     """x picks single columns of w: the product must return exactly those entries, so a wrong
     operand layout (rows, k order) shows as a wrong element, not as a small error."""
