@@ -219,40 +219,61 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
         const int half = pro.rot / 2;
         const float* cs = pro.rope ? pro.rope + (size_t)p * pro.rot : nullptr;
         const bf16* row = qkv + (size_t)t * q_stride;
-        for (int task = wave; task < ntask; task += 4) {
-            if (task == G + 1) {                          // v: copied, transposed into the page
-                const bf16* x = row + (size_t)(nh + nkv + kvh) * D;
-                bf16* col = v_cache + ((size_t)table[last_page] * nkv + kvh) * D * PAGE + (p % PAGE);
-                for (int i = lane; i < D; i += 64) col[(size_t)i * PAGE] = x[i];
-                continue;
-            }
-            const bool is_k = task == G;
-            const bf16* x = row + (size_t)(is_k ? nh + kvh : kvh * G + task) * D;
-            const float* w = is_k ? pro.k_w : pro.q_w;
-            bf16* dst = is_k ? k_cache + (((size_t)table[last_page] * nkv + kvh) * PAGE + (p % PAGE)) * D
-                             : sm_q + task * D;
-            float inv = 1.f;
-            if (w) {
-                float ss = 0.f;
-                for (int i = lane; i < D; i += 64) {
-                    const float v = static_cast<float>(x[i]);
-                    ss += v * v;
+        if (D == 128 && (pro.rot == 128 || pro.rot == 0)) {
+            // 16 lanes a head, as the separate kernel does it (and to the same bits)
+            const int j = threadIdx.x & 15;
+            for (int task = threadIdx.x >> 4; task < ntask; task += 16) {
+                if (task == G + 1) {                      // v: copied, transposed into the page
+                    const head_chunk raw = *reinterpret_cast<const head_chunk*>(row + (size_t)(nh + nkv + kvh) * D + 8 * j);
+                    bf16* col = v_cache + ((size_t)table[last_page] * nkv + kvh) * D * PAGE + (p % PAGE);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) col[(size_t)(8 * j + e) * PAGE] = raw[e];
+                    continue;
                 }
-                ss = wave_sum(ss);
-                inv = rsqrtf(ss / (float)D + pro.eps);
+                const bool is_k = task == G;
+                const bf16* x = row + (size_t)(is_k ? nh + kvh : kvh * G + task) * D + 8 * j;
+                bf16* dst = is_k ? k_cache + (((size_t)table[last_page] * nkv + kvh) * PAGE + (p % PAGE)) * D
+                                 : sm_q + task * D;
+                const head_chunk done = head128_norm_rope(*reinterpret_cast<const head_chunk*>(x), j,
+                                                          is_k ? pro.k_w : pro.q_w, pro.eps, cs);
+                *reinterpret_cast<head_chunk*>(dst + 8 * j) = done;
             }
-            for (int i = lane; i < half; i += 64) {
-                float a = static_cast<float>(x[i]) * inv, b = static_cast<float>(x[i + half]) * inv;
-                if (w) { a *= w[i]; b *= w[i + half]; }
-                float c = 1.f, sn = 0.f;
-                if (cs) { c = cs[i]; sn = cs[half + i]; }
-                dst[i] = static_cast<bf16>(a * c - b * sn);
-                dst[i + half] = static_cast<bf16>(a * sn + b * c);
-            }
-            for (int i = pro.rot + lane; i < D; i += 64) {
-                float a = static_cast<float>(x[i]) * inv;
-                if (w) a *= w[i];
-                dst[i] = static_cast<bf16>(a);
+        } else {
+            for (int task = wave; task < ntask; task += 4) {
+                if (task == G + 1) {                          // v: copied, transposed into the page
+                    const bf16* x = row + (size_t)(nh + nkv + kvh) * D;
+                    bf16* col = v_cache + ((size_t)table[last_page] * nkv + kvh) * D * PAGE + (p % PAGE);
+                    for (int i = lane; i < D; i += 64) col[(size_t)i * PAGE] = x[i];
+                    continue;
+                }
+                const bool is_k = task == G;
+                const bf16* x = row + (size_t)(is_k ? nh + kvh : kvh * G + task) * D;
+                const float* w = is_k ? pro.k_w : pro.q_w;
+                bf16* dst = is_k ? k_cache + (((size_t)table[last_page] * nkv + kvh) * PAGE + (p % PAGE)) * D
+                                 : sm_q + task * D;
+                float inv = 1.f;
+                if (w) {
+                    float ss = 0.f;
+                    for (int i = lane; i < D; i += 64) {
+                        const float v = static_cast<float>(x[i]);
+                        ss += v * v;
+                    }
+                    ss = wave_sum(ss);
+                    inv = rsqrtf(ss / (float)D + pro.eps);
+                }
+                for (int i = lane; i < half; i += 64) {
+                    float a = static_cast<float>(x[i]) * inv, b = static_cast<float>(x[i + half]) * inv;
+                    if (w) { a *= w[i]; b *= w[i + half]; }
+                    float c = 1.f, sn = 0.f;
+                    if (cs) { c = cs[i]; sn = cs[half + i]; }
+                    dst[i] = static_cast<bf16>(a * c - b * sn);
+                    dst[i + half] = static_cast<bf16>(a * sn + b * c);
+                }
+                for (int i = pro.rot + lane; i < D; i += 64) {
+                    float a = static_cast<float>(x[i]) * inv;
+                    if (w) a *= w[i];
+                    dst[i] = static_cast<bf16>(a);
+                }
             }
         }
         __syncthreads();      // q is in LDS; the owner's k and v have reached memory

@@ -64,6 +64,65 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
     return total;
 }
 
+// ---------------------------------------------------------------------------------------------
+// A head of 128 bfloat16 entries held by a group of 16 neighbouring lanes (lane j of the group
+// has entries 8 j .. 8 j + 7): RMSNorm over the head and half-split rotary embedding without
+// leaving the registers.  Lanes talk through DPP moves inside their row of 16; all 16 lanes of
+// a group must be active.  Used by the q/k norm + rotary kernel and by the decode attention's
+// own prologue, which therefore agree to the bit.
+typedef __bf16 head_chunk __attribute__((ext_vector_type(8)));
+
+template <int CTRL> __device__ __forceinline__ float row_move(float v) {   // a DPP move inside a row of 16
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over the 16 lanes of a row; the pairs are added in the same order in every lane, so all
+// lanes end with the same bits.
+__device__ __forceinline__ float row16_sum(float v, int j) {
+    v += row_move<0xB1>(v);                                   // lane ^ 1
+    v += row_move<0x4E>(v);                                   // lane ^ 2
+    const float up = row_move<0x124>(v), down = row_move<0x12C>(v);   // rotations by 4 and by 12
+    // which of the two rotations brought lane j ^ 4 depends on the direction of the rotation:
+    // the lane index itself is sent along to tell
+    const int from_up = __builtin_bit_cast(int, row_move<0x124>(__builtin_bit_cast(float, j)));
+    v += (from_up == (j ^ 4)) ? up : down;                    // lane ^ 4
+    v += row_move<0x128>(v);                                  // lane ^ 8
+    return v;
+}
+
+// x: the lane's 8 entries (raw).  w: the norm's 128 weights or null.  cs: the position's row of
+// the rotary table (64 cosines, then 64 sines) or null.  Entry i pairs with entry i + 64.
+__device__ __forceinline__ head_chunk head128_norm_rope(head_chunk x, int j, const float* __restrict__ w,
+                                                        float eps, const float* __restrict__ cs) {
+    float f[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = static_cast<float>(x[e]);
+    if (w) {
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss = __fmaf_rn(f[e], f[e], ss);
+        ss = row16_sum(ss, j);
+        const float inv = rsqrtf(ss / 128.f + eps);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = __fmul_rn(__fmul_rn(f[e], inv), w[8 * j + e]);
+    }
+    if (cs) {
+        const int i0 = 8 * (j & 7);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float other = row_move<0x128>(f[e]);        // the partner entry, 64 further on or back
+            const float c = cs[i0 + e], sn = cs[64 + i0 + e];
+            // first half: a c - b s (a own, b partner); second half: a s + b c (b own, a partner)
+            const float own_c = __fmul_rn(f[e], c), other_s = __fmul_rn(other, sn);
+            f[e] = (j < 8) ? __fsub_rn(own_c, other_s) : __fadd_rn(other_s, own_c);
+        }
+    }
+    head_chunk out;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = static_cast<bf16>(f[e]);
+    return out;
+}
+
 // Error text of the last failed call on this thread; entry points return 0 on success.
 void set_error(const char* fmt, ...);
 

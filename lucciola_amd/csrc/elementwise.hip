@@ -239,6 +239,39 @@ __global__ void qk_norm_rope_write_kernel(T* __restrict__ qkv, int T_tokens, int
     }
 }
 
+// The same for bfloat16 heads of 128 entries that rotate whole or not at all: 16 lanes a head,
+// 16-byte loads and stores, 16 heads a workgroup.
+__global__ __launch_bounds__(256) void qk_norm_rope_write128_kernel(
+    bf16* __restrict__ qkv, int T_tokens, int nh, int nkv, const float* __restrict__ q_w,
+    const float* __restrict__ k_w, float eps, const int* __restrict__ positions,
+    const float* __restrict__ rope_table, bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
+    const int* __restrict__ slots, int page_size) {
+    constexpr int d = 128;
+    const int heads = nh + 2 * nkv;
+    const long long g = (long long)blockIdx.x * 16 + (threadIdx.x >> 4);
+    if (g >= (long long)T_tokens * heads) return;          // whole groups of 16 lanes leave together
+    const int t = (int)(g / heads), head = (int)(g - (long long)t * heads), j = threadIdx.x & 15;
+    bf16* x = qkv + ((size_t)t * heads + head) * d + 8 * j;
+    const bool is_q = head < nh, is_k = !is_q && head < nh + nkv;
+    const int kvh = is_q ? 0 : (is_k ? head - nh : head - nh - nkv);
+    const int slot = (!is_q && slots && k_cache) ? slots[t] : -1;
+    const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot - page * page_size : 0;
+    const head_chunk raw = *reinterpret_cast<const head_chunk*>(x);
+    if (!is_q && !is_k) {      // v: copied, transposed into the page
+        if (slot >= 0) {
+            bf16* col = v_cache + ((size_t)page * nkv + kvh) * d * page_size + off;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) col[(size_t)(8 * j + e) * page_size] = raw[e];
+        }
+        return;
+    }
+    const float* cs = rope_table ? rope_table + (size_t)positions[t] * d : nullptr;
+    const head_chunk done = head128_norm_rope(raw, j, is_q ? q_w : k_w, eps, cs);
+    *reinterpret_cast<head_chunk*>(x) = done;
+    if (is_k && slot >= 0)
+        *reinterpret_cast<head_chunk*>(k_cache + (((size_t)page * nkv + kvh) * page_size + off) * d + 8 * j) = done;
+}
+
 // ------------------------------------------------------------------------------- SwiGLU
 // gu: [T, 2 I] (gate columns, then up columns) -> out [T, I]
 template <typename T>
@@ -337,6 +370,15 @@ LC_API int lc_qk_norm_rope_write(void* qkv, int dt, int T, int nh, int nkv, int 
     LC_CHECK(!(k_cache && slots) || (v_cache && page_size > 0),
              "qk_norm_rope_write: cache write needs v_cache and a page size");
     if (!rope_table) rot = 0;
+    if (dt == DT_BF16 && d == 128 && (rot == 0 || rot == 128) && (q_w == nullptr) == (k_w == nullptr) &&
+        (uintptr_t)qkv % 16 == 0 && (uintptr_t)k_cache % 16 == 0) {
+        const long long groups = (long long)T * (nh + 2 * nkv);
+        qk_norm_rope_write128_kernel<<<(unsigned)((groups + 15) / 16), 256, 0, stream>>>(
+            (bf16*)qkv, T, nh, nkv, q_w, k_w, eps, positions, rope_table, (bf16*)k_cache, (bf16*)v_cache,
+            slots, page_size);
+        LC_LAUNCH_CHECK("qk_norm_rope_write128");
+        return 0;
+    }
     const int waves = 4;
     dim3 grid(T, (nh + 2 * nkv + waves - 1) / waves);
     if (dt == DT_F32)

@@ -100,7 +100,7 @@ def make_rope_table(positions, rot, theta):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 4), (6, 2, 48, 16), (5, 5, 32, 8), (8, 1, 128, 16),
-                                           (3, 1, 80, 2), (2, 2, 256, 32)])
+                                           (3, 1, 80, 2), (2, 2, 256, 32), (32, 8, 128, 16), (3, 3, 128, 4)])
 def test_qk_norm_rope_write(dtype, nh, nkv, d, page):
     T, pages = 37, 40
     qkv = rnd(T, (nh + 2 * nkv) * d, dtype=dtype, seed=9)
