@@ -25,6 +25,9 @@ FLAGS = [
     "-fvisibility=hidden", "-fno-gpu-rdc",
     # packed float32 instructions are switched off for every kernel of this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the kernels keep accumulators and operands in register arrays that only fully unrolled
+    # loops can index; no size estimate may stop an unroll that the source asks for
+    "-mllvm", "-pragma-unroll-threshold=1000000",
 ]
 
 
