@@ -41,10 +41,13 @@ __global__ void embedding_kernel(const int* __restrict__ ids, const TW* __restri
 // ------------------------------------------------------------------------------- RMSNorm
 // One workgroup per output row r.  src row = rows ? rows[r] : r.
 //   v = h[src] (+ delta[src]);  if (write_h) h[src] = v;  out[r] = v * rsqrt(mean(v^2)+eps) * w
+// With sumsq: out[r] = v * w and sumsq[r] = sum(v^2): the row's factor is left to the product
+// that reads out (gemm_bf16.hip, scaled rows).
 template <typename T>
 __global__ void rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delta,
                                const int* __restrict__ rows, const float* __restrict__ w,
-                               float eps, T* __restrict__ out, int n, int write_h) {
+                               float eps, T* __restrict__ out, int n, int write_h,
+                               float* __restrict__ sumsq) {
     __shared__ float scratch[16];
     const int r = blockIdx.x;
     const int src = rows ? rows[r] : r;
@@ -60,7 +63,8 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delt
         ss += v * v;
     }
     ss = block_sum(ss, scratch);
-    const float inv = rsqrtf(ss / (float)n + eps);
+    const float inv = sumsq ? 1.f : rsqrtf(ss / (float)n + eps);
+    if (sumsq && threadIdx.x == 0) sumsq[r] = ss;
     T* o = out + (size_t)r * n;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
         float v = hr[i];
@@ -91,7 +95,8 @@ constexpr int RN_THREADS = 256, RN_CHUNKS = 4;   // 256 threads x 4 chunks x 8 e
 template <typename T>
 __global__ __launch_bounds__(RN_THREADS) void rmsnorm_vec_kernel(
     float* __restrict__ h, const T* __restrict__ delta, const int* __restrict__ rows,
-    const float* __restrict__ w, float eps, T* __restrict__ out, int n, int write_h) {
+    const float* __restrict__ w, float eps, T* __restrict__ out, int n, int write_h,
+    float* __restrict__ sumsq) {
     __shared__ float scratch[16];
     const int r = blockIdx.x;
     const int src = rows ? rows[r] : r;
@@ -124,7 +129,8 @@ __global__ __launch_bounds__(RN_THREADS) void rmsnorm_vec_kernel(
         }
     }
     ss = block_sum(ss, scratch);
-    const float inv = rsqrtf(ss / (float)n + eps);
+    const float inv = sumsq ? 1.f : rsqrtf(ss / (float)n + eps);
+    if (sumsq && threadIdx.x == 0) sumsq[r] = ss;
     T* o = out + (size_t)r * n;
 #pragma unroll
     for (int c = 0; c < RN_CHUNKS; ++c) {
@@ -308,8 +314,10 @@ LC_API int lc_embedding(const int* ids, const void* table, int table_dt, float* 
     return 0;
 }
 
+// sumsq (may be null): R floats; then out = (h + delta) * w without the rows' factors, and
+// sumsq[r] = the row's sum of squares.
 LC_API int lc_rmsnorm(float* h, const void* delta, const int* rows, const float* w, float eps,
-                      void* out, int dt, int R, int n, int write_h, hipStream_t stream) {
+                      void* out, int dt, int R, int n, int write_h, float* sumsq, hipStream_t stream) {
     LC_CHECK(R >= 0 && n > 0, "rmsnorm: bad sizes R=%d n=%d", R, n);
     if (R == 0) return 0;
     LC_CHECK(h && w && out, "rmsnorm: null pointer");
@@ -321,17 +329,17 @@ LC_API int lc_rmsnorm(float* h, const void* delta, const int* rows, const float*
     if (dt == DT_F32) {
         if (vec)
             rmsnorm_vec_kernel<float><<<R, RN_THREADS, 0, stream>>>(h, (const float*)delta, rows, w, eps,
-                                                                    (float*)out, n, write_h);
+                                                                    (float*)out, n, write_h, sumsq);
         else
             rmsnorm_kernel<float><<<R, threads, 0, stream>>>(h, (const float*)delta, rows, w, eps,
-                                                             (float*)out, n, write_h);
+                                                             (float*)out, n, write_h, sumsq);
     } else if (dt == DT_BF16) {
         if (vec)
             rmsnorm_vec_kernel<bf16><<<R, RN_THREADS, 0, stream>>>(h, (const bf16*)delta, rows, w, eps,
-                                                                   (bf16*)out, n, write_h);
+                                                                   (bf16*)out, n, write_h, sumsq);
         else
             rmsnorm_kernel<bf16><<<R, threads, 0, stream>>>(h, (const bf16*)delta, rows, w, eps,
-                                                            (bf16*)out, n, write_h);
+                                                            (bf16*)out, n, write_h, sumsq);
     } else {
         LC_CHECK(false, "rmsnorm: unknown dtype %d", dt);
     }

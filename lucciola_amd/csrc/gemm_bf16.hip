@@ -55,17 +55,63 @@ __device__ __forceinline__ float swiglu_f(float g, float u) {
 // ------------------------------------------------------------------------------- skinny
 constexpr int SK_KBLOCK = 128; // k elements per wave iteration
 
+// What a skinny product can take over from the norm kernels around it (decode steps are
+// bound by the number of kernels they start, not by the work of the small ones):
+//   SCALE (with epilogue 0 or 1): x holds rows h * norm_weight that still lack their common
+//     factor rsqrt(mean(h^2) + eps); scale_partials [scale_count][16] holds pieces of every
+//     row's sum of squares (row m at [piece][m]); the factor is applied to the float32 sums.
+//   epilogue 2: resid [M, N] is the float32 residual stream: resid += x . w^T in place; the
+//     kernel also leaves next_x = bf16(resid * next_w) and, per workgroup, the sums of squares
+//     of its columns of the new rows in next_partials [gridDim.x][16]: what a SCALE product
+//     (or rmsnorm) needs to go on without a norm kernel in between.
+struct SkinnyFuse {
+    const float* scale_partials;
+    int scale_count;
+    float scale_eps;
+    float* resid;
+    const float* next_w;
+    bf16* next_x;
+    float* next_partials;
+};
+constexpr int SK_MAX_PIECES = 512;   // pieces of a sum of squares that a SCALE product reads
+
 // MT: tiles of 16 rows of x; NT: tiles of 16 rows of w per workgroup; the WAVES waves of a
 // workgroup take the k blocks in turn.
-template <int MT, int NT, int WAVES, int UNROLL, int EPI, typename TO>
+template <int MT, int NT, int WAVES, int UNROLL, int EPI, bool SCALE, typename TO>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __restrict__ x,
                                                                  const bf16* __restrict__ w,
                                                                  TO* __restrict__ out, int M, int N,
-                                                                 int K) {
+                                                                 int K, SkinnyFuse fuse) {
+    static_assert(WAVES == 16, "the epilogues lay 1024 threads over a workgroup's results");
+    static_assert(!(SCALE || EPI == 2) || MT == 1, "fused norms are for up to 16 rows");
+    static_assert(EPI != 2 || NT <= 4, "epilogue 2 gives every result a thread of its own");
+    static_assert(!(SCALE && EPI == 2), "both would use the same words of LDS");
     __shared__ float red[WAVES * MT * NT * 256];
+    __shared__ float pieces[WAVES][16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, g = lane >> 4;
     const int n0 = blockIdx.x * (16 * NT);
+
+    // loads whose values are wanted only after the products; issued first, they are back
+    // before the first operand is
+    float piece[SK_MAX_PIECES / 64];
+    if (SCALE) {
+#pragma unroll
+        for (int i = 0; i < SK_MAX_PIECES / 64; ++i) {
+            const int p = (threadIdx.x >> 4) + 64 * i;
+            piece[i] = p < fuse.scale_count ? fuse.scale_partials[p * 16 + r] : 0.f;
+        }
+    }
+    // epilogue 2: thread idx < NT * 256 owns the result (m, n) of tile idx / 256
+    const int e_tile = threadIdx.x >> 8, e_v = (threadIdx.x >> 6) & 3;
+    const int e_m = r, e_n = n0 + e_tile * 16 + g * 4 + e_v;
+    const bool e_mine = EPI == 2 && threadIdx.x < NT * 256 && e_m < M && e_n < N;
+    float e_resid = 0.f, e_w = 0.f;
+    if (e_mine) {
+        e_resid = fuse.resid[(size_t)e_m * N + e_n];
+        e_w = fuse.next_w[e_n];
+    }
+
     const bf16* wp[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) wp[nt] = w + (size_t)min(n0 + nt * 16 + r, N - 1) * K + g * 8;
@@ -108,7 +154,49 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 #pragma unroll
             for (int v = 0; v < 4; ++v)
                 red[((wave * NT + nt) * MT + mt) * 256 + v * 64 + lane] = acc[nt][mt][v];
+    if (SCALE) {
+        // this wave's pieces of the rows' sums of squares: lanes r, r + 16, r + 32, r + 48 hold row r
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < SK_MAX_PIECES / 64; ++i) sum += piece[i];
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        if (g == 0) pieces[wave][r] = sum;
+    }
     __syncthreads();
+    if (EPI == 2) {
+        float total = 0.f;
+        if (threadIdx.x < NT * 256) {
+#pragma unroll
+            for (int wv = 0; wv < WAVES; ++wv) total += red[wv * NT * 256 + threadIdx.x];
+        }
+        float sq = 0.f;
+        if (e_mine) {
+            const float v = e_resid + total;
+            fuse.resid[(size_t)e_m * N + e_n] = v;
+            fuse.next_x[(size_t)e_m * N + e_n] = static_cast<bf16>(v * e_w);
+            sq = v * v;
+        }
+        // a row's squares: over the wave's four column groups, then over the waves that hold results
+        sq += __shfl_xor(sq, 16, 64);
+        sq += __shfl_xor(sq, 32, 64);
+        if (g == 0) pieces[wave][r] = sq;
+        __syncthreads();
+        if (threadIdx.x < 16) {
+            float row = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < NT * 4; ++wv) row += pieces[wv][threadIdx.x];
+            fuse.next_partials[(size_t)blockIdx.x * 16 + threadIdx.x] = row;
+        }
+        return;
+    }
+    float factor[1] = {1.f};   // of row (threadIdx.x % 16): every result a thread sums is in that row
+    if (SCALE) {
+        float ss = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < WAVES; ++wv) ss += pieces[wv][r];
+        factor[0] = rsqrtf(ss / (float)K + fuse.scale_eps);
+    }
     if (EPI == 0) {
         for (int idx = threadIdx.x; idx < NT * MT * 256; idx += WAVES * 64) {
             float total = 0.f;
@@ -117,7 +205,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
             const int tile = idx >> 8, v = (idx >> 6) & 3, l = idx & 63;
             const int nt = tile / MT, mt = tile % MT;
             const int m = mt * 16 + (l & 15), n = n0 + nt * 16 + (l >> 4) * 4 + v;
-            if (m < M && n < N) store_out<TO>(out + (size_t)m * N + n, total);
+            if (m < M && n < N) store_out<TO>(out + (size_t)m * N + n, total * factor[0]);
         }
     } else {
         // rows of w come in blocks of 16: 8 gate rows, then their 8 up rows; out has N / 2 columns
@@ -133,7 +221,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
             const int nt = tile / MT, mt = tile % MT;
             const int m = mt * 16 + (l & 15), n = n0 + nt * 16 + (l >> 4) * 4 + v;   // gate row, n % 16 < 8
             const int col = (n >> 4) * 8 + (n & 7);
-            if (m < M && n < N) store_out<TO>(out + (size_t)m * (N / 2) + col, swiglu_f(g, u));
+            if (m < M && n < N) store_out<TO>(out + (size_t)m * (N / 2) + col, swiglu_f(g * factor[0], u * factor[0]));
         }
     }
 }
@@ -560,10 +648,36 @@ static long long workspace_words(int M, int N, int K) {
     return 0;
 }
 
-template <int MT, int NT, int WAVES, int UNROLL, int EPI, typename TO>
-static void launch_skinny(const bf16* x, const bf16* w, TO* out, int M, int N, int K, hipStream_t s) {
+template <int MT, int NT, int WAVES, int UNROLL, int EPI, bool SCALE, typename TO>
+static void launch_skinny(const bf16* x, const bf16* w, TO* out, int M, int N, int K, SkinnyFuse fuse,
+                          hipStream_t s) {
     const int rows = 16 * NT;
-    gemm_skinny_kernel<MT, NT, WAVES, UNROLL, EPI, TO><<<(N + rows - 1) / rows, WAVES * 64, 0, s>>>(x, w, out, M, N, K);
+    gemm_skinny_kernel<MT, NT, WAVES, UNROLL, EPI, SCALE, TO><<<(N + rows - 1) / rows, WAVES * 64, 0, s>>>(
+        x, w, out, M, N, K, fuse);
+}
+
+// The skinny kernel's shape for M <= 16 rows.  Measured: with one or two rows of x a deeper
+// unroll keeps more of w in flight; from about 12 rows on, x costs as much to fetch as w, and
+// two row tiles per workgroup share it (only where that still leaves every CU two workgroups).
+enum : int { SKINNY_DEEP = 0, SKINNY_PLAIN = 1, SKINNY_WIDE = 2 };
+static int skinny_shape(int M, int N) {
+    if (M <= 2) return SKINNY_DEEP;
+    if (M >= 12 && N >= 32 * 2 * kCUs) return SKINNY_WIDE;
+    return SKINNY_PLAIN;
+}
+static int skinny_workgroups(int M, int N) {
+    const int rows = skinny_shape(M, N) == SKINNY_WIDE ? 32 : 16;
+    return (N + rows - 1) / rows;
+}
+
+template <int EPI, bool SCALE, typename TO>
+static void launch_skinny_any(const bf16* x, const bf16* w, TO* out, int M, int N, int K, SkinnyFuse fuse,
+                              hipStream_t s) {
+    switch (skinny_shape(M, N)) {
+    case SKINNY_DEEP: launch_skinny<1, 1, 16, 4, EPI, SCALE, TO>(x, w, out, M, N, K, fuse, s); break;
+    case SKINNY_WIDE: launch_skinny<1, 2, 16, 2, EPI, SCALE, TO>(x, w, out, M, N, K, fuse, s); break;
+    default:          launch_skinny<1, 1, 16, 2, EPI, SCALE, TO>(x, w, out, M, N, K, fuse, s); break;
+    }
 }
 
 template <int BM, int BN, int STAGES, int EPI, typename TO>
@@ -607,12 +721,7 @@ template <int EPI, typename TO>
 static int launch_bf16(const bf16* x, const bf16* w, TO* out, float* workspace, int M, int N, int K,
                        hipStream_t s) {
     if (M <= 16 && g_force_tile == TILE_AUTO) {
-        // measured: with one or two rows of x a deeper unroll keeps more of w in flight; from
-        // about 12 rows on, x costs as much to fetch as w, and two row tiles per workgroup
-        // share it (only where that still leaves every CU two workgroups)
-        if (M <= 2) launch_skinny<1, 1, 16, 4, EPI, TO>(x, w, out, M, N, K, s);
-        else if (M >= 12 && N >= 32 * 2 * kCUs) launch_skinny<1, 2, 16, 2, EPI, TO>(x, w, out, M, N, K, s);
-        else launch_skinny<1, 1, 16, 2, EPI, TO>(x, w, out, M, N, K, s);
+        launch_skinny_any<EPI, false, TO>(x, w, out, M, N, K, SkinnyFuse{}, s);
         LC_LAUNCH_CHECK("gemm_skinny");
         return 0;
     }
@@ -675,5 +784,61 @@ LC_API int lc_gemm_bf16(const void* x, const void* w, void* out, int out_dt, int
         return epilogue ? launch_bf16<1, float>(xb, wb, (float*)out, workspace, M, N, K, stream)
                         : launch_bf16<0, float>(xb, wb, (float*)out, workspace, M, N, K, stream);
     LC_CHECK(false, "gemm_bf16: unknown output dtype %d", out_dt);
+    return 0;
+}
+
+// ------------------------------------------------------------------- norms folded into products
+// For steps of up to 16 rows (decode), where a norm kernel costs its start and nothing else.
+// The residual stream h [M, H] is float32.  A "prepared norm" of h for a norm weight g is the
+// pair (xg = bf16(h * g) [M, H], pieces [count][16] of every row's sum of squares): what is
+// missing is each row's factor rsqrt(mean(h^2) + eps), which a product can apply to its sums.
+
+// Number of pieces that lc_gemm_bf16_residual writes for these sizes; 0: the fused kernels do
+// not take these sizes (more than 16 rows, K not a multiple of 128, a forced tile shape, more
+// pieces than a scaled product reads).
+LC_API int lc_gemm_bf16_residual_pieces(int M, int N, int K) {
+    if (!lc_gemm_bf16_supported(M, N, K) || M > 16 || g_force_tile != TILE_AUTO) return 0;
+    const int pieces = skinny_workgroups(M, N);
+    return pieces <= SK_MAX_PIECES ? pieces : 0;
+}
+
+// resid [M, N] += x [M, K] . w [N, K]^T (float32, in place); next_x [M, N] = bf16(resid * next_w);
+// next_pieces [lc_gemm_bf16_residual_pieces(M, N, K)][16]: sums of squares of the new rows.
+LC_API int lc_gemm_bf16_residual(const void* x, const void* w, float* resid, const float* next_w,
+                                 void* next_x, float* next_pieces, int M, int N, int K,
+                                 hipStream_t stream) {
+    LC_CHECK(lc_gemm_bf16_residual_pieces(M, N, K) > 0,
+             "gemm_bf16_residual: sizes M=%d N=%d K=%d are not supported", M, N, K);
+    LC_CHECK(x && w && resid && next_w && next_x && next_pieces, "gemm_bf16_residual: null pointer");
+    LC_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_bf16_residual: operands must be 16-byte aligned");
+    SkinnyFuse fuse{};
+    fuse.resid = resid;
+    fuse.next_w = next_w;
+    fuse.next_x = (bf16*)next_x;
+    fuse.next_partials = next_pieces;
+    launch_skinny_any<2, false, float>((const bf16*)x, (const bf16*)w, (float*)nullptr, M, N, K, fuse, stream);
+    LC_LAUNCH_CHECK("gemm_skinny");
+    return 0;
+}
+
+// out = (x . w^T) with row m scaled by rsqrt(sum_p pieces[p][m] / K + eps) before the epilogue
+// (0: plain, bfloat16 [M, N]; 1: SwiGLU as in lc_gemm_bf16, bfloat16 [M, N / 2]).
+LC_API int lc_gemm_bf16_scaled_rows(const void* x, const void* w, void* out, int M, int N, int K,
+                                    int epilogue, const float* pieces, int count, float eps,
+                                    hipStream_t stream) {
+    LC_CHECK(lc_gemm_bf16_supported(M, N, K) && M <= 16 && g_force_tile == TILE_AUTO,
+             "gemm_bf16_scaled_rows: sizes M=%d N=%d K=%d are not supported", M, N, K);
+    LC_CHECK(count >= 1 && count <= SK_MAX_PIECES, "gemm_bf16_scaled_rows: %d pieces (at most %d)", count, SK_MAX_PIECES);
+    LC_CHECK(x && w && out && pieces, "gemm_bf16_scaled_rows: null pointer");
+    LC_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_bf16_scaled_rows: operands must be 16-byte aligned");
+    LC_CHECK(epilogue == 0 || (epilogue == 1 && N % 16 == 0),
+             "gemm_bf16_scaled_rows: the SwiGLU epilogue needs N (%d) to be a multiple of 16", N);
+    SkinnyFuse fuse{};
+    fuse.scale_partials = pieces;
+    fuse.scale_count = count;
+    fuse.scale_eps = eps;
+    if (epilogue) launch_skinny_any<1, true, bf16>((const bf16*)x, (const bf16*)w, (bf16*)out, M, N, K, fuse, stream);
+    else launch_skinny_any<0, true, bf16>((const bf16*)x, (const bf16*)w, (bf16*)out, M, N, K, fuse, stream);
+    LC_LAUNCH_CHECK("gemm_skinny");
     return 0;
 }

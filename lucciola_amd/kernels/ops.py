@@ -23,12 +23,15 @@ DT_F32, DT_BF16 = 0, 1
 _ARG = {"p": ctypes.c_void_p, "i": ctypes.c_int, "f": ctypes.c_float}
 _SIGNATURES = {
     "lc_embedding": "ppipiiip",
-    "lc_rmsnorm": "ppppfpiiiip",
+    "lc_rmsnorm": "ppppfpiiiipp",
     "lc_rmsnorm_act": "ppfpiiip",
     "lc_gemm_generic": "pipipiiiip",
     "lc_gemm_bf16": "pppiiiiipp",
     "lc_gemm_bf16_supported": "iii",
     "lc_gemm_bf16_force_tile": "i",
+    "lc_gemm_bf16_residual_pieces": "iii",
+    "lc_gemm_bf16_residual": "ppppppiiip",
+    "lc_gemm_bf16_scaled_rows": "pppiiiipifp",
     "lc_qk_norm_rope_write": "piiiiippfppipppip",
     "lc_attention_generic": "pipppipppiiiiiifip",
     "lc_attn_bf16_supported": "iiii",
@@ -125,19 +128,74 @@ def embedding(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
 
 
 # ------------------------------------------------------------------------------ norms
-def rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
-            out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+# Steps of up to 16 rows (decode) are bound by the number of kernels they start.  There the
+# norm between two products need not be a kernel of its own: the product before it can add its
+# result to the residual stream and leave the sums of squares (a PendingProduct completed by
+# ``rmsnorm(..., scaled=True)``), and the product after it can apply the rows' factors to its
+# sums (it is given ScaledRows).  Both are only ever handed to code that asks for them; anyone
+# else gets tensors.
+@dataclass
+class PendingProduct:
+    """``x . w^T`` that has not been computed yet: a branch's last product, waiting to be
+    added to the residual stream by the kernel that computes it."""
+
+    x: torch.Tensor
+    w: torch.Tensor
+    out_dtype: torch.dtype
+
+    def value(self) -> torch.Tensor:
+        return gemm(self.x, self.w, self.out_dtype)
+
+
+@dataclass
+class ScaledRows:
+    """The normed residual stream short of each row's factor: ``x`` = bf16(h * weight) [T, n];
+    ``pieces`` [count, 16] float32 hold pieces of the rows' sums of squares (row t at
+    [piece, t]); the factor of row t is rsqrt(sum of its pieces / n + eps)."""
+
+    x: torch.Tensor
+    pieces: torch.Tensor
+    count: int
+    eps: float
+    h: torch.Tensor            # the stream and the weight, for whoever needs the rows themselves
+    weight: torch.Tensor
+
+    def value(self) -> torch.Tensor:
+        return rmsnorm(self.h, None, self.weight, self.eps, self.x.dtype)
+
+
+def value(t):
+    """The tensor that ``t`` stands for (``t`` itself if it is one)."""
+    return t.value() if isinstance(t, (PendingProduct, ScaledRows)) else t
+
+
+def rmsnorm(h: torch.Tensor, delta, weight: torch.Tensor, eps: float,
+            out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None, scaled: bool = False):
     """RMSNorm of the float32 residual stream ``h`` [T, n], with the pending branch output
-    ``delta`` [T, n] added first.
+    ``delta`` [T, n] (a tensor or a PendingProduct) added first.
 
     Without ``rows``: ``h += delta`` in place and every row is normed.  With ``rows`` (int32
     [R]): only those rows are normed (``h`` stays as it is) and the result is [R, n].
+    ``scaled``: the caller also takes ScaledRows, and gets them where that saves a kernel.
     """
     _need(h, "rmsnorm h", torch.float32, 2)
     _need(weight, "rmsnorm weight", torch.float32, 1)
     T, n = h.shape
     if weight.shape[0] != n:
         raise KernelError(f"rmsnorm: weight has {weight.shape[0]} entries for rows of {n}")
+    scaled = (scaled and rows is None and out_dtype == torch.bfloat16 and 0 < T <= 16
+              and _fast_gemm_ok(T, 16, n))
+    if isinstance(delta, PendingProduct):
+        M, K = delta.x.shape
+        pieces = (library().lc_gemm_bf16_residual_pieces(M, n, K)
+                  if scaled and delta.w.shape[0] == n and M == T else 0)
+        if pieces:
+            xg = torch.empty((T, n), dtype=torch.bfloat16, device=h.device)
+            parts = torch.empty((pieces, 16), dtype=torch.float32, device=h.device)
+            _call("lc_gemm_bf16_residual", _ptr(delta.x), _ptr(delta.w), _ptr(h), _ptr(weight),
+                  _ptr(xg), _ptr(parts), _c_int(M), _c_int(n), _c_int(K), _stream())
+            return ScaledRows(xg, parts, pieces, float(eps), h, weight)
+        delta = delta.value()
     if delta is not None:
         _need(delta, "rmsnorm delta", out_dtype, 2)
         if tuple(delta.shape) != (T, n):
@@ -146,10 +204,11 @@ def rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor
         _need(rows, "rmsnorm rows", torch.int32, 1)
     R = T if rows is None else rows.shape[0]
     out = torch.empty((R, n), dtype=out_dtype, device=h.device)
+    parts = torch.empty((1, 16), dtype=torch.float32, device=h.device) if scaled else None
     _call("lc_rmsnorm", _ptr(h), _ptr(delta), _ptr(rows), _ptr(weight), _c_float(eps), _ptr(out),
           _c_int(_dt(out)), _c_int(R), _c_int(n),
-          _c_int(1 if (rows is None and delta is not None) else 0), _stream())
-    return out
+          _c_int(1 if (rows is None and delta is not None) else 0), _ptr(parts), _stream())
+    return ScaledRows(out, parts, 1, float(eps), h, weight) if scaled else out
 
 
 def rmsnorm_act(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
@@ -166,8 +225,32 @@ def rmsnorm_act(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tens
 
 
 # ------------------------------------------------------------------------------ products
-def gemm(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """``x`` [M, K] times ``w`` [N, K] transposed -> [M, N]; float32 accumulation."""
+def _scaled_product(x: "ScaledRows", w: torch.Tensor, epilogue: int) -> Optional[torch.Tensor]:
+    """``x`` with its rows' factors times ``w`` transposed in one kernel, or None if there is
+    no such kernel for these operands."""
+    M, K = x.x.shape
+    N = w.shape[0]
+    if not (w.dtype == torch.bfloat16 and x.x.dtype == torch.bfloat16 and w.shape[1] == K
+            and library().lc_gemm_bf16_residual_pieces(M, 16, K)):
+        return None
+    out = torch.empty((M, N // 2 if epilogue else N), dtype=torch.bfloat16, device=w.device)
+    _call("lc_gemm_bf16_scaled_rows", _ptr(x.x), _ptr(w), _ptr(out), _c_int(M), _c_int(N),
+          _c_int(K), _c_int(epilogue), _ptr(x.pieces), _c_int(x.count), _c_float(x.eps), _stream())
+    return out
+
+
+def gemm(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None, defer: bool = False):
+    """``x`` [M, K] times ``w`` [N, K] transposed -> [M, N]; float32 accumulation.
+
+    ``x`` may be ScaledRows.  ``defer``: the result is a branch's output that goes to the
+    residual stream; where the kernel that computes it can add it there itself, a
+    PendingProduct comes back instead of a tensor."""
+    if isinstance(x, ScaledRows):
+        if out_dtype in (None, torch.bfloat16) and not defer:
+            out = _scaled_product(x, w, 0)
+            if out is not None:
+                return out
+        x = x.value()
     _need(x, "gemm x", None, 2)
     _need(w, "gemm w", None, 2)
     M, K = x.shape
@@ -175,6 +258,9 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = No
     if K != K2:
         raise KernelError(f"gemm: x is [{M}, {K}] but w is [{N}, {K2}]")
     out_dtype = out_dtype or x.dtype
+    if (defer and out_dtype == torch.bfloat16 and x.dtype == torch.bfloat16
+            and w.dtype == torch.bfloat16 and library().lc_gemm_bf16_residual_pieces(M, N, K)):
+        return PendingProduct(x, w, out_dtype)
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     if M == 0:
         return out
@@ -201,7 +287,13 @@ def gemm_swiglu_supported(x_dtype, w: torch.Tensor, K: int) -> bool:
 
 def gemm_swiglu(x: torch.Tensor, w_interleaved: torch.Tensor) -> torch.Tensor:
     """``silu(x . gate^T) * (x . up^T)`` in one kernel, with gate and up interleaved by
-    :func:`interleave_gate_up`; bfloat16 only.  [M, K] x [2 I, K] -> [M, I]."""
+    :func:`interleave_gate_up`; bfloat16 only.  [M, K] x [2 I, K] -> [M, I].  ``x`` may be
+    ScaledRows."""
+    if isinstance(x, ScaledRows):
+        out = _scaled_product(x, w_interleaved, 1) if w_interleaved.shape[0] % 16 == 0 else None
+        if out is not None:
+            return out
+        x = x.value()
     _need(x, "gemm_swiglu x", torch.bfloat16, 2)
     _need(w_interleaved, "gemm_swiglu w", torch.bfloat16, 2)
     M, K = x.shape

@@ -25,6 +25,7 @@ from .feed_forward import stack_rows
 @MIXERS.register("attention")
 class Attention(Part):
     graph_safe = True   # launches only kernels whose arguments stay put between steps
+    takes_scaled_rows = True   # x may be ops.ScaledRows; the output may be an ops.PendingProduct
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  scale: Optional[float] = None, qk_norm: Optional[PartSpec] = None,
@@ -86,4 +87,4 @@ class Attention(Part):
         prologue = ops.QKPrologue(q_w, k_w, eps, table, attn.slots if site.writes_cache else None)
         o = ops.attention(qkv, attn, k_cache, v_cache, self.nh, self.nkv, self.d, site.page_size,
                           self.scale, self.window or 0, prologue)
-        return ops.gemm(o, self.o, self.dtype)
+        return ops.gemm(o, self.o, self.dtype, defer=True)

@@ -7,11 +7,16 @@ names (``LayerSpec.names``).
 
 Interfaces (all tensors on the GPU; "act" is the engine's activation dtype):
   Norm            add_norm(stream) -> act [T, n]; add_norm_rows(stream, rows) -> act [R, n];
-                  fused_rms() -> (weight float32 [n], eps) or None
+                  fused_rms() -> (weight float32 [n], eps) or None.  A norm with
+                  offers_scaled_rows = True also has add_norm(stream, scaled=True), which may
+                  return ops.ScaledRows; stream.pending may be an ops.PendingProduct
   PositionEncoding  rotary_table(max_position) -> float32 [positions, rot] or None;
                   apply(qkv, nh, nkv, d, positions) in place, when there is no table
   Mixer           forward(x act [T, H], site: SiteView) -> act [T, H]; cache_need() -> spec
   FeedForward     forward(x act [T, H]) -> act [T, H]
+                  A mixer or feed-forward with takes_scaled_rows = True may be given
+                  ops.ScaledRows as x (ops.gemm and ops.gemm_swiglu take them) and may return
+                  ops.gemm(..., defer=True); ops.value(t) turns either into a tensor
   Block           forward(stream, site) -> None (updates the stream)
 """
 from __future__ import annotations
@@ -41,7 +46,7 @@ class ResidualStream:
 
     def __init__(self, h: torch.Tensor):
         self.h = h
-        self.pending: Optional[torch.Tensor] = None
+        self.pending = None      # a tensor [T, H] or an ops.PendingProduct
 
 
 class Part:

@@ -24,6 +24,7 @@ def stack_rows(tensors):
 @FEED_FORWARDS.register("gated_mlp")
 class GatedMLP(Part):
     graph_safe = True   # launches only kernels whose arguments stay put between steps
+    takes_scaled_rows = True   # x may be ops.ScaledRows; the output may be an ops.PendingProduct
 
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
         super().__init__(hidden_size=hidden_size, intermediate_size=intermediate_size,
@@ -55,4 +56,4 @@ class GatedMLP(Part):
             z = ops.gemm_swiglu(x, self.gate_up)
         else:
             z = ops.swiglu(ops.gemm(x, self.gate_up, self.dtype))
-        return ops.gemm(z, self.down, self.dtype)
+        return ops.gemm(z, self.down, self.dtype, defer=True)

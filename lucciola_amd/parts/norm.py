@@ -16,6 +16,7 @@ from .base import BuildContext, Part, ResidualStream
 @NORMS.register("rms")
 class RMSNorm(Part):
     graph_safe = True   # launches only kernels whose arguments stay put between steps
+    offers_scaled_rows = True   # add_norm(stream, scaled=True) may return ops.ScaledRows
 
     def __init__(self, size: int, eps: float):
         super().__init__(size=size, eps=eps)
@@ -30,9 +31,10 @@ class RMSNorm(Part):
         self.weight = tensors["weight"]
         self.dtype = ctx.dtype
 
-    def add_norm(self, stream: ResidualStream) -> torch.Tensor:
-        """Add the pending branch output into the stream and return the normed stream."""
-        x = ops.rmsnorm(stream.h, stream.pending, self.weight, self.eps, self.dtype)
+    def add_norm(self, stream: ResidualStream, scaled: bool = False):
+        """Add the pending branch output into the stream and return the normed stream
+        (``scaled``: the caller also takes ops.ScaledRows)."""
+        x = ops.rmsnorm(stream.h, stream.pending, self.weight, self.eps, self.dtype, scaled=scaled)
         stream.pending = None
         return x
 

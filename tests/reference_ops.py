@@ -14,7 +14,7 @@ def embedding(ids, table):
     return table[ids.long()].to(torch.float32)
 
 
-def rmsnorm(h, delta, weight, eps, out_dtype, rows=None):
+def rmsnorm(h, delta, weight, eps, out_dtype, rows=None, scaled=False):   # never hands out scaled rows
     if rows is None:
         if delta is not None:
             h += delta.to(torch.float32)
@@ -33,7 +33,7 @@ def rmsnorm_act(x, weight, eps):
     return (v * inv * weight.to(F64)).to(x.dtype)
 
 
-def gemm(x, w, out_dtype=None):
+def gemm(x, w, out_dtype=None, defer=False):   # never defers
     return (x.to(F64) @ w.to(F64).T).to(out_dtype or x.dtype)
 
 

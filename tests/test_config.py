@@ -66,7 +66,7 @@ def test_sliding_window_layers():
     assert off.sliding_window is None and set(off.layer_types) == {"full_attention"}
 
 
-@pytest.mark.parametrize("key", ["A", "B", "C"])
+@pytest.mark.parametrize("key", ["A", "B", "C", "D"])
 def test_round_trip(key, tmp_path):
     cfg = Qwen3Config.from_dict(configs.ALL[key][0])
     (tmp_path / "config.json").write_text(json.dumps(cfg.to_dict()))

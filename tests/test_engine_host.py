@@ -28,12 +28,13 @@ def make(cfg, seed, page, blocks, dtype="float32"):
     return make_runner(cfg, weights, page, blocks, dtype, "cpu"), weights
 
 
-@pytest.mark.parametrize("key", ["A", "B", "C"])
+@pytest.mark.parametrize("key", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("family", ["whole", "tail", "chunked", "mixed"])
 def test_step_function_matches_plain(monkeypatch, key, family):
     reference_ops.install(monkeypatch)
     cfg, page, seed = configs.ALL[key]
-    lengths = {"A": [5, 11, 17, 40], "B": [1, 9, 30, 64, 45], "C": [70, 33, 50, 3, 61]}[key]
+    lengths = {"A": [5, 11, 17, 40], "B": [1, 9, 30, 64, 45], "C": [70, 33, 50, 3, 61],
+               "D": [37, 2, 50, 16]}[key]
     prompts = prompts_for(cfg, lengths, seed)
     steps = {"whole": traces.whole, "tail": traces.tail_decode, "chunked": traces.chunked,
              "mixed": traces.mixed}[family](prompts)

@@ -27,7 +27,8 @@ DEV = "cuda:0"
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 # error of a row of logits: max |difference| / max |logit|
 TOL = {"float32": 2e-5, "bfloat16": 3e-2}
-LENGTHS = {"A": [5, 11, 17, 40, 130], "B": [1, 9, 30, 64, 45, 200], "C": [70, 33, 50, 3, 61, 150]}
+LENGTHS = {"A": [5, 11, 17, 40, 130], "B": [1, 9, 30, 64, 45, 200], "C": [70, 33, 50, 3, 61, 150],
+           "D": [37, 2, 90, 16, 140]}
 
 _cache = {}
 
@@ -43,7 +44,7 @@ def case(key):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("key", ["A", "B", "C"])
+@pytest.mark.parametrize("key", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("family", ["whole", "tail", "chunked", "mixed"])
 def test_replay_families(dtype, key, family):
     cfg, page, weights, prompts, refs = case(key)
@@ -140,7 +141,7 @@ def test_long_decoding(dtype, key):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("key", ["A", "B", "C"])
+@pytest.mark.parametrize("key", ["A", "B", "C", "D"])
 def test_first_tokens(dtype, key):
     cfg, page, seed = configs.ALL[key]
     weights = random_weights(cfg, seed)
@@ -158,7 +159,7 @@ def engine_for(cfg, weights, page, blocks, dtype, **kw):
                                                  device=DEV, **kw))
 
 
-@pytest.mark.parametrize("key", ["A", "B", "C"])
+@pytest.mark.parametrize("key", ["A", "B", "C", "D"])
 def test_greedy_generation_through_the_engine(key):
     cfg, page, seed = configs.ALL[key]
     weights = random_weights(cfg, seed, std=0.3)

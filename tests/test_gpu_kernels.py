@@ -296,6 +296,63 @@ def test_gemm_bf16_last_round_cut_along_k(tile, M, N, K):
     close(fused, (g / (1 + torch.exp(-g)) * u).to(torch.bfloat16), torch.bfloat16, scale=K ** 0.5)
 
 
+@pytest.mark.parametrize("M,H,K,N2", [(1, 128, 128, 48), (2, 384, 256, 1000), (5, 256, 640, 272), (8, 4096, 512, 2064),
+                                      (11, 640, 128, 16), (12, 16384, 128, 16416), (16, 1152, 384, 130)])
+def test_norm_folded_into_the_products_around_it(M, H, K, N2):
+    """Up to 16 rows: the product before a norm adds its result to the stream and leaves
+    bf16(h * weight) and the pieces of the rows' sums of squares; the product after it applies
+    the rows' factors to its sums.  Each piece is checked against the plain formulas, and the
+    chain against norm-then-product; the first norm of a model has no product before it."""
+    eps = 3e-6
+    h = rnd(M, H, seed=70, scale=2.0)
+    x = rnd(M, K, dtype=torch.bfloat16, seed=71)
+    w = rnd(H, K, dtype=torch.bfloat16, seed=72, scale=K ** -0.5)
+    g = 1 + rnd(H, seed=73, scale=0.2)
+    w2 = rnd(N2, H, dtype=torch.bfloat16, seed=74, scale=H ** -0.5)
+    pending = ops.gemm(x, w, torch.bfloat16, defer=True)
+    assert isinstance(pending, ops.PendingProduct)
+    h_want = h.double() + x.double() @ w.double().T
+    h_got = h.clone()
+    rows = ops.rmsnorm(h_got, pending, g, eps, torch.bfloat16, scaled=True)
+    assert isinstance(rows, ops.ScaledRows) and rows.count == rows.pieces.shape[0]
+    torch.testing.assert_close(h_got.double(), h_want, rtol=1e-5, atol=1e-5)
+    close(rows.x, (h_got.double() * g.double()).to(torch.bfloat16), torch.bfloat16)
+    torch.testing.assert_close(rows.pieces[:, :M].double().sum(0), (h_got.double() ** 2).sum(1), rtol=1e-5, atol=0)
+    normed = h_got.double() * torch.rsqrt((h_got.double() ** 2).mean(1, keepdim=True) + eps) * g.double()
+    close(ops.value(rows), normed.to(torch.bfloat16), torch.bfloat16)
+    # the product takes the rounded rows h * g and applies the factors to its float32 sums
+    factors = torch.rsqrt((h_got.double() ** 2).mean(1, keepdim=True) + eps)
+    full = (rows.x.double() @ w2.double().T) * factors
+    got = ops.gemm(rows, w2, torch.bfloat16)
+    close(got, full.to(torch.bfloat16), torch.bfloat16, scale=2.0)
+    w2e = w2[:N2 // 16 * 16]
+    blocks = full[:, :N2 // 16 * 16].view(M, -1, 2, 8)
+    gate, up = blocks[:, :, 0, :].reshape(M, -1), blocks[:, :, 1, :].reshape(M, -1)
+    close(ops.gemm_swiglu(rows, w2e), (gate / (1 + torch.exp(-gate)) * up).to(torch.bfloat16), torch.bfloat16, scale=2.0)
+    # and the chain is the product of the normed rows, up to the rounding of those rows to bfloat16
+    exact = normed @ w2.double().T
+    assert float((got.double() - exact).norm() / exact.norm()) < 6e-3
+    # the same rows from the norm kernel alone (no product before it), with and without a branch to add
+    for delta in (None, rnd(M, H, dtype=torch.bfloat16, seed=75)):
+        h2 = h.clone()
+        alone = ops.rmsnorm(h2, delta, g, eps, torch.bfloat16, scaled=True)
+        assert isinstance(alone, ops.ScaledRows) and alone.count == 1
+        h2_want = h.double() + (0 if delta is None else delta.double())
+        torch.testing.assert_close(h2.double(), h2_want, rtol=1e-6, atol=1e-6)
+        normed2 = h2.double() * torch.rsqrt((h2.double() ** 2).mean(1, keepdim=True) + eps) * g.double()
+        exact2 = normed2 @ w2.double().T
+        assert float((ops.gemm(alone, w2, torch.bfloat16).double() - exact2).norm() / exact2.norm()) < 6e-3
+    # whoever does not ask for scaled rows gets tensors, and the pending product is added all the same
+    h3 = h.clone()
+    plain_rows = ops.rmsnorm(h3, ops.gemm(x, w, torch.bfloat16, defer=True), g, eps, torch.bfloat16)
+    assert isinstance(plain_rows, torch.Tensor)
+    torch.testing.assert_close(h3.double(), h_want, rtol=2e-2, atol=2e-2)   # the branch was rounded to bfloat16 first
+    # more than 16 rows, float32, or a width the matrix-core kernels do not take: nothing is deferred
+    assert isinstance(ops.gemm(rnd(17, K, dtype=torch.bfloat16), w, torch.bfloat16, defer=True), torch.Tensor)
+    assert isinstance(ops.gemm(x.float(), w.float(), torch.float32, defer=True), torch.Tensor)
+    assert isinstance(ops.rmsnorm(rnd(M, 72), None, 1 + rnd(72), eps, torch.bfloat16, scaled=True), torch.Tensor)
+
+
 def test_gemm_bf16_one_hot_rows_and_columns():
     """x picks single columns of w: the product must return exactly those entries, so a wrong
     operand layout (rows, k order) shows as a wrong element, not as a small error."""

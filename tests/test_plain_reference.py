@@ -138,7 +138,7 @@ def test_softmax_vectors_of_the_reference():
         assert plain.sample_token(x, 1e-3, 0.5) == len(x) - 1     # temperature -> 0 is the argmax
 
 
-@pytest.mark.parametrize("key", ["A", "B", "C"])
+@pytest.mark.parametrize("key", ["A", "B", "C", "D"])
 def test_residual_wiring(key):
     cfg, _, seed = configs.ALL[key]
     w = {k: v.clone() for k, v in random_weights(cfg, seed).items()}
@@ -155,7 +155,7 @@ def test_residual_wiring(key):
     assert not torch.allclose(full, want)
 
 
-@pytest.mark.parametrize("key", ["A", "B", "C"])
+@pytest.mark.parametrize("key", ["A", "B", "C", "D"])
 def test_shifting_all_positions_changes_nothing(key):
     cfg, _, seed = configs.ALL[key]
     w = random_weights(cfg, seed)

@@ -113,7 +113,7 @@ def test_kept_dtypes():
                       {"x": ParamDecl((2,))}, torch.device("cpu"))
 
 
-@pytest.mark.parametrize("key", ["A", "B", "C"])
+@pytest.mark.parametrize("key", ["A", "B", "C", "D"])
 def test_random_model_folder(tmp_path, key):
     cfg, _, seed = configs.ALL[key]
     folder = write_model_folder(str(tmp_path / "m"), cfg, seed)
