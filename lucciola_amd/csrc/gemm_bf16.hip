@@ -58,11 +58,13 @@ constexpr int SK_KBLOCK = 128; // k elements per wave iteration
 // What a skinny product can take over from the norm kernels around it (decode steps are
 // bound by the number of kernels they start, not by the work of the small ones):
 //   SCALE (with epilogue 0 or 1): x holds rows h * norm_weight that still lack their common
-//     factor rsqrt(mean(h^2) + eps); scale_partials [scale_count][16] holds pieces of every
-//     row's sum of squares (row m at [piece][m]); the factor is applied to the float32 sums.
+//     factor rsqrt(mean(h^2) + eps); scale_partials [scale_count][stride] holds pieces of every
+//     row's sum of squares (row m at [piece][m]; stride: M rounded up to a power of two, so
+//     that every workgroup reads no more of them than it must); the factor is applied to the
+//     float32 sums.
 //   epilogue 2: resid [M, N] is the float32 residual stream: resid += x . w^T in place; the
 //     kernel also leaves next_x = bf16(resid * next_w) and, per workgroup, the sums of squares
-//     of its columns of the new rows in next_partials [gridDim.x][16]: what a SCALE product
+//     of its columns of the new rows in next_partials [gridDim.x][stride]: what a SCALE product
 //     (or rmsnorm) needs to go on without a norm kernel in between.
 struct SkinnyFuse {
     const float* scale_partials;
@@ -72,6 +74,7 @@ struct SkinnyFuse {
     const float* next_w;
     bf16* next_x;
     float* next_partials;
+    int stride;
 };
 constexpr int SK_MAX_PIECES = 512;   // pieces of a sum of squares that a SCALE product reads
 
@@ -97,9 +100,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
     float piece[SK_MAX_PIECES / 64];
     if (SCALE) {
 #pragma unroll
-        for (int i = 0; i < SK_MAX_PIECES / 64; ++i) {
-            const int p = (threadIdx.x >> 4) + 64 * i;
-            piece[i] = p < fuse.scale_count ? fuse.scale_partials[p * 16 + r] : 0.f;
+        for (int i = 0; i < SK_MAX_PIECES / 64; ++i) {   // thread t: row t % stride of pieces t / stride + ...
+            const int at = threadIdx.x + WAVES * 64 * i;
+            piece[i] = at < fuse.scale_count * fuse.stride ? fuse.scale_partials[at] : 0.f;
         }
     }
     // epilogue 2: thread idx < NT * 256 owns the result (m, n) of tile idx / 256
@@ -155,13 +158,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
             for (int v = 0; v < 4; ++v)
                 red[((wave * NT + nt) * MT + mt) * 256 + v * 64 + lane] = acc[nt][mt][v];
     if (SCALE) {
-        // this wave's pieces of the rows' sums of squares: lanes r, r + 16, r + 32, r + 48 hold row r
+        // this wave's pieces of the rows' sums of squares: the lanes l with l % stride = m hold row m
         float sum = 0.f;
 #pragma unroll
         for (int i = 0; i < SK_MAX_PIECES / 64; ++i) sum += piece[i];
-        sum += __shfl_xor(sum, 16, 64);
-        sum += __shfl_xor(sum, 32, 64);
-        if (g == 0) pieces[wave][r] = sum;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1)
+            if (off >= fuse.stride) sum += __shfl_xor(sum, off, 64);
+        if (lane < fuse.stride) pieces[wave][lane] = sum;
     }
     __syncthreads();
     if (EPI == 2) {
@@ -182,19 +186,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
         sq += __shfl_xor(sq, 32, 64);
         if (g == 0) pieces[wave][r] = sq;
         __syncthreads();
-        if (threadIdx.x < 16) {
+        if (threadIdx.x < fuse.stride) {
             float row = 0.f;
 #pragma unroll
             for (int wv = 0; wv < NT * 4; ++wv) row += pieces[wv][threadIdx.x];
-            fuse.next_partials[(size_t)blockIdx.x * 16 + threadIdx.x] = row;
+            fuse.next_partials[(size_t)blockIdx.x * fuse.stride + threadIdx.x] = row;
         }
         return;
     }
     float factor[1] = {1.f};   // of row (threadIdx.x % 16): every result a thread sums is in that row
     if (SCALE) {
         float ss = 0.f;
+        if (r < fuse.stride) {
 #pragma unroll
-        for (int wv = 0; wv < WAVES; ++wv) ss += pieces[wv][r];
+            for (int wv = 0; wv < WAVES; ++wv) ss += pieces[wv][r];
+        }
         factor[0] = rsqrtf(ss / (float)K + fuse.scale_eps);
     }
     if (EPI == 0) {
@@ -790,8 +796,15 @@ LC_API int lc_gemm_bf16(const void* x, const void* w, void* out, int out_dt, int
 // ------------------------------------------------------------------- norms folded into products
 // For steps of up to 16 rows (decode), where a norm kernel costs its start and nothing else.
 // The residual stream h [M, H] is float32.  A "prepared norm" of h for a norm weight g is the
-// pair (xg = bf16(h * g) [M, H], pieces [count][16] of every row's sum of squares): what is
+// pair (xg = bf16(h * g) [M, H], pieces [count][stride] of every row's sum of squares): what is
 // missing is each row's factor rsqrt(mean(h^2) + eps), which a product can apply to its sums.
+// The pieces of row m lie at [piece][m] with lc_gemm_bf16_piece_stride(M) floats per piece.
+
+LC_API int lc_gemm_bf16_piece_stride(int M) {
+    int stride = 1;
+    while (stride < M) stride *= 2;
+    return stride;
+}
 
 // Number of pieces that lc_gemm_bf16_residual writes for these sizes; 0: the fused kernels do
 // not take these sizes (more than 16 rows, K not a multiple of 128, a forced tile shape, more
@@ -803,7 +816,7 @@ LC_API int lc_gemm_bf16_residual_pieces(int M, int N, int K) {
 }
 
 // resid [M, N] += x [M, K] . w [N, K]^T (float32, in place); next_x [M, N] = bf16(resid * next_w);
-// next_pieces [lc_gemm_bf16_residual_pieces(M, N, K)][16]: sums of squares of the new rows.
+// next_pieces [lc_gemm_bf16_residual_pieces(M, N, K)][stride]: sums of squares of the new rows.
 LC_API int lc_gemm_bf16_residual(const void* x, const void* w, float* resid, const float* next_w,
                                  void* next_x, float* next_pieces, int M, int N, int K,
                                  hipStream_t stream) {
@@ -816,6 +829,7 @@ LC_API int lc_gemm_bf16_residual(const void* x, const void* w, float* resid, con
     fuse.next_w = next_w;
     fuse.next_x = (bf16*)next_x;
     fuse.next_partials = next_pieces;
+    fuse.stride = lc_gemm_bf16_piece_stride(M);
     launch_skinny_any<2, false, float>((const bf16*)x, (const bf16*)w, (float*)nullptr, M, N, K, fuse, stream);
     LC_LAUNCH_CHECK("gemm_skinny");
     return 0;
@@ -837,6 +851,7 @@ LC_API int lc_gemm_bf16_scaled_rows(const void* x, const void* w, void* out, int
     fuse.scale_partials = pieces;
     fuse.scale_count = count;
     fuse.scale_eps = eps;
+    fuse.stride = lc_gemm_bf16_piece_stride(M);
     if (epilogue) launch_skinny_any<1, true, bf16>((const bf16*)x, (const bf16*)w, (bf16*)out, M, N, K, fuse, stream);
     else launch_skinny_any<0, true, bf16>((const bf16*)x, (const bf16*)w, (bf16*)out, M, N, K, fuse, stream);
     LC_LAUNCH_CHECK("gemm_skinny");

@@ -30,6 +30,7 @@ _SIGNATURES = {
     "lc_gemm_bf16_supported": "iii",
     "lc_gemm_bf16_force_tile": "i",
     "lc_gemm_bf16_residual_pieces": "iii",
+    "lc_gemm_bf16_piece_stride": "i",
     "lc_gemm_bf16_residual": "ppppppiiip",
     "lc_gemm_bf16_scaled_rows": "pppiiiipifp",
     "lc_qk_norm_rope_write": "piiiiippfppipppip",
@@ -150,8 +151,8 @@ class PendingProduct:
 @dataclass
 class ScaledRows:
     """The normed residual stream short of each row's factor: ``x`` = bf16(h * weight) [T, n];
-    ``pieces`` [count, 16] float32 hold pieces of the rows' sums of squares (row t at
-    [piece, t]); the factor of row t is rsqrt(sum of its pieces / n + eps)."""
+    ``pieces`` [count, T rounded up to a power of two] float32 hold pieces of the rows' sums of
+    squares (row t at [piece, t]); the factor of row t is rsqrt(sum of its pieces / n + eps)."""
 
     x: torch.Tensor
     pieces: torch.Tensor
@@ -191,7 +192,8 @@ def rmsnorm(h: torch.Tensor, delta, weight: torch.Tensor, eps: float,
                   if scaled and delta.w.shape[0] == n and M == T else 0)
         if pieces:
             xg = torch.empty((T, n), dtype=torch.bfloat16, device=h.device)
-            parts = torch.empty((pieces, 16), dtype=torch.float32, device=h.device)
+            parts = torch.empty((pieces, library().lc_gemm_bf16_piece_stride(T)), dtype=torch.float32,
+                                device=h.device)
             _call("lc_gemm_bf16_residual", _ptr(delta.x), _ptr(delta.w), _ptr(h), _ptr(weight),
                   _ptr(xg), _ptr(parts), _c_int(M), _c_int(n), _c_int(K), _stream())
             return ScaledRows(xg, parts, pieces, float(eps), h, weight)
@@ -204,7 +206,8 @@ def rmsnorm(h: torch.Tensor, delta, weight: torch.Tensor, eps: float,
         _need(rows, "rmsnorm rows", torch.int32, 1)
     R = T if rows is None else rows.shape[0]
     out = torch.empty((R, n), dtype=out_dtype, device=h.device)
-    parts = torch.empty((1, 16), dtype=torch.float32, device=h.device) if scaled else None
+    parts = (torch.empty((1, library().lc_gemm_bf16_piece_stride(T)), dtype=torch.float32, device=h.device)
+             if scaled else None)
     _call("lc_rmsnorm", _ptr(h), _ptr(delta), _ptr(rows), _ptr(weight), _c_float(eps), _ptr(out),
           _c_int(_dt(out)), _c_int(R), _c_int(n),
           _c_int(1 if (rows is None and delta is not None) else 0), _ptr(parts), _stream())
