@@ -78,22 +78,42 @@ struct SkinnyFuse {
 };
 constexpr int SK_MAX_PIECES = 512;   // pieces of a sum of squares that a SCALE product reads
 
-// MT: tiles of 16 rows of x; NT: tiles of 16 rows of w per workgroup; the WAVES waves of a
-// workgroup take the k blocks in turn.
-template <int MT, int NT, int WAVES, int UNROLL, int EPI, bool SCALE, typename TO>
+// the k blocks of one tile's rows of w that a wave works on (a block past the end is loaded, not used)
+template <int XR, int WAVES>
+__device__ __forceinline__ void load_w_blocks(bf16x8 (&a)[XR][4], const bf16* wp, int wave, int kblocks) {
+#pragma unroll
+    for (int i = 0; i < XR; ++i) {
+        const int kb = min(wave + i * WAVES, kblocks - 1);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) a[i][j] = *reinterpret_cast<const bf16x8*>(wp + kb * SK_KBLOCK + j * 32);
+    }
+}
+
+// MT: tiles of 16 rows of x; NT: tiles of 16 rows of w per workgroup tile; the WAVES waves of a
+// workgroup take the k blocks in turn.  A workgroup takes the tiles blockIdx.x, blockIdx.x +
+// gridDim.x, ...  XR = 0: one tile per workgroup is the intended use, and x is read as it is
+// needed.  XR > 0 (K <= XR * WAVES * 128): every wave keeps the part of x that its k blocks
+// need in registers for all of its workgroup's tiles.  Every workgroup has to fetch x through
+// its CU's path from L2, which is what bounds this kernel from a few rows of x on: with three
+// tiles per workgroup, x costs a third.
+template <int MT, int NT, int WAVES, int UNROLL, int EPI, bool SCALE, int XR, typename TO>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __restrict__ x,
                                                                  const bf16* __restrict__ w,
                                                                  TO* __restrict__ out, int M, int N,
                                                                  int K, SkinnyFuse fuse) {
     static_assert(WAVES == 16, "the epilogues lay 1024 threads over a workgroup's results");
-    static_assert(!(SCALE || EPI == 2) || MT == 1, "fused norms are for up to 16 rows");
-    static_assert(EPI != 2 || NT <= 4, "epilogue 2 gives every result a thread of its own");
+    static_assert(MT == 1, "up to 16 rows of x");
     static_assert(!(SCALE && EPI == 2), "both would use the same words of LDS");
-    __shared__ float red[WAVES * MT * NT * 256];
+    static_assert(XR == 0 || NT == 1, "x stays in registers for single tiles only");
+    // a wave's sums of one tile take RS floats: 256 and a pad that puts the four quarters of
+    // the waves, which the epilogue's lanes read side by side, on different banks
+    constexpr int RS = 256 + 4;
+    __shared__ float red[WAVES * NT * RS];
     __shared__ float pieces[WAVES][16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * (16 * NT);
+    const int tiles = (N + 16 * NT - 1) / (16 * NT);
+    const int kblocks = K / SK_KBLOCK;
 
     // loads whose values are wanted only after the products; issued first, they are back
     // before the first operand is
@@ -105,130 +125,193 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
             piece[i] = at < fuse.scale_count * fuse.stride ? fuse.scale_partials[at] : 0.f;
         }
     }
-    // epilogue 2: thread idx < NT * 256 owns the result (m, n) of tile idx / 256
-    const int e_tile = threadIdx.x >> 8, e_v = (threadIdx.x >> 6) & 3;
-    const int e_m = r, e_n = n0 + e_tile * 16 + g * 4 + e_v;
-    const bool e_mine = EPI == 2 && threadIdx.x < NT * 256 && e_m < M && e_n < N;
-    float e_resid = 0.f, e_w = 0.f;
-    if (e_mine) {
-        e_resid = fuse.resid[(size_t)e_m * N + e_n];
-        e_w = fuse.next_w[e_n];
-    }
-
-    const bf16* wp[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) wp[nt] = w + (size_t)min(n0 + nt * 16 + r, N - 1) * K + g * 8;
-    const bf16* xp[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) xp[mt] = x + (size_t)min(mt * 16 + r, M - 1) * K + g * 8;
-
-    floatx4 acc[NT][MT];
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-    const int kblocks = K / SK_KBLOCK;
-#pragma unroll UNROLL
-    for (int kb = wave; kb < kblocks; kb += WAVES) {
-        const int k0 = kb * SK_KBLOCK;
-        bf16x8 a[NT][4];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) a[nt][j] = *reinterpret_cast<const bf16x8*>(wp[nt] + k0 + j * 32);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            bf16x8 b[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) b[j] = *reinterpret_cast<const bf16x8*>(xp[mt] + k0 + j * 32);
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][j], b[j], acc[nt][mt], 0, 0, 0);
-        }
-    }
-    // acc[nt][mt][v] = partial out[m = mt*16 + lane%16][n = n0 + nt*16 + (lane/16)*4 + v]
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int v = 0; v < 4; ++v)
-                red[((wave * NT + nt) * MT + mt) * 256 + v * 64 + lane] = acc[nt][mt][v];
-    if (SCALE) {
-        // this wave's pieces of the rows' sums of squares: the lanes l with l % stride = m hold row m
-        float sum = 0.f;
+    // the rows' sums of squares go through LDS: each wave leaves its pieces' sums there ...
+    auto leave_pieces = [&]() {
+        float sum = 0.f;       // the lanes l with l % stride = m hold row m
 #pragma unroll
         for (int i = 0; i < SK_MAX_PIECES / 64; ++i) sum += piece[i];
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1)
             if (off >= fuse.stride) sum += __shfl_xor(sum, off, 64);
         if (lane < fuse.stride) pieces[wave][lane] = sum;
-    }
-    __syncthreads();
-    if (EPI == 2) {
-        float total = 0.f;
-        if (threadIdx.x < NT * 256) {
-#pragma unroll
-            for (int wv = 0; wv < WAVES; ++wv) total += red[wv * NT * 256 + threadIdx.x];
-        }
-        float sq = 0.f;
-        if (e_mine) {
-            const float v = e_resid + total;
-            fuse.resid[(size_t)e_m * N + e_n] = v;
-            fuse.next_x[(size_t)e_m * N + e_n] = static_cast<bf16>(v * e_w);
-            sq = v * v;
-        }
-        // a row's squares: over the wave's four column groups, then over the waves that hold results
-        sq += __shfl_xor(sq, 16, 64);
-        sq += __shfl_xor(sq, 32, 64);
-        if (g == 0) pieces[wave][r] = sq;
-        __syncthreads();
-        if (threadIdx.x < fuse.stride) {
-            float row = 0.f;
-#pragma unroll
-            for (int wv = 0; wv < NT * 4; ++wv) row += pieces[wv][threadIdx.x];
-            fuse.next_partials[(size_t)blockIdx.x * fuse.stride + threadIdx.x] = row;
-        }
-        return;
-    }
-    float factor[1] = {1.f};   // of row (threadIdx.x % 16): every result a thread sums is in that row
-    if (SCALE) {
+    };
+    // ... and, after a barrier, every lane gets the factor of row r
+    auto row_factor = [&]() {
         float ss = 0.f;
         if (r < fuse.stride) {
 #pragma unroll
             for (int wv = 0; wv < WAVES; ++wv) ss += pieces[wv][r];
         }
-        factor[0] = rsqrtf(ss / (float)K + fuse.scale_eps);
+        return rsqrtf(ss / (float)K + fuse.scale_eps);
+    };
+    float factor = 1.f;
+    if (SCALE && XR > 0) {   // a workgroup of many tiles waits for them once, and needs the registers
+        leave_pieces();
+        __syncthreads();
+        factor = row_factor();
     }
-    if (EPI == 0) {
-        for (int idx = threadIdx.x; idx < NT * MT * 256; idx += WAVES * 64) {
-            float total = 0.f;
+    const bf16* xp[MT];
 #pragma unroll
-            for (int wv = 0; wv < WAVES; ++wv) total += red[wv * NT * MT * 256 + idx];
-            const int tile = idx >> 8, v = (idx >> 6) & 3, l = idx & 63;
-            const int nt = tile / MT, mt = tile % MT;
-            const int m = mt * 16 + (l & 15), n = n0 + nt * 16 + (l >> 4) * 4 + v;
-            if (m < M && n < N) store_out<TO>(out + (size_t)m * N + n, total * factor[0]);
+    for (int mt = 0; mt < MT; ++mt) xp[mt] = x + (size_t)min(mt * 16 + r, M - 1) * K + g * 8;
+    bf16x8 xb[XR > 0 ? XR : 1][4];
+    if (XR > 0) {
+#pragma unroll
+        for (int i = 0; i < XR; ++i) {
+            const int kb = min(wave + i * WAVES, kblocks - 1);   // a block past the end is loaded, not used
+#pragma unroll
+            for (int j = 0; j < 4; ++j) xb[i][j] = *reinterpret_cast<const bf16x8*>(xp[0] + kb * SK_KBLOCK + j * 32);
+        }
+    }
+
+    // XR of 1 or 2: registers are left for the next tile's part of w as well
+    constexpr bool AHEAD = XR == 1 || XR == 2;
+    bf16x8 a_now[XR > 0 ? XR : 1][4], a_next[XR > 0 ? XR : 1][4];
+    bool first = true;
+    // one tile: its rows of w are in a_use (XR > 0 with AHEAD) or loaded here; a_fill takes the next tile's
+    auto one_tile = [&](const int tile, bf16x8 (&a_use)[XR > 0 ? XR : 1][4], bf16x8 (&a_fill)[XR > 0 ? XR : 1][4]) {
+        const int n0 = tile * (16 * NT);
+        // The epilogue's layout: wave q and lane (row m = lane % 16, quarter = lane / 16) add up,
+        // over the waves 4 quarter .. 4 quarter + 3, the sums for row m and column
+        // n0 + 16 nt + 4 (q % 4) + q / 4; the quarters then meet by two lane exchanges, and the
+        // lanes of quarter 0 own the result.
+        const int e_n = n0 + (wave & 3) * 4 + (wave >> 2);
+        float e_resid[NT], e_w[NT];
+        if (EPI == 2) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const bool mine = g == 0 && r < M && e_n + nt * 16 < N;
+                e_resid[nt] = mine ? fuse.resid[(size_t)r * N + e_n + nt * 16] : 0.f;
+                e_w[nt] = mine ? fuse.next_w[e_n + nt * 16] : 0.f;
+            }
+        }
+
+        const bf16* wp[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) wp[nt] = w + (size_t)min(n0 + nt * 16 + r, N - 1) * K + g * 8;
+
+        floatx4 acc[NT][MT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+        if constexpr (XR > 0) {
+            if (!AHEAD) load_w_blocks<XR, WAVES>(a_use, wp[0], wave, kblocks);
+            if (AHEAD && tile + gridDim.x < tiles) {
+                // the next tile's rows of w are on their way while this tile's sums meet in LDS
+                const int n_next = (tile + gridDim.x) * 16;
+                load_w_blocks<XR, WAVES>(a_fill, w + (size_t)min(n_next + r, N - 1) * K + g * 8, wave, kblocks);
+            }
+#pragma unroll
+            for (int i = 0; i < XR; ++i) {
+                if (wave + i * WAVES < kblocks) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_use[i][j], xb[i][j], acc[0][0], 0, 0, 0);
+                }
+            }
+        } else {
+#pragma unroll UNROLL
+            for (int kb = wave; kb < kblocks; kb += WAVES) {
+                const int k0 = kb * SK_KBLOCK;
+                bf16x8 a[NT][4];
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) a[nt][j] = *reinterpret_cast<const bf16x8*>(wp[nt] + k0 + j * 32);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    bf16x8 b[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) b[j] = *reinterpret_cast<const bf16x8*>(xp[mt] + k0 + j * 32);
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][j], b[j], acc[nt][mt], 0, 0, 0);
+                }
+            }
+        }
+        // acc[nt][0][v] = partial out[m = lane%16][n = n0 + nt*16 + (lane/16)*4 + v], kept at [v * 64 + lane]
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) red[(wave * NT + nt) * RS + v * 64 + lane] = acc[nt][0][v];
+        if (SCALE && XR == 0 && first) leave_pieces();
+        first = false;
+        __syncthreads();
+        // element e of a tile's 256 sums, over all waves (every lane of the four quarters gets it)
+        auto total_of = [&](int nt, int e) {
+            float t = 0.f;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) t += red[((g * 4 + k) * NT + nt) * RS + e];
+            t += __shfl_xor(t, 16, 64);
+            t += __shfl_xor(t, 32, 64);
+            return t;
+        };
+        const int e_mine = wave * 16 + r;     // = v * 64 + (lane of the product) with v = wave / 4
+        if (EPI == 2) {
+            float sq = 0.f;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const float t = total_of(nt, e_mine);
+                if (g == 0 && r < M && e_n + nt * 16 < N) {
+                    const float v = e_resid[nt] + t;
+                    fuse.resid[(size_t)r * N + e_n + nt * 16] = v;
+                    fuse.next_x[(size_t)r * N + e_n + nt * 16] = static_cast<bf16>(v * e_w[nt]);
+                    sq += v * v;
+                }
+            }
+            // a row's squares: every wave holds one column of each of the tile's blocks of 16
+            if (g == 0) pieces[wave][r] = sq;
+            __syncthreads();
+            if (threadIdx.x < fuse.stride) {
+                float row = 0.f;
+#pragma unroll
+                for (int wv = 0; wv < WAVES; ++wv) row += pieces[wv][threadIdx.x];
+                fuse.next_partials[(size_t)tile * fuse.stride + threadIdx.x] = row;
+            }
+        } else {
+            if (SCALE && XR == 0) factor = row_factor();
+            if (EPI == 0) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const float t = total_of(nt, e_mine);
+                    const int n = e_n + nt * 16;
+                    if (g == 0 && r < M && n < N) store_out<TO>(out + (size_t)r * N + n, t * factor);
+                }
+            } else {
+                // rows of w come in blocks of 16: 8 gate rows, then their 8 up rows; out has N / 2
+                // columns.  The waves with q % 4 < 2 hold gate rows; the up row of each is two
+                // waves (32 elements) further on.
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    if ((wave & 3) < 2) {
+                        const float gate = total_of(nt, e_mine), up = total_of(nt, e_mine + 32);
+                        const int n = e_n + nt * 16;
+                        const int col = (n >> 4) * 8 + (n & 7);
+                        if (g == 0 && r < M && n < N)
+                            store_out<TO>(out + (size_t)r * (N / 2) + col, swiglu_f(gate * factor, up * factor));
+                    }
+                }
+            }
+        }
+        if (tile + gridDim.x < tiles) __syncthreads();   // red and pieces are written again
+    };
+    if constexpr (AHEAD) {
+        // two sets of registers take turns, so that no value has to be moved (a move would
+        // wait for the loads that are meant to stay in flight)
+        int tile = blockIdx.x;
+        if (tile < tiles) load_w_blocks<XR, WAVES>(a_now, w + (size_t)min(tile * 16 + r, N - 1) * K + g * 8, wave, kblocks);
+        while (tile < tiles) {
+            one_tile(tile, a_now, a_next);
+            tile += gridDim.x;
+            if (tile >= tiles) break;
+            one_tile(tile, a_next, a_now);
+            tile += gridDim.x;
         }
     } else {
-        // rows of w come in blocks of 16: 8 gate rows, then their 8 up rows; out has N / 2 columns
-        for (int idx = threadIdx.x; idx < NT * MT * 128; idx += WAVES * 64) {
-            const int tile = idx >> 7, v = (idx >> 5) & 3, l = idx & 31;   // l: lane of the gate half
-            const int gi = tile * 256 + v * 64 + l, ui = gi + 32;
-            float g = 0.f, u = 0.f;
-#pragma unroll
-            for (int wv = 0; wv < WAVES; ++wv) {
-                g += red[wv * NT * MT * 256 + gi];
-                u += red[wv * NT * MT * 256 + ui];
-            }
-            const int nt = tile / MT, mt = tile % MT;
-            const int m = mt * 16 + (l & 15), n = n0 + nt * 16 + (l >> 4) * 4 + v;   // gate row, n % 16 < 8
-            const int col = (n >> 4) * 8 + (n & 7);
-            if (m < M && n < N) store_out<TO>(out + (size_t)m * (N / 2) + col, swiglu_f(g * factor[0], u * factor[0]));
-        }
+        for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x) one_tile(tile, a_now, a_now);
     }
 }
 
@@ -654,35 +737,54 @@ static long long workspace_words(int M, int N, int K) {
     return 0;
 }
 
-template <int MT, int NT, int WAVES, int UNROLL, int EPI, bool SCALE, typename TO>
+template <int MT, int NT, int WAVES, int UNROLL, int EPI, bool SCALE, int XR, typename TO>
 static void launch_skinny(const bf16* x, const bf16* w, TO* out, int M, int N, int K, SkinnyFuse fuse,
-                          hipStream_t s) {
-    const int rows = 16 * NT;
-    gemm_skinny_kernel<MT, NT, WAVES, UNROLL, EPI, SCALE, TO><<<(N + rows - 1) / rows, WAVES * 64, 0, s>>>(
+                          int workgroups, hipStream_t s) {
+    gemm_skinny_kernel<MT, NT, WAVES, UNROLL, EPI, SCALE, XR, TO><<<workgroups, WAVES * 64, 0, s>>>(
         x, w, out, M, N, K, fuse);
 }
 
 // The skinny kernel's shape for M <= 16 rows.  Measured: with one or two rows of x a deeper
-// unroll keeps more of w in flight; from about 12 rows on, x costs as much to fetch as w, and
-// two row tiles per workgroup share it (only where that still leaves every CU two workgroups).
-enum : int { SKINNY_DEEP = 0, SKINNY_PLAIN = 1, SKINNY_WIDE = 2 };
-static int skinny_shape(int M, int N) {
+// unroll keeps more of w in flight.  From a few rows on, fetching x costs a good part of what w
+// costs: where there are more tiles than CUs and K allows it, one workgroup a CU takes several
+// tiles and keeps x in registers (its registers leave room for one workgroup a CU only, which
+// costs more than x does below 7 rows, unless the tiles are so few that the plain shape would
+// not fill the CUs twice); else, from about 12 rows on, two row tiles per workgroup share x
+// (only where that still leaves every CU two workgroups).
+enum : int { SKINNY_DEEP = 0, SKINNY_PLAIN = 1, SKINNY_WIDE = 2, SKINNY_KEEP_X = 3 };
+constexpr int SK_KEEP_MAX = 3;   // k blocks of x per wave that fit in registers beside w's
+static int g_force_skinny = -1;
+static int skinny_shape(int M, int N, int K) {
+    if (g_force_skinny >= 0 && (g_force_skinny != SKINNY_KEEP_X || K <= SK_KEEP_MAX * 16 * SK_KBLOCK))
+        return g_force_skinny;
     if (M <= 2) return SKINNY_DEEP;
+    const int tiles = (N + 15) / 16;
+    if (K <= SK_KEEP_MAX * 16 * SK_KBLOCK && tiles > kCUs && (M >= 7 || tiles <= 2 * kCUs)) return SKINNY_KEEP_X;
     if (M >= 12 && N >= 32 * 2 * kCUs) return SKINNY_WIDE;
     return SKINNY_PLAIN;
 }
-static int skinny_workgroups(int M, int N) {
-    const int rows = skinny_shape(M, N) == SKINNY_WIDE ? 32 : 16;
+// number of tiles, which is also the number of pieces that epilogue 2 writes
+static int skinny_tiles(int M, int N, int K) {
+    const int rows = skinny_shape(M, N, K) == SKINNY_WIDE ? 32 : 16;
     return (N + rows - 1) / rows;
 }
 
 template <int EPI, bool SCALE, typename TO>
 static void launch_skinny_any(const bf16* x, const bf16* w, TO* out, int M, int N, int K, SkinnyFuse fuse,
                               hipStream_t s) {
-    switch (skinny_shape(M, N)) {
-    case SKINNY_DEEP: launch_skinny<1, 1, 16, 4, EPI, SCALE, TO>(x, w, out, M, N, K, fuse, s); break;
-    case SKINNY_WIDE: launch_skinny<1, 2, 16, 2, EPI, SCALE, TO>(x, w, out, M, N, K, fuse, s); break;
-    default:          launch_skinny<1, 1, 16, 2, EPI, SCALE, TO>(x, w, out, M, N, K, fuse, s); break;
+    const int tiles = skinny_tiles(M, N, K);
+    switch (skinny_shape(M, N, K)) {
+    case SKINNY_DEEP: launch_skinny<1, 1, 16, 4, EPI, SCALE, 0, TO>(x, w, out, M, N, K, fuse, tiles, s); break;
+    case SKINNY_WIDE: launch_skinny<1, 2, 16, 2, EPI, SCALE, 0, TO>(x, w, out, M, N, K, fuse, tiles, s); break;
+    case SKINNY_KEEP_X: {
+        const int groups = tiles < kCUs ? tiles : kCUs, per_wave = (K / SK_KBLOCK + 15) / 16;   // one a CU fits
+
+        if (per_wave == 1) launch_skinny<1, 1, 16, 1, EPI, SCALE, 1, TO>(x, w, out, M, N, K, fuse, groups, s);
+        else if (per_wave == 2) launch_skinny<1, 1, 16, 1, EPI, SCALE, 2, TO>(x, w, out, M, N, K, fuse, groups, s);
+        else launch_skinny<1, 1, 16, 1, EPI, SCALE, 3, TO>(x, w, out, M, N, K, fuse, groups, s);
+        break;
+    }
+    default:          launch_skinny<1, 1, 16, 2, EPI, SCALE, 0, TO>(x, w, out, M, N, K, fuse, tiles, s); break;
     }
 }
 
@@ -755,6 +857,15 @@ LC_API int lc_gemm_bf16_supported(int M, int N, int K) {
     return 1;
 }
 
+// Forces the shape of the skinny kernel for every later product of up to 16 rows (0: deep
+// unroll, 1: plain, 2: two row tiles of w a workgroup, 3: several tiles a workgroup with x kept
+// in registers, where K allows it; -1: choose by size again).  For tests and tuning.
+LC_API int lc_gemm_bf16_force_skinny(int shape) {
+    LC_CHECK(shape >= -1 && shape <= SKINNY_KEEP_X, "gemm_bf16: no skinny shape %d", shape);
+    g_force_skinny = shape;
+    return 0;
+}
+
 // Forces the tile shape of the tiled kernel for every later product of any M (-1: choose by
 // size again).  For tests and tuning; not for use while other threads launch products.
 LC_API int lc_gemm_bf16_force_tile(int tile) {
@@ -811,7 +922,7 @@ LC_API int lc_gemm_bf16_piece_stride(int M) {
 // pieces than a scaled product reads).
 LC_API int lc_gemm_bf16_residual_pieces(int M, int N, int K) {
     if (!lc_gemm_bf16_supported(M, N, K) || M > 16 || g_force_tile != TILE_AUTO) return 0;
-    const int pieces = skinny_workgroups(M, N);
+    const int pieces = skinny_tiles(M, N, K);
     return pieces <= SK_MAX_PIECES ? pieces : 0;
 }
 

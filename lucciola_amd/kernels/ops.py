@@ -29,6 +29,7 @@ _SIGNATURES = {
     "lc_gemm_bf16": "pppiiiiipp",
     "lc_gemm_bf16_supported": "iii",
     "lc_gemm_bf16_force_tile": "i",
+    "lc_gemm_bf16_force_skinny": "i",
     "lc_gemm_bf16_residual_pieces": "iii",
     "lc_gemm_bf16_piece_stride": "i",
     "lc_gemm_bf16_residual": "ppppppiiip",
@@ -320,6 +321,13 @@ def force_gemm_tile(tile: int) -> None:
     """Make the tiled bfloat16 product use one tile shape for every size (0: 64x128, 1: 128x128,
     2: 256x128, 3: 256x192, 4: 256x256; -1: choose by size again).  For tests and tuning."""
     _call("lc_gemm_bf16_force_tile", _c_int(tile))
+
+
+def force_gemm_skinny(shape: int) -> None:
+    """Make the bfloat16 product of up to 16 rows use one shape of its kernel (0: deep unroll,
+    1: plain, 2: two row tiles a workgroup, 3: several tiles a workgroup with x in registers;
+    -1: choose by size again).  For tests and tuning."""
+    _call("lc_gemm_bf16_force_skinny", _c_int(shape))
 
 
 def _fast_gemm_ok(M: int, N: int, K: int) -> bool:

@@ -297,7 +297,7 @@ def test_gemm_bf16_last_round_cut_along_k(tile, M, N, K):
 
 
 @pytest.mark.parametrize("M,H,K,N2", [(1, 128, 128, 48), (2, 384, 256, 1000), (5, 256, 640, 272), (8, 4096, 512, 2064),
-                                      (11, 640, 128, 16), (12, 16384, 128, 16416), (16, 1152, 384, 130)])
+                                      (11, 640, 128, 16), (12, 16384, 6272, 16416), (12, 8192, 128, 48), (16, 1152, 384, 130)])
 def test_norm_folded_into_the_products_around_it(M, H, K, N2):
     """Up to 16 rows: the product before a norm adds its result to the stream and leaves
     bf16(h * weight) and the pieces of the rows' sums of squares; the product after it applies
@@ -466,3 +466,36 @@ def test_attention_window_edge(dtype, d, page, new):
             assert float((got - 7.0).abs().max()) < 0.1
         else:
             assert float(got.abs().max()) < 5.0          # a mix of ordinary values, not the marked one
+
+
+@pytest.mark.parametrize("shape", [-1, 0, 1, 2, 3])
+@pytest.mark.parametrize("M,N,K", [(3, 8240, 128), (8, 16400, 512), (16, 8208, 4096), (5, 9000, 5120), (9, 24576, 6144),
+                                   (1, 48, 256), (7, 4112, 1024)])
+def test_gemm_bf16_few_rows_every_shape(M, N, K, shape):
+    """Every shape of the kernel for up to 16 rows, chosen by size and forced; among the sizes,
+    more column tiles than the CUs hold workgroups, where a workgroup takes several tiles and
+    its waves keep their part of x in registers (one, two or three k blocks a wave, the last
+    ones partly unused).  Plain, with the SwiGLU epilogue, with scaled rows, float32 output."""
+    ops.force_gemm_skinny(shape)
+    try:
+        few_rows_case(M, N, K)
+    finally:
+        ops.force_gemm_skinny(-1)
+
+
+def few_rows_case(M, N, K):
+    x = rnd(M, K, dtype=torch.bfloat16, seed=80)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=81, scale=K ** -0.5)
+    want = x.double() @ w.double().T
+    close(ops.gemm(x, w, torch.float32), want.float(), torch.float32, scale=4.0)
+    close(ops.gemm(x, w, torch.bfloat16), want.to(torch.bfloat16), torch.bfloat16, scale=2.0)
+    even = N // 16 * 16
+    blocks = want[:, :even].reshape(M, -1, 2, 8)
+    gate, up = blocks[:, :, 0, :].reshape(M, -1), blocks[:, :, 1, :].reshape(M, -1)
+    close(ops.gemm_swiglu(x, w[:even]), (gate / (1 + torch.exp(-gate)) * up).to(torch.bfloat16), torch.bfloat16, scale=2.0)
+    h = rnd(M, K, seed=82, scale=1.5)
+    g = 1 + rnd(K, seed=83, scale=0.2)
+    rows = ops.rmsnorm(h, None, g, 1e-6, torch.bfloat16, scaled=True)
+    factors = torch.rsqrt((h.double() ** 2).mean(1, keepdim=True) + 1e-6)
+    close(ops.gemm(rows, w, torch.bfloat16), ((rows.x.double() @ w.double().T) * factors).to(torch.bfloat16),
+          torch.bfloat16, scale=2.0)
