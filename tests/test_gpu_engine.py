@@ -72,10 +72,10 @@ def random_configuration(seed):
     group = rng.choice([1, 2, 3, 4, 5, 6, 8])
     cfg = {
         "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
-        "num_hidden_layers": layers, "hidden_size": rng.choice([24, 40, 75, 100, 136, 200]),
+        "num_hidden_layers": layers, "hidden_size": rng.choice([24, 40, 75, 100, 128, 136, 200, 256]),
         "num_attention_heads": kv * group, "num_key_value_heads": kv,
         "head_dim": rng.choice([16, 32, 48, 64, 80, 96, 112, 128]),
-        "intermediate_size": rng.choice([16, 57, 88, 130, 256, 301]),
+        "intermediate_size": rng.choice([16, 57, 88, 128, 130, 256, 301, 384]),
         "vocab_size": rng.randint(50, 700),
         "rope_theta": rng.choice([10000.0, 50000.0, 1000000.0]),
         "rms_norm_eps": rng.choice([1e-6, 3e-6, 1e-5]),
@@ -94,7 +94,7 @@ def random_configuration(seed):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("seed", range(8))
+@pytest.mark.parametrize("seed", range(12))
 def test_random_configurations(seed, dtype):
     """Configurations drawn at random, replayed mixed (pages used again) and with a decoded
     tail: sizes that no fixed test names must give right results too, through whichever kernel
