@@ -357,7 +357,8 @@ __global__ __launch_bounds__(128) void attn_decode_join_kernel(const float* __re
 }
 
 // ------------------------------------------------------------------------------- prefill
-// tiles: [NT, 4] = (request, first token row, rows (<= 64), position of the first row).
+// tiles: [NT, 4] = (request, first token row, rows (<= 64), position of the first row), the
+// tiles that see the fewest keys first.
 // A workgroup takes one tile and HPW heads of one kv head and walks the pages the tile can
 // see, PF_NP pages (64 keys) at a time.  Its 256 threads bring a group of pages into LDS
 // together (the next group's loads are in flight in registers meanwhile), and every wave
@@ -369,6 +370,7 @@ __global__ __launch_bounds__(128) void attn_decode_join_kernel(const float* __re
 // Key rows are padded by 16 bytes in LDS, which spreads the 16 keys of an operand read over
 // all banks; value pages are interleaved in pairs and rotated for the same reason.
 constexpr int PF_NP = 4;   // even: value pages go to LDS in pairs
+
 
 template <int D, int HPW>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
@@ -384,14 +386,25 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     __shared__ __attribute__((aligned(16))) bf16 ks[2][NP * KPAGE];
     __shared__ __attribute__((aligned(16))) bf16 vs[2][NP * VPAGE];
 
-    const int* tile = tiles + (size_t)blockIdx.x * 4;
+    // Which tile and which heads.  Workgroups start in the order of their number (x fastest)
+    // and two fit on a CU; the tiles come shortest first, and a tile's heads are neighbours, so
+    // that the workgroups that read the same keys and values run at the same time.  Measured:
+    // with more workgroups than fit at once, shortest first is the fastest order (the long ones
+    // at the end all take about as long as each other); when all fit at once, nobody takes over
+    // from a CU that is done early, and the second workgroup of a CU should be as long as its
+    // first is short: the second half of the numbers takes the tasks from the longest down.
+    const int total = gridDim.x * gridDim.y, number = blockIdx.y * gridDim.x + blockIdx.x;
+    const int half = (total + 1) / 2;
+    const int task = (total <= 2 * 256 && number >= half) ? total - 1 - (number - half) : number;
+    const int tile_index = task / gridDim.y, heads_index = task - tile_index * gridDim.y;
+    const int* tile = tiles + (size_t)tile_index * 4;
     const int req = tile[0], row0 = tile[1], rows = tile[2], pos0 = tile[3];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int q = lane & 15, kg = lane >> 4;
     const int G = nh / nkv;
-    const int h = HPW == 2 ? blockIdx.y * 2 + (wave >> 1) : blockIdx.y;
+    const int h = HPW == 2 ? heads_index * 2 + (wave >> 1) : heads_index;
     const int wrow = HPW == 2 ? (wave & 1) * 32 : wave * 16;
-    const int kvh = (blockIdx.y * HPW) / G;
+    const int kvh = (heads_index * HPW) / G;
     const bool active = h < nh && wrow < rows;
     const int* table = block_table + (size_t)req * max_blocks;
 
