@@ -43,21 +43,30 @@ __global__ void embedding_kernel(const int* __restrict__ ids, const TW* __restri
 //   v = h[src] (+ delta[src]);  if (write_h) h[src] = v;  out[r] = v * rsqrt(mean(v^2)+eps) * w
 // With sumsq: out[r] = v * w and sumsq[r] = sum(v^2): the row's factor is left to the product
 // that reads out (gemm_bf16.hip, scaled rows).
+// With shares > 0, delta is not a tensor of T but float32 [shares][all rows of h][n]: the shares
+// of a product that was cut along K (gemm_bf16.hip), added here in their order.
 template <typename T>
 __global__ void rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delta,
                                const int* __restrict__ rows, const float* __restrict__ w,
                                float eps, T* __restrict__ out, int n, int write_h,
-                               float* __restrict__ sumsq) {
+                               float* __restrict__ sumsq, int shares, size_t share_stride) {
     __shared__ float scratch[16];
     const int r = blockIdx.x;
     const int src = rows ? rows[r] : r;
     float* hr = h + (size_t)src * n;
-    const T* dr = delta ? delta + (size_t)src * n : nullptr;
+    const T* dr = (delta && !shares) ? delta + (size_t)src * n : nullptr;
+    const float* pr = shares ? reinterpret_cast<const float*>(delta) + (size_t)src * n : nullptr;
+    auto branch = [&](int i) {
+        if (dr) return to_f32(dr[i]);
+        float t = 0.f;
+        for (int s = 0; s < shares; ++s) t += pr[s * share_stride + i];
+        return t;
+    };
     float ss = 0.f;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
         float v = hr[i];
-        if (dr) {
-            v += to_f32(dr[i]);
+        if (dr || pr) {
+            v += branch(i);
             if (write_h) hr[i] = v;
         }
         ss += v * v;
@@ -68,7 +77,7 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delt
     T* o = out + (size_t)r * n;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
         float v = hr[i];
-        if (dr && !write_h) v += to_f32(dr[i]);
+        if ((dr || pr) && !write_h) v += branch(i);
         o[i] = from_f32<T>(v * inv * w[i]);
     }
 }
@@ -96,12 +105,13 @@ template <typename T>
 __global__ __launch_bounds__(RN_THREADS) void rmsnorm_vec_kernel(
     float* __restrict__ h, const T* __restrict__ delta, const int* __restrict__ rows,
     const float* __restrict__ w, float eps, T* __restrict__ out, int n, int write_h,
-    float* __restrict__ sumsq) {
+    float* __restrict__ sumsq, int shares, size_t share_stride) {
     __shared__ float scratch[16];
     const int r = blockIdx.x;
     const int src = rows ? rows[r] : r;
     float* hr = h + (size_t)src * n;
-    const T* dr = delta ? delta + (size_t)src * n : nullptr;
+    const T* dr = (delta && !shares) ? delta + (size_t)src * n : nullptr;
+    const float* pr = shares ? reinterpret_cast<const float*>(delta) + (size_t)src * n : nullptr;
     const int chunks = n / 8;
     Pack8<float> hv[RN_CHUNKS];
     Pack8<T> dv[RN_CHUNKS];
@@ -111,6 +121,22 @@ __global__ __launch_bounds__(RN_THREADS) void rmsnorm_vec_kernel(
         if (chunk < chunks) {
             hv[c] = *reinterpret_cast<const Pack8<float>*>(hr + chunk * 8);
             if (dr) dv[c] = *reinterpret_cast<const Pack8<T>*>(dr + chunk * 8);
+        }
+    }
+    if (pr) {   // the shares of the branch's product, in their order, then the stream
+#pragma unroll
+        for (int c = 0; c < RN_CHUNKS; ++c) {
+            const int chunk = threadIdx.x + c * RN_THREADS;
+            if (chunk < chunks) {
+                Pack8<float> sum = *reinterpret_cast<const Pack8<float>*>(pr + chunk * 8);
+                for (int s = 1; s < shares; ++s) {
+                    const Pack8<float> part = *reinterpret_cast<const Pack8<float>*>(pr + s * share_stride + chunk * 8);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) sum.set(i, sum.get(i) + part.get(i));
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) hv[c].set(i, hv[c].get(i) + sum.get(i));
+            }
         }
     }
     float ss = 0.f;
@@ -125,7 +151,7 @@ __global__ __launch_bounds__(RN_THREADS) void rmsnorm_vec_kernel(
                 hv[c].set(i, v);
                 ss += v * v;
             }
-            if (dr && write_h) *reinterpret_cast<Pack8<float>*>(hr + chunk * 8) = hv[c];
+            if ((dr || pr) && write_h) *reinterpret_cast<Pack8<float>*>(hr + chunk * 8) = hv[c];
         }
     }
     ss = block_sum(ss, scratch);
@@ -316,8 +342,13 @@ LC_API int lc_embedding(const int* ids, const void* table, int table_dt, float* 
 
 // sumsq (may be null): R floats; then out = (h + delta) * w without the rows' factors, and
 // sumsq[r] = the row's sum of squares.
+// shares > 0: delta is float32 [shares][h_rows][n], the shares of a product cut along K; what
+// is added to h is their sum in the order of the shares.
 LC_API int lc_rmsnorm(float* h, const void* delta, const int* rows, const float* w, float eps,
-                      void* out, int dt, int R, int n, int write_h, float* sumsq, hipStream_t stream) {
+                      void* out, int dt, int R, int n, int write_h, float* sumsq, int shares,
+                      int h_rows, hipStream_t stream) {
+    LC_CHECK(shares >= 0 && (shares == 0 || (delta && h_rows > 0)), "rmsnorm: bad shares %d", shares);
+    const size_t share_stride = (size_t)h_rows * n;
     LC_CHECK(R >= 0 && n > 0, "rmsnorm: bad sizes R=%d n=%d", R, n);
     if (R == 0) return 0;
     LC_CHECK(h && w && out, "rmsnorm: null pointer");
@@ -329,17 +360,17 @@ LC_API int lc_rmsnorm(float* h, const void* delta, const int* rows, const float*
     if (dt == DT_F32) {
         if (vec)
             rmsnorm_vec_kernel<float><<<R, RN_THREADS, 0, stream>>>(h, (const float*)delta, rows, w, eps,
-                                                                    (float*)out, n, write_h, sumsq);
+                                                                    (float*)out, n, write_h, sumsq, shares, share_stride);
         else
             rmsnorm_kernel<float><<<R, threads, 0, stream>>>(h, (const float*)delta, rows, w, eps,
-                                                             (float*)out, n, write_h, sumsq);
+                                                             (float*)out, n, write_h, sumsq, shares, share_stride);
     } else if (dt == DT_BF16) {
         if (vec)
             rmsnorm_vec_kernel<bf16><<<R, RN_THREADS, 0, stream>>>(h, (const bf16*)delta, rows, w, eps,
-                                                                   (bf16*)out, n, write_h, sumsq);
+                                                                   (bf16*)out, n, write_h, sumsq, shares, share_stride);
         else
             rmsnorm_kernel<bf16><<<R, threads, 0, stream>>>(h, (const bf16*)delta, rows, w, eps,
-                                                            (bf16*)out, n, write_h, sumsq);
+                                                            (bf16*)out, n, write_h, sumsq, shares, share_stride);
     } else {
         LC_CHECK(false, "rmsnorm: unknown dtype %d", dt);
     }

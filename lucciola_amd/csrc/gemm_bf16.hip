@@ -968,3 +968,40 @@ LC_API int lc_gemm_bf16_scaled_rows(const void* x, const void* w, void* out, int
     LC_LAUNCH_CHECK("gemm_skinny");
     return 0;
 }
+
+// ------------------------------------------------------------------ products left as shares
+// Where the product of more than 16 rows is cut along K (few tiles, see splitk_shares), the
+// shares' float32 sums can be handed on as they are: the norm kernel that adds the product to
+// the residual stream sums them itself, in the order of the shares, and the reduction kernel
+// and the rounding of the product to bfloat16 fall away.
+
+// Number of shares that lc_gemm_bf16_partials writes for these sizes (0: this product is not cut).
+LC_API int lc_gemm_bf16_shares(int M, int N, int K) {
+    if (!lc_gemm_bf16_supported(M, N, K) || M <= 16) return 0;
+    const int shares = splitk_shares(M, N, K);
+    return shares > 1 ? shares : 0;
+}
+
+// partials [lc_gemm_bf16_shares(M, N, K)][M][N] float32: x . w^T is their sum.
+LC_API int lc_gemm_bf16_partials(const void* x, const void* w, float* partials, int M, int N, int K,
+                                 hipStream_t stream) {
+    const int shares = lc_gemm_bf16_shares(M, N, K);
+    LC_CHECK(shares > 1, "gemm_bf16_partials: the product M=%d N=%d K=%d is not cut along K", M, N, K);
+    LC_CHECK(x && w && partials, "gemm_bf16_partials: null pointer");
+    LC_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0) && (uintptr_t)partials % 8 == 0,
+             "gemm_bf16_partials: operands must be 16-byte aligned");
+    const bf16* xb = (const bf16*)x;
+    const bf16* wb = (const bf16*)w;
+    if (pick_tile(M, N, K) == TILE_64x128) {
+        const int tiles_m = (M + 63) / 64, tiles = tiles_m * ((N + 127) / 128);
+        gemm_tiled_kernel<64, 128, 4, 0, true, float><<<dim3(tiles, shares), 256, 0, stream>>>(
+            xb, wb, nullptr, partials, M, N, K, tiles_m, 0, tiles, 0);
+    } else {
+        const int tiles_m = (M + 127) / 128, tiles = tiles_m * ((N + 127) / 128);
+        gemm_tiled_kernel<128, 128, 2, 0, true, float><<<dim3(tiles, shares), 256, 0, stream>>>(
+            xb, wb, nullptr, partials, M, N, K, tiles_m, 0, tiles, 0);
+    }
+    LC_LAUNCH_CHECK("gemm_tiled");
+    return 0;
+}
+

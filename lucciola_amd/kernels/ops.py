@@ -23,7 +23,7 @@ DT_F32, DT_BF16 = 0, 1
 _ARG = {"p": ctypes.c_void_p, "i": ctypes.c_int, "f": ctypes.c_float}
 _SIGNATURES = {
     "lc_embedding": "ppipiiip",
-    "lc_rmsnorm": "ppppfpiiiipp",
+    "lc_rmsnorm": "ppppfpiiiipiip",
     "lc_rmsnorm_act": "ppfpiiip",
     "lc_gemm_generic": "pipipiiiip",
     "lc_gemm_bf16": "pppiiiiipp",
@@ -32,6 +32,8 @@ _SIGNATURES = {
     "lc_gemm_bf16_force_skinny": "i",
     "lc_gemm_bf16_residual_pieces": "iii",
     "lc_gemm_bf16_piece_stride": "i",
+    "lc_gemm_bf16_shares": "iii",
+    "lc_gemm_bf16_partials": "pppiiip",
     "lc_gemm_bf16_residual": "ppppppiiip",
     "lc_gemm_bf16_scaled_rows": "pppiiiipifp",
     "lc_qk_norm_rope_write": "piiiiippfppipppip",
@@ -198,8 +200,19 @@ def rmsnorm(h: torch.Tensor, delta, weight: torch.Tensor, eps: float,
             _call("lc_gemm_bf16_residual", _ptr(delta.x), _ptr(delta.w), _ptr(h), _ptr(weight),
                   _ptr(xg), _ptr(parts), _c_int(M), _c_int(n), _c_int(K), _stream())
             return ScaledRows(xg, parts, pieces, float(eps), h, weight)
-        delta = delta.value()
-    if delta is not None:
+        shares = library().lc_gemm_bf16_shares(M, n, K) if (delta.w.shape[0] == n and M == T) else 0
+        if shares:
+            # the product is cut along K anyway: its shares are summed in the norm kernel
+            partials = torch.empty((shares, T, n), dtype=torch.float32, device=h.device)
+            _call("lc_gemm_bf16_partials", _ptr(delta.x), _ptr(delta.w), _ptr(partials), _c_int(M),
+                  _c_int(n), _c_int(K), _stream())
+            delta = partials
+        else:
+            shares = 0
+            delta = delta.value()
+    else:
+        shares = 0
+    if delta is not None and not shares:
         _need(delta, "rmsnorm delta", out_dtype, 2)
         if tuple(delta.shape) != (T, n):
             raise KernelError(f"rmsnorm: delta {tuple(delta.shape)} does not match h {(T, n)}")
@@ -211,7 +224,8 @@ def rmsnorm(h: torch.Tensor, delta, weight: torch.Tensor, eps: float,
              if scaled else None)
     _call("lc_rmsnorm", _ptr(h), _ptr(delta), _ptr(rows), _ptr(weight), _c_float(eps), _ptr(out),
           _c_int(_dt(out)), _c_int(R), _c_int(n),
-          _c_int(1 if (rows is None and delta is not None) else 0), _ptr(parts), _stream())
+          _c_int(1 if (rows is None and delta is not None) else 0), _ptr(parts), _c_int(shares),
+          _c_int(T), _stream())
     return ScaledRows(out, parts, 1, float(eps), h, weight) if scaled else out
 
 
@@ -262,8 +276,8 @@ def gemm(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None, defer: boo
     if K != K2:
         raise KernelError(f"gemm: x is [{M}, {K}] but w is [{N}, {K2}]")
     out_dtype = out_dtype or x.dtype
-    if (defer and out_dtype == torch.bfloat16 and x.dtype == torch.bfloat16
-            and w.dtype == torch.bfloat16 and library().lc_gemm_bf16_residual_pieces(M, N, K)):
+    if (defer and out_dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+            and (library().lc_gemm_bf16_residual_pieces(M, N, K) or library().lc_gemm_bf16_shares(M, N, K))):
         return PendingProduct(x, w, out_dtype)
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     if M == 0:

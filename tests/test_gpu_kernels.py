@@ -347,8 +347,10 @@ def test_norm_folded_into_the_products_around_it(M, H, K, N2):
     plain_rows = ops.rmsnorm(h3, ops.gemm(x, w, torch.bfloat16, defer=True), g, eps, torch.bfloat16)
     assert isinstance(plain_rows, torch.Tensor)
     torch.testing.assert_close(h3.double(), h_want, rtol=2e-2, atol=2e-2)   # the branch was rounded to bfloat16 first
-    # more than 16 rows, float32, or a width the matrix-core kernels do not take: nothing is deferred
-    assert isinstance(ops.gemm(rnd(17, K, dtype=torch.bfloat16), w, torch.bfloat16, defer=True), torch.Tensor)
+    # more than 16 rows (unless the product is cut along K anyway), float32, or a width the
+    # matrix-core kernels do not take: nothing is deferred
+    more = ops.gemm(rnd(17, K, dtype=torch.bfloat16), w, torch.bfloat16, defer=True)
+    assert isinstance(more, ops.PendingProduct) == (ops.library().lc_gemm_bf16_shares(17, H, K) > 1)
     assert isinstance(ops.gemm(x.float(), w.float(), torch.float32, defer=True), torch.Tensor)
     assert isinstance(ops.rmsnorm(rnd(M, 72), None, 1 + rnd(72), eps, torch.bfloat16, scaled=True), torch.Tensor)
 
@@ -499,3 +501,31 @@ def few_rows_case(M, N, K):
     factors = torch.rsqrt((h.double() ** 2).mean(1, keepdim=True) + 1e-6)
     close(ops.gemm(rows, w, torch.bfloat16), ((rows.x.double() @ w.double().T) * factors).to(torch.bfloat16),
           torch.bfloat16, scale=2.0)
+
+
+@pytest.mark.parametrize("M,H,K", [(40, 512, 2048), (64, 4096, 4096), (100, 384, 1024), (17, 1152, 1536)])
+def test_norm_sums_the_shares_of_a_product_cut_along_k(M, H, K):
+    """More than 16 rows and few tiles: the product before a norm is cut along K; its shares
+    stay float32 and the norm kernel adds them to the stream itself (all rows, and chosen rows
+    with the stream left alone)."""
+    eps = 1e-6
+    h = rnd(M, H, seed=90, scale=2.0)
+    x = rnd(M, K, dtype=torch.bfloat16, seed=91)
+    w = rnd(H, K, dtype=torch.bfloat16, seed=92, scale=K ** -0.5)
+    g = 1 + rnd(H, seed=93, scale=0.2)
+    assert ops.library().lc_gemm_bf16_shares(M, H, K) > 1
+    pending = ops.gemm(x, w, torch.bfloat16, defer=True)
+    assert isinstance(pending, ops.PendingProduct)
+    h_want = h.double() + x.double() @ w.double().T
+    normed = h_want * torch.rsqrt((h_want ** 2).mean(1, keepdim=True) + eps) * g.double()
+    rows = torch.tensor([M - 1, 0, 3], dtype=torch.int32, device=DEV)
+    h_rows = h.clone()
+    got_rows = ops.rmsnorm(h_rows, pending, g, eps, torch.bfloat16, rows=rows)
+    assert torch.equal(h_rows, h)
+    close(got_rows, normed[rows.long()].to(torch.bfloat16), torch.bfloat16)
+    h_got = h.clone()
+    got = ops.rmsnorm(h_got, pending, g, eps, torch.bfloat16, scaled=True)
+    assert isinstance(got, torch.Tensor)
+    torch.testing.assert_close(h_got.double(), h_want, rtol=1e-5, atol=1e-5)
+    close(got, normed.to(torch.bfloat16), torch.bfloat16)
+    close(ops.value(pending), (x.double() @ w.double().T).to(torch.bfloat16), torch.bfloat16, scale=2.0)
