@@ -630,10 +630,10 @@ LC_API int lc_attn_decode_splits(int num_decode, int nkv, int max_ctx) {
     if (num_decode <= 0) return 1;
     const int pages = (max_ctx + PAGE - 1) / PAGE;
     const long long base = (long long)num_decode * nkv;
-    long long splits = (1024 + base - 1) / base;          // aim at ~4 workgroups per CU
+    long long splits = (512 + base - 1) / base;           // two workgroups a CU: measured to beat four
     const int most = (pages + 7) / 8;                     // at least 8 pages per workgroup
     if (splits > most) splits = most;
-    if (splits > 64) splits = 64;
+    if (splits > 32) splits = 32;
     if (splits < 1) splits = 1;
     return (int)splits;
 }
