@@ -358,7 +358,7 @@ __global__ __launch_bounds__(128) void attn_decode_join_kernel(const float* __re
 
 // ------------------------------------------------------------------------------- prefill
 // tiles: [NT, 4] = (request, first token row, rows (<= 64), position of the first row), the
-// tiles that see the fewest keys first.
+// tiles that see the most keys first.
 // A workgroup takes one tile and HPW heads of one kv head and walks the pages the tile can
 // see, PF_NP pages (64 keys) at a time.  Its 256 threads bring a group of pages into LDS
 // together (the next group's loads are in flight in registers meanwhile), and every wave
@@ -387,12 +387,12 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     __shared__ __attribute__((aligned(16))) bf16 vs[2][NP * VPAGE];
 
     // Which tile and which heads.  Workgroups start in the order of their number (x fastest)
-    // and two fit on a CU; the tiles come shortest first, and a tile's heads are neighbours, so
-    // that the workgroups that read the same keys and values run at the same time.  Measured:
-    // with more workgroups than fit at once, shortest first is the fastest order (the long ones
-    // at the end all take about as long as each other); when all fit at once, nobody takes over
-    // from a CU that is done early, and the second workgroup of a CU should be as long as its
-    // first is short: the second half of the numbers takes the tasks from the longest down.
+    // and two fit on a CU; the tiles come longest first, and a tile's heads are neighbours, so
+    // that the workgroups that read the same keys and values run at the same time.  With more
+    // workgroups than fit at once, whoever is done takes the longest tile that is left.  When
+    // all fit at once, nobody takes over from a CU that is done early, and the second workgroup
+    // of a CU should be as short as its first is long: the second half of the numbers takes the
+    // tasks from the shortest up.
     const int total = gridDim.x * gridDim.y, number = blockIdx.y * gridDim.x + blockIdx.x;
     const int half = (total + 1) / 2;
     const int task = (total <= 2 * 256 && number >= half) ? total - 1 - (number - half) : number;

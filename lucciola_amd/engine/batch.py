@@ -161,9 +161,9 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
                 continue
             for t0 in range(0, n, PREFILL_TILE):
                 tile_list.append((r, q_start[r] + t0, min(PREFILL_TILE, n - t0), first_pos[r] + t0))
-        # the tiles that see the fewest keys first: the order in which the kernel's workgroups
-        # start (measured to be the fastest; it changes no tile's result)
-        tile_list.sort(key=lambda t: t[3] + t[2])
+        # the tiles that see the most keys first: the kernel's workgroups start in this order,
+        # and whoever is done takes the longest that is left (the order changes no tile's result)
+        tile_list.sort(key=lambda t: -(t[3] + t[2]))
         tiles = [v for t in tile_list for v in t]
 
     pk = _Packer()
