@@ -363,7 +363,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
     constexpr int LPA = BM * 8 / 256, LPB = BN * 8 / 256, LP = LPA + LPB;   // load instructions per thread and stage
     constexpr int NM = TM * TN, NR = TM + TN;                 // products and operand reads per k-step
     constexpr int A_STAGE = BM * TL_K * 2, B_STAGE = BN * TL_K * 2;          // bytes
-    static_assert(S >= 2 && (S - 1) * LP <= 63, "the load counter holds 63");
+    static_assert(S >= 2 && (S == 2 ? 2 : S - 1) * LP <= 63, "the load counter holds 63");
     static_assert(S * (A_STAGE + B_STAGE) <= 160 * 1024, "LDS");
     __shared__ __attribute__((aligned(1024))) char lds[S * (A_STAGE + B_STAGE)];   // A stages, then B stages
 
@@ -413,8 +413,15 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
             __builtin_amdgcn_global_load_lds((glb_ptr_t)(wg[idx - LPA] + kb * TL_K),
                 (lds_ptr_t)(lds + S * A_STAGE + stage * B_STAGE + ((idx - LPA) * 4 + wave) * 1024), 16, 0, 0);
     };
+    // With two stages, a block's loads are issued a block early: in the last k-step of block it,
+    // once every wave has read the last of the stage, block it + 2 goes into it, behind block
+    // it + 1 that is still arriving.  (Issued only after block it + 1 has landed, the loads
+    // would start with nothing in flight: their first data would be a whole latency away, and
+    // the way from L2 into the CU, which bounds these kernels, would stand idle meanwhile.)
+    constexpr bool EARLY = S == 2;
+    constexpr int AHEAD = EARLY ? 2 : S - 1;                  // blocks in flight at the start
 #pragma unroll
-    for (int s = 0; s < S - 1; ++s)
+    for (int s = 0; s < AHEAD; ++s)
         if (s < nk) {
 #pragma unroll
             for (int i = 0; i < LP; ++i) issue_one(i, s, s);
@@ -472,8 +479,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
     constexpr int BAR = NM / 4;                                // the product after which a block's last k-step syncs
     constexpr int QT = NM - BAR - 1 > 0 ? (NR + (NM - BAR - 1) - 1) / (NM - BAR - 1) : NR;
 
-    // block 0 has landed when at most the S-2 younger blocks are still in flight
-    if (nk >= S - 1) wait_vmcnt<(S - 2) * LP>(); else wait_vmcnt<0>();
+    // block 0 has landed when at most the younger blocks are still in flight
+    if (nk >= AHEAD) wait_vmcnt<(AHEAD - 1) * LP>(); else wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int r = 0; r < NR; ++r) read_one(r, 0, 0, 0);
@@ -496,7 +503,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 #pragma unroll
                     for (int r = k * QR; r < (k + 1) * QR; ++r)
                         if (r < NR) read_one(r, stage, ks + 1, nxt);
-                    if (LOAD && ks == 0 && (k >= RS || NM == RS)) {
+                    if (LOAD && !EARLY && ks == 0 && (k >= RS || NM == RS)) {
                         const int first = NM == RS ? k * QL : (k - RS) * QL;
 #pragma unroll
                         for (int l = first; l < first + QL; ++l)
@@ -510,7 +517,16 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
                     product(k, cur);
                     __builtin_amdgcn_sched_barrier(0);
                     if (LOAD) {
-                        if (k == BAR) { wait_vmcnt<(S - 2) * LP>(); __builtin_amdgcn_s_barrier(); }
+                        if (k == BAR && EARLY) {
+                            __builtin_amdgcn_s_barrier();          // nobody reads this stage any more
+#pragma unroll
+                            for (int l = 0; l < LP; ++l) issue_one(l, it + 2, stage);
+                            wait_vmcnt<LP>();                      // block it + 1 has landed
+                            __builtin_amdgcn_s_barrier();
+                        } else if (k == BAR) {
+                            wait_vmcnt<(S - 2) * LP>();
+                            __builtin_amdgcn_s_barrier();
+                        }
                         if (NM - BAR - 1 > 0) {
 #pragma unroll
                             for (int r = (k - BAR - 1) * QT; r < (k - BAR) * QT; ++r)
@@ -535,7 +551,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
         lstage = lstage + 1 == S ? 0 : lstage + 1;
     };
     int it = 0;
-    for (; it + S - 1 < nk; ++it) block(it, std::true_type{});
+    for (; it + AHEAD < nk; ++it) block(it, std::true_type{});
     for (; it < nk; ++it) block(it, std::false_type{});
 
     // acc[i][j][v]: row m = (v/4)*8 + (lane/32)*4 + v%4, column n = lane%32 of the 32x32 tile.
