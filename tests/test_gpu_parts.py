@@ -466,3 +466,56 @@ def test_block_arrangement_alone():
     pending = -0.5 * plain.rmsnorm(h1, w2.cpu(), 1e-6)
     torch.testing.assert_close(stream.h.double().cpu(), h1, rtol=1e-5, atol=1e-5)
     torch.testing.assert_close(stream.pending.double().cpu(), pending, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("rows", [6, 16, 40])
+def test_block_mixes_parts_that_take_scaled_rows_with_parts_that_do_not(rows):
+    """Widths that the fused decode kernels take (bfloat16, 128 wide): a stand-in mixer that
+    knows nothing of scaled rows or pending products beside the real feed-forward that uses
+    both, and two blocks in a row so that a pending product meets the next block's norm.  Few
+    rows (fused norms), 16 (their limit) and 40 (more: products cut along K hand their shares to
+    the norm) must all give what the plain formulas give."""
+    from lucciola_amd.config.registry import BLOCKS
+
+    class Scale:                                  # takes and returns tensors only
+        def __init__(self, factor):
+            self.factor = factor
+
+        def forward(self, x, site=None):
+            assert isinstance(x, torch.Tensor)
+            return (x.float() * self.factor).to(x.dtype)
+
+    H, I, eps = 128, 2048, 1e-6
+    ctx = BuildContext(torch.bfloat16, DEV)
+    norm_w = [1 + rnd(H, seed=40 + i, scale=0.1) for i in range(4)]
+    norms = []
+    for w in norm_w:
+        n = build_part(NORMS, PartSpec("rms", {"size": H, "eps": eps}))
+        n.bind({"weight": w}, ctx)
+        norms.append(n)
+    ffs, ff_w = [], []
+    for i in range(2):
+        ff = build_part(FEED_FORWARDS, PartSpec("gated_mlp", {"hidden_size": H, "intermediate_size": I}))
+        w = {"gate_proj": rnd(I, H, seed=50 + i, scale=H ** -0.5, dtype=torch.bfloat16),
+             "up_proj": rnd(I, H, seed=52 + i, scale=H ** -0.5, dtype=torch.bfloat16),
+             "down_proj": rnd(H, I, seed=54 + i, scale=I ** -0.5, dtype=torch.bfloat16)}
+        ff.bind(dict(w), ctx)
+        ffs.append(ff)
+        ff_w.append({"m." + k + ".weight": v.cpu() for k, v in w.items()})
+    make = BLOCKS.get("prenorm_residual")
+    blocks = [make(Scale(0.5), ffs[0], norms[0], norms[1]), make(Scale(-0.25), ffs[1], norms[2], norms[3])]
+    h = rnd(rows, H, seed=60)
+    stream = ResidualStream(h.clone())
+    for block in blocks:
+        block.forward(stream, None)
+    # plain formulas, float64
+    want = h.double().cpu()
+    pending = torch.zeros_like(want)
+    for i, factor in enumerate((0.5, -0.25)):
+        want = want + pending
+        want = want + factor * plain.rmsnorm(want, norm_w[2 * i].cpu(), eps)
+        pending = plain.mlp_block(plain.rmsnorm(want, norm_w[2 * i + 1].cpu(), eps), ff_w[i], "m.")
+    if rows <= 16:
+        assert isinstance(stream.pending, ops.PendingProduct)
+    assert rel(stream.h, want) < 2e-2
+    assert rel(ops.value(stream.pending), pending) < 3e-2
