@@ -708,20 +708,28 @@ static TailPlan tail_plan(int t, int M, int N, int K) {
 }
 
 // The tile for a product with M > 16.  Up to 64 rows: the 64-row tile.  Beyond: the shape with
-// the least estimated time, (rounds of tiles a CU works through) x (tile area) / (measured
-// relative rate of the shape: larger tiles move fewer bytes per product).
+// the least estimated time in microseconds.  A CU works through a round of tiles in
+// (tile area) x K x 2 / (4.63 MFLOP/us x the shape's relative rate) (measured at K = 4096: larger
+// tiles move fewer bytes per product); a last round that is cut along K takes its share of
+// that, plus the time to write and read its float32 partial tiles (about 4 TB/s) and to start
+// two more kernels.
 static int pick_tile(int M, int N, int K) {
     if (g_force_tile != TILE_AUTO) return g_force_tile;
     if (M <= 64) return TILE_64x128;
-    const double rate[TILE_COUNT] = {0.0, 0.87, 1.0, 1.1, 1.2};
+    const double rate[TILE_COUNT] = {0.0, 0.82, 0.90, 0.94, 1.0};
     int best = TILE_128x128;
     double best_cost = 0.0;
     for (int t = TILE_128x128; t < TILE_COUNT; ++t) {
         const long long tiles = tile_count(t, M, N);
-        double rounds = (double)((tiles + kCUs - 1) / kCUs);
+        const double area = (double)tile_bm(t) * tile_bn(t);
+        const double round_us = area * K * 2.0 / (4.63e6 * rate[t]) + 3.0;
         const TailPlan tail = tail_plan(t, M, N, K);
-        if (tail.shares > 1) rounds = (double)(tiles / kCUs) + 1.0 / tail.shares + 0.1;
-        const double cost = rounds * tile_bm(t) * tile_bn(t) / rate[t];
+        double cost;
+        if (tail.shares > 1)
+            cost = (double)(tiles / kCUs) * round_us + round_us / tail.shares +
+                   (double)tail.rest * tail.shares * area * 8.0 / 4.0e6 + 10.0;
+        else
+            cost = (double)((tiles + kCUs - 1) / kCUs) * round_us;
         if (t == TILE_128x128 || cost < best_cost) { best = t; best_cost = cost; }
     }
     return best;
