@@ -970,12 +970,17 @@ LC_API int lc_gemm_bf16_residual(const void* x, const void* w, float* resid, con
     return 0;
 }
 
+// Whether lc_gemm_bf16_scaled_rows takes these sizes.
+LC_API int lc_gemm_bf16_scaled_rows_supported(int M, int N, int K) {
+    return lc_gemm_bf16_supported(M, N, K) && M <= 16 && g_force_tile == TILE_AUTO;
+}
+
 // out = (x . w^T) with row m scaled by rsqrt(sum_p pieces[p][m] / K + eps) before the epilogue
 // (0: plain, bfloat16 [M, N]; 1: SwiGLU as in lc_gemm_bf16, bfloat16 [M, N / 2]).
 LC_API int lc_gemm_bf16_scaled_rows(const void* x, const void* w, void* out, int M, int N, int K,
                                     int epilogue, const float* pieces, int count, float eps,
                                     hipStream_t stream) {
-    LC_CHECK(lc_gemm_bf16_supported(M, N, K) && M <= 16 && g_force_tile == TILE_AUTO,
+    LC_CHECK(lc_gemm_bf16_scaled_rows_supported(M, N, K),
              "gemm_bf16_scaled_rows: sizes M=%d N=%d K=%d are not supported", M, N, K);
     LC_CHECK(count >= 1 && count <= SK_MAX_PIECES, "gemm_bf16_scaled_rows: %d pieces (at most %d)", count, SK_MAX_PIECES);
     LC_CHECK(x && w && out && pieces, "gemm_bf16_scaled_rows: null pointer");

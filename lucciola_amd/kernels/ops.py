@@ -36,6 +36,7 @@ _SIGNATURES = {
     "lc_gemm_bf16_partials": "pppiiip",
     "lc_gemm_bf16_residual": "ppppppiiip",
     "lc_gemm_bf16_scaled_rows": "pppiiiipifp",
+    "lc_gemm_bf16_scaled_rows_supported": "iii",
     "lc_qk_norm_rope_write": "piiiiippfppipppip",
     "lc_attention_generic": "pipppipppiiiiiifip",
     "lc_attn_bf16_supported": "iiii",
@@ -187,8 +188,8 @@ def rmsnorm(h: torch.Tensor, delta, weight: torch.Tensor, eps: float,
     T, n = h.shape
     if weight.shape[0] != n:
         raise KernelError(f"rmsnorm: weight has {weight.shape[0]} entries for rows of {n}")
-    scaled = (scaled and rows is None and out_dtype == torch.bfloat16 and 0 < T <= 16
-              and _fast_gemm_ok(T, 16, n))
+    scaled = (scaled and rows is None and out_dtype == torch.bfloat16 and T > 0
+              and bool(library().lc_gemm_bf16_scaled_rows_supported(T, 16, n)))
     if isinstance(delta, PendingProduct):
         M, K = delta.x.shape
         pieces = (library().lc_gemm_bf16_residual_pieces(M, n, K)
@@ -249,7 +250,7 @@ def _scaled_product(x: "ScaledRows", w: torch.Tensor, epilogue: int) -> Optional
     M, K = x.x.shape
     N = w.shape[0]
     if not (w.dtype == torch.bfloat16 and x.x.dtype == torch.bfloat16 and w.shape[1] == K
-            and library().lc_gemm_bf16_residual_pieces(M, 16, K)):
+            and x.count <= 512 and library().lc_gemm_bf16_scaled_rows_supported(M, N, K)):
         return None
     out = torch.empty((M, N // 2 if epilogue else N), dtype=torch.bfloat16, device=w.device)
     _call("lc_gemm_bf16_scaled_rows", _ptr(x.x), _ptr(w), _ptr(out), _c_int(M), _c_int(N),
