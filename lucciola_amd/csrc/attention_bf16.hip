@@ -169,8 +169,8 @@ __device__ __forceinline__ void attend_range(AttnState<D, QT>& st, const bf16x8 
 }
 
 // ------------------------------------------------------------------------------- decode
-// What the decode kernel does to the raw q, k, v of its token before it attends, when the
-// step has no separate kernel for it: RMSNorm over the head (weights optional), rotary
+// What an attention kernel does to the raw q (the decode kernel also: k, v) of its tokens before
+// it attends, when the step has no separate kernel for it: RMSNorm over the head (weights optional), rotary
 // embedding of the first `rot` entries (table optional: row p holds rot/2 cosines, then rot/2
 // sines), and, if write_kv, the token's k and v into their place in the cache.  The formulas
 // and their order are those of the separate kernel (elementwise.hip, qk_norm_rope_write).
@@ -377,7 +377,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     const bf16* __restrict__ qkv, int q_stride, const bf16* __restrict__ k_cache,
     const bf16* __restrict__ v_cache, bf16* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ block_table, int max_blocks, int nh, int nkv, float scale_log2,
-    int window) {
+    int window, DecodePrologue pro) {
     constexpr int QT = HPW, NP = PF_NP;
     constexpr int KLD = D + 8;
     constexpr int KPAGE = PAGE * KLD, VPAGE = D * PAGE;   // elements of a page in LDS
@@ -422,6 +422,50 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
                            (size_t)min(h, nh - 1) * D + kg * 8;
 #pragma unroll
         for (int i = 0; i < D / 32; ++i) bq[c][i] = *reinterpret_cast<const bf16x8*>(qrow + i * 32);
+        if constexpr (D == 128) {
+            // q arrives raw: RMSNorm over the head and the rotary embedding right here, on the
+            // operand registers (the lane holds entries 32 i + 8 kg + e of its row, i < 4, so an
+            // entry and its partner 64 further on sit in the same lane).  The formulas and the
+            // order of their roundings are those of head128_norm_rope; only the sum of squares
+            // is added up in another order.
+            if (pro.enabled) {
+                float f[4][8];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) f[i][e] = static_cast<float>(bq[c][i][e]);
+                if (pro.q_w) {
+                    float ss = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) ss = __fmaf_rn(f[i][e], f[i][e], ss);
+                    ss = column_sum(ss);
+                    const float inv = rsqrtf(ss / 128.f + pro.eps);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            f[i][e] = __fmul_rn(__fmul_rn(f[i][e], inv), pro.q_w[i * 32 + kg * 8 + e]);
+                }
+                if (pro.rope) {
+                    const float* cs = pro.rope + (size_t)p * 128;     // 64 cosines, then 64 sines
+#pragma unroll
+                    for (int i = 0; i < 2; ++i)
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            const float cosv = cs[i * 32 + kg * 8 + e], sinv = cs[64 + i * 32 + kg * 8 + e];
+                            const float a = f[i][e], b = f[i + 2][e];
+                            f[i][e] = __fsub_rn(__fmul_rn(a, cosv), __fmul_rn(b, sinv));
+                            f[i + 2][e] = __fadd_rn(__fmul_rn(a, sinv), __fmul_rn(b, cosv));
+                        }
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) bq[c][i][e] = static_cast<bf16>(f[i][e]);
+            }
+        }
     }
     // pages the workgroup walks, and the part of them this wave needs
     const int t_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
@@ -603,13 +647,13 @@ static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* 
 template <int D>
 static int launch_prefill(const bf16* qkv, int q_stride, const bf16* k, const bf16* v, bf16* out,
                           const int* tiles, const int* table, int max_blocks, int NT, int nh,
-                          int nkv, float scale_log2, int window, hipStream_t s) {
+                          int nkv, float scale_log2, int window, DecodePrologue pro, hipStream_t s) {
     if ((nh / nkv) % 2 == 0)
         attn_prefill_kernel<D, 2><<<dim3(NT, nh / 2), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
-                                                                   max_blocks, nh, nkv, scale_log2, window);
+                                                                   max_blocks, nh, nkv, scale_log2, window, pro);
     else
         attn_prefill_kernel<D, 1><<<dim3(NT, nh), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
-                                                               max_blocks, nh, nkv, scale_log2, window);
+                                                               max_blocks, nh, nkv, scale_log2, window, pro);
     LC_LAUNCH_CHECK("attn_prefill");
     return 0;
 }
@@ -677,18 +721,30 @@ LC_API int lc_attn_decode_bf16(const void* qkv, int q_stride, void* k_cache, voi
     return 0;
 }
 
+// Whether the prefill kernel can norm and rotate q itself for this head size and rotary width
+// (whole heads of 128 that rotate whole or not at all).
+LC_API int lc_attn_prefill_prepares_q(int d, int rot) { return d == 128 && (rot == 0 || rot == 128); }
+
+// prologue != 0 (lc_attn_prefill_prepares_q(d, rot) must hold): q in qkv is raw; the kernel norms
+// (q_w may be null) and rotates it itself (rope_table may be null).  The step's keys and values
+// are in the cache either way.
 LC_API int lc_attn_prefill_bf16(const void* qkv, int q_stride, const void* k_cache, const void* v_cache,
                                 void* out, const int* tiles, const int* block_table, int max_blocks,
                                 int num_tiles, int nh, int nkv, int d, int page_size, float scale,
-                                int window, hipStream_t stream) {
+                                int window, int prologue, const float* q_w, float eps,
+                                const float* rope_table, int rot, hipStream_t stream) {
     if (num_tiles == 0) return 0;
     LC_CHECK(lc_attn_bf16_supported(nh, nkv, d, page_size),
              "attn_prefill_bf16: unsupported sizes nh=%d nkv=%d d=%d page=%d", nh, nkv, d, page_size);
     LC_CHECK(qkv && k_cache && v_cache && out && tiles && block_table, "attn_prefill_bf16: null pointer");
     LC_CHECK(q_stride % 8 == 0 && (uintptr_t)qkv % 16 == 0, "attn_prefill_bf16: q must be 16-byte aligned");
+    if (!rope_table) rot = 0;
+    LC_CHECK(!prologue || lc_attn_prefill_prepares_q(d, rot),
+             "attn_prefill_bf16: the kernel cannot prepare q for head size %d with %d rotary entries", d, rot);
     const float sl2 = scale * 1.4426950408889634f;
+    DecodePrologue pro = {q_w, nullptr, rope_table, eps, rot, 0, prologue};
 #define CALL(DD) launch_prefill<DD>((const bf16*)qkv, q_stride, (const bf16*)k_cache, (const bf16*)v_cache, \
-        (bf16*)out, tiles, block_table, max_blocks, num_tiles, nh, nkv, sl2, window, stream)
+        (bf16*)out, tiles, block_table, max_blocks, num_tiles, nh, nkv, sl2, window, pro, stream)
     LC_DISPATCH_D(d, CALL)
 #undef CALL
     return 0;

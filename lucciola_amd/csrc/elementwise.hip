@@ -204,13 +204,13 @@ __global__ void qk_norm_rope_write_kernel(T* __restrict__ qkv, int T_tokens, int
                                           const int* __restrict__ positions,
                                           const float* __restrict__ rope_table, int rot,
                                           T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                          const int* __restrict__ slots, int page_size) {
+                                          const int* __restrict__ slots, int page_size, int first_head) {
     const int t = blockIdx.x;
     const int wave = threadIdx.x / kWave;
     const int lane = threadIdx.x & (kWave - 1);
     const int waves = blockDim.x / kWave;
     const int heads = nh + 2 * nkv;
-    const int head = blockIdx.y * waves + wave;
+    const int head = first_head + blockIdx.y * waves + wave;     // heads before first_head are left alone
     if (head >= heads) return;
     T* x = qkv + ((size_t)t * heads + head) * d;
 
@@ -277,12 +277,12 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write128_kernel(
     bf16* __restrict__ qkv, int T_tokens, int nh, int nkv, const float* __restrict__ q_w,
     const float* __restrict__ k_w, float eps, const int* __restrict__ positions,
     const float* __restrict__ rope_table, bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
-    const int* __restrict__ slots, int page_size) {
+    const int* __restrict__ slots, int page_size, int first_head) {
     constexpr int d = 128;
-    const int heads = nh + 2 * nkv;
+    const int heads = nh + 2 * nkv, span = heads - first_head;   // heads before first_head are left alone
     const long long g = (long long)blockIdx.x * 16 + (threadIdx.x >> 4);
-    if (g >= (long long)T_tokens * heads) return;          // whole groups of 16 lanes leave together
-    const int t = (int)(g / heads), head = (int)(g - (long long)t * heads), j = threadIdx.x & 15;
+    if (g >= (long long)T_tokens * span) return;           // whole groups of 16 lanes leave together
+    const int t = (int)(g / span), head = first_head + (int)(g - (long long)t * span), j = threadIdx.x & 15;
     bf16* x = qkv + ((size_t)t * heads + head) * d + 8 * j;
     const bool is_q = head < nh, is_k = !is_q && head < nh + nkv;
     const int kvh = is_q ? 0 : (is_k ? head - nh : head - nh - nkv);
@@ -398,9 +398,11 @@ LC_API int lc_qk_norm_rope_write(void* qkv, int dt, int T, int nh, int nkv, int 
                                  const float* q_w, const float* k_w, float eps,
                                  const int* positions, const float* rope_table, int rot,
                                  void* k_cache, void* v_cache, const int* slots, int page_size,
-                                 hipStream_t stream) {
+                                 int first_head, hipStream_t stream) {
     LC_CHECK(T >= 0 && nh > 0 && nkv > 0 && d > 0, "qk_norm_rope_write: bad sizes T=%d nh=%d nkv=%d d=%d",
              T, nh, nkv, d);
+    LC_CHECK(first_head == 0 || first_head == nh, "qk_norm_rope_write: first head %d (0: all heads, %d: k and v only)",
+             first_head, nh);
     if (T == 0) return 0;
     LC_CHECK(qkv, "qk_norm_rope_write: null qkv");
     LC_CHECK(rot >= 0 && rot <= d && rot % 2 == 0,
@@ -411,23 +413,23 @@ LC_API int lc_qk_norm_rope_write(void* qkv, int dt, int T, int nh, int nkv, int 
     if (!rope_table) rot = 0;
     if (dt == DT_BF16 && d == 128 && (rot == 0 || rot == 128) && (q_w == nullptr) == (k_w == nullptr) &&
         (uintptr_t)qkv % 16 == 0 && (uintptr_t)k_cache % 16 == 0) {
-        const long long groups = (long long)T * (nh + 2 * nkv);
+        const long long groups = (long long)T * (nh + 2 * nkv - first_head);
         qk_norm_rope_write128_kernel<<<(unsigned)((groups + 15) / 16), 256, 0, stream>>>(
             (bf16*)qkv, T, nh, nkv, q_w, k_w, eps, positions, rope_table, (bf16*)k_cache, (bf16*)v_cache,
-            slots, page_size);
+            slots, page_size, first_head);
         LC_LAUNCH_CHECK("qk_norm_rope_write128");
         return 0;
     }
     const int waves = 4;
-    dim3 grid(T, (nh + 2 * nkv + waves - 1) / waves);
+    dim3 grid(T, (nh + 2 * nkv - first_head + waves - 1) / waves);
     if (dt == DT_F32)
         qk_norm_rope_write_kernel<float><<<grid, waves * kWave, 0, stream>>>(
             (float*)qkv, T, nh, nkv, d, q_w, k_w, eps, positions, rope_table, rot,
-            (float*)k_cache, (float*)v_cache, slots, page_size);
+            (float*)k_cache, (float*)v_cache, slots, page_size, first_head);
     else if (dt == DT_BF16)
         qk_norm_rope_write_kernel<bf16><<<grid, waves * kWave, 0, stream>>>(
             (bf16*)qkv, T, nh, nkv, d, q_w, k_w, eps, positions, rope_table, rot,
-            (bf16*)k_cache, (bf16*)v_cache, slots, page_size);
+            (bf16*)k_cache, (bf16*)v_cache, slots, page_size, first_head);
     else
         LC_CHECK(false, "qk_norm_rope_write: unknown dtype %d", dt);
     LC_LAUNCH_CHECK("qk_norm_rope_write");

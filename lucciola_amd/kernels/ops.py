@@ -37,12 +37,13 @@ _SIGNATURES = {
     "lc_gemm_bf16_residual": "ppppppiiip",
     "lc_gemm_bf16_scaled_rows": "pppiiiipifp",
     "lc_gemm_bf16_scaled_rows_supported": "iii",
-    "lc_qk_norm_rope_write": "piiiiippfppipppip",
+    "lc_qk_norm_rope_write": "piiiiippfppipppiip",
     "lc_attention_generic": "pipppipppiiiiiifip",
     "lc_attn_bf16_supported": "iiii",
     "lc_attn_decode_splits": "iii",
     "lc_attn_decode_bf16": "pippppppppp" + "iiiiii" + "f" + "ii" + "ippfpii" + "p",
-    "lc_attn_prefill_bf16": "pippppp" + "iiiiii" + "f" + "i" + "p",
+    "lc_attn_prefill_bf16": "pippppp" + "iiiiii" + "f" + "i" + "ipfpi" + "p",
+    "lc_attn_prefill_prepares_q": "ii",
     "lc_swiglu": "ppiiip",
     "lc_sample": "pppppiip",
     "lc_sample_workspace": "i",
@@ -355,12 +356,13 @@ def qk_norm_rope_write(qkv: torch.Tensor, nh: int, nkv: int, d: int,
                        eps: float, positions: Optional[torch.Tensor],
                        rope_table: Optional[torch.Tensor],
                        k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                       slots: Optional[torch.Tensor], page_size: int) -> None:
+                       slots: Optional[torch.Tensor], page_size: int, skip_q: bool = False) -> None:
     """In place on ``qkv`` [T, (nh + 2 nkv) d]: per-head RMSNorm of q and k (if weights are
     given), rotation by ``rope_table`` [positions, rot] (cos | sin halves) at each token's
     position, and the write of k and v into their cache slot ``slots`` [T]
     (page * page_size + offset; negative: no write).  Key cache [pages, nkv, page_size, d],
-    value cache [pages, nkv, d, page_size]."""
+    value cache [pages, nkv, d, page_size].  ``skip_q``: q is left raw (the attention kernels
+    prepare it themselves)."""
     _need(qkv, "qkv", None, 2)
     T = qkv.shape[0]
     if qkv.shape[1] != (nh + 2 * nkv) * d:
@@ -389,7 +391,7 @@ def qk_norm_rope_write(qkv: torch.Tensor, nh: int, nkv: int, d: int,
     _call("lc_qk_norm_rope_write", _ptr(qkv), _c_int(_dt(qkv)), _c_int(T), _c_int(nh), _c_int(nkv),
           _c_int(d), _ptr(q_weight), _ptr(k_weight), _c_float(eps), _ptr(positions),
           _ptr(rope_table), _c_int(rot), _ptr(k_cache), _ptr(v_cache), _ptr(slots),
-          _c_int(page_size), _stream())
+          _c_int(page_size), _c_int(nh if skip_q else 0), _stream())
 
 
 def _check_caches(k_cache, v_cache, nkv, page_size, d) -> None:
@@ -444,8 +446,8 @@ def attention(qkv: torch.Tensor, batch: AttentionBatch, k_cache: torch.Tensor,
               window: int = 0, prologue: Optional[QKPrologue] = None) -> torch.Tensor:
     """Causal attention of the q heads in ``qkv`` [T, (nh + 2 nkv) d] over the cached keys and
     values -> [T, nh d].  Without ``prologue`` the step's own keys and values have been written
-    already and q is ready; with it, ``qkv`` is raw: a step of single tokens does the prologue
-    inside the decode kernel, any other step runs :func:`qk_norm_rope_write` first."""
+    already and q is ready; with it, ``qkv`` is raw, and what is left raw in it afterwards is
+    not defined (q stays raw where the attention kernels prepare it on the fly)."""
     _need(qkv, "qkv", None, 2)
     _need(k_cache, "k cache", qkv.dtype, 4)
     _need(v_cache, "v cache", qkv.dtype, 4)
@@ -460,11 +462,22 @@ def attention(qkv: torch.Tensor, batch: AttentionBatch, k_cache: torch.Tensor,
     lib = library()
     fast = (qkv.dtype == torch.bfloat16 and batch.decode_tokens is not None
             and batch.prefill_tiles is not None and lib.lc_attn_bf16_supported(nh, nkv, d, page_size))
-    in_kernel = fast and prologue is not None and batch.num_decode == T
-    if prologue is not None and not in_kernel:
+    # who prepares q, k, v (norm, rotation, cache write) when they arrive raw: a step of single
+    # tokens does it all inside the decode kernel; otherwise a kernel of its own does k and v,
+    # and q too unless both attention kernels can prepare their q themselves
+    rope = prologue.rope_table if prologue is not None else None
+    if rope is not None:
+        _need(rope, "rotary table", torch.float32, 2)
+    rot = rope.shape[1] if rope is not None else 0
+    all_in_decode = fast and prologue is not None and batch.num_decode == T
+    own_q = (fast and prologue is not None and not all_in_decode
+             and (prologue.q_weight is None) == (prologue.k_weight is None)
+             and bool(lib.lc_attn_prefill_prepares_q(d, rot)))
+    if prologue is not None and not all_in_decode:
         qk_norm_rope_write(qkv, nh, nkv, d, prologue.q_weight, prologue.k_weight, prologue.eps,
                            batch.positions, prologue.rope_table, k_cache, v_cache, prologue.slots,
-                           page_size)
+                           page_size, skip_q=own_q)
+    in_kernel = all_in_decode or own_q
     if fast:
         mb = batch.block_table.shape[1]
         nd = batch.num_decode
@@ -474,9 +487,6 @@ def attention(qkv: torch.Tensor, batch: AttentionBatch, k_cache: torch.Tensor,
             if splits > 1:
                 part_o = torch.empty((nd * nh * splits * d,), dtype=torch.float32, device=qkv.device)
                 part_ml = torch.empty((nd * nh * splits * 2,), dtype=torch.float32, device=qkv.device)
-            rope = prologue.rope_table if in_kernel else None
-            if rope is not None:
-                _need(rope, "rotary table", torch.float32, 2)
             _call("lc_attn_decode_bf16", _ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
                   _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(batch.decode_tokens),
                   _ptr(batch.tok_req), _ptr(batch.positions), _ptr(batch.block_table), mb, nd, nh,
@@ -484,14 +494,17 @@ def attention(qkv: torch.Tensor, batch: AttentionBatch, k_cache: torch.Tensor,
                   1 if in_kernel else 0,
                   _ptr(prologue.q_weight if in_kernel else None),
                   _ptr(prologue.k_weight if in_kernel else None),
-                  _c_float(prologue.eps if in_kernel else 0.0), _ptr(rope),
-                  rope.shape[1] if rope is not None else 0,
-                  1 if in_kernel and prologue.slots is not None else 0, _stream())
+                  _c_float(prologue.eps if in_kernel else 0.0), _ptr(rope if in_kernel else None),
+                  rot if in_kernel else 0,
+                  1 if all_in_decode and prologue.slots is not None else 0, _stream())
         nt = batch.prefill_tiles.shape[0]
         if nt > 0:
             _call("lc_attn_prefill_bf16", _ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
                   _ptr(out), _ptr(batch.prefill_tiles), _ptr(batch.block_table), mb, nt, nh, nkv, d,
-                  page_size, scale, window, _stream())
+                  page_size, scale, window, 1 if own_q else 0,
+                  _ptr(prologue.q_weight if own_q else None),
+                  _c_float(prologue.eps if own_q else 0.0), _ptr(rope if own_q else None),
+                  rot if own_q else 0, _stream())
         return out
     _call("lc_attention_generic", _ptr(qkv), _c_int(qkv.shape[1]), _ptr(k_cache), _ptr(v_cache),
           _ptr(out), _c_int(_dt(qkv)), _ptr(batch.tok_req), _ptr(batch.positions),

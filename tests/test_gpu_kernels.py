@@ -428,6 +428,43 @@ def test_attention_decode_with_prologue_in_the_kernel(nh, nkv, d, window, rot, n
     close(got3, want, torch.bfloat16, atol=attention_atol(torch.bfloat16, vc1))
 
 
+@pytest.mark.parametrize("nh,nkv,d,window,rot,normed", [(32, 8, 128, 0, 128, True), (12, 4, 128, 40, 128, True),
+                                                        (6, 6, 128, 0, 0, True), (4, 2, 128, 0, 128, False),
+                                                        (6, 2, 96, 24, 96, True), (8, 1, 64, 0, 32, False)])
+def test_attention_mixed_step_with_raw_q(nh, nkv, d, window, rot, normed):
+    """Portions of prompts beside single tokens, q, k, v raw: a kernel of its own prepares k and
+    v; where the head size allows (128, rotated whole or not at all) it leaves q alone and both
+    attention kernels norm and rotate their q themselves, elsewhere it prepares q too.  Either
+    way the output is that of preparing everything first, and the caches agree to the bit."""
+    lengths = [1, 70, 300, 2049, 16, 150, 5000, 64]
+    new = [1, 70, 1, 130, 16, 2, 1, 1]
+    qkv, batch, kc, vc = paged_case(lengths, new, nh, nkv, d, 16, torch.bfloat16, seed=95)
+    qw = (1 + 0.1 * rnd(d, seed=96)) if normed else None
+    kw = (1 + 0.1 * rnd(d, seed=97)) if normed else None
+    table = None
+    if rot:
+        ang = torch.arange(6000, dtype=torch.float64)[:, None] * (10000.0 ** (-torch.arange(rot // 2, dtype=torch.float64) * 2 / rot))
+        table = torch.cat([ang.cos(), ang.sin()], 1).float().to(DEV)
+    pos = batch.positions.tolist()
+    req = batch.tok_req.tolist()
+    slots = torch.tensor([int(batch.block_table[r, p // 16]) * 16 + p % 16 for r, p in zip(req, pos)],
+                         dtype=torch.int32, device=DEV)
+    qkv1, kc1, vc1 = qkv.clone(), kc.clone(), vc.clone()
+    ops.qk_norm_rope_write(qkv1, nh, nkv, d, qw, kw, 1e-6, batch.positions, table, kc1, vc1, slots, 16)
+    want = ops.attention(qkv1, batch, kc1, vc1, nh, nkv, d, 16, d ** -0.5, window)
+    qkv2, kc2, vc2 = qkv.clone(), kc.clone(), vc.clone()
+    got = ops.attention(qkv2, batch, kc2, vc2, nh, nkv, d, 16, d ** -0.5, window,
+                        ops.QKPrologue(qw, kw, 1e-6, table, slots))
+    assert torch.equal(kc2, kc1) and torch.equal(vc2, vc1)
+    own_q = bool(ops.library().lc_attn_prefill_prepares_q(d, rot))
+    assert own_q == (d == 128)
+    q_cols = nh * d
+    assert torch.equal(qkv2[:, :q_cols], (qkv if own_q else qkv1)[:, :q_cols])     # q raw or prepared
+    assert torch.equal(qkv2[:, q_cols:q_cols + nkv * d], qkv1[:, q_cols:q_cols + nkv * d])   # k prepared
+    close(got, want, torch.bfloat16, atol=attention_atol(torch.bfloat16, vc1))
+    assert float((got.float() - want.float()).abs().max()) <= 2.0 ** -6 * float(want.float().abs().max())
+
+
 @pytest.mark.parametrize("M,I,K", [(1, 16, 128), (8, 200, 256), (33, 1000, 128), (64, 96, 384), (65, 136, 256),
                                    (300, 520, 128), (2048, 256, 256), (40, 2048, 1024), (64, 12288, 512),
                                    (2, 72, 640), (14, 8200, 256), (16, 8192, 128)])
