@@ -648,7 +648,9 @@ template <int D>
 static int launch_prefill(const bf16* qkv, int q_stride, const bf16* k, const bf16* v, bf16* out,
                           const int* tiles, const int* table, int max_blocks, int NT, int nh,
                           int nkv, float scale_log2, int window, DecodePrologue pro, hipStream_t s) {
-    if ((nh / nkv) % 2 == 0)
+    // pairs of heads share the keys and values they read; with so few tiles that half of the CUs
+    // would get nothing to do, single heads and twice the workgroups are faster (measured)
+    if ((nh / nkv) % 2 == 0 && (long long)NT * (nh / 2) > 128)
         attn_prefill_kernel<D, 2><<<dim3(NT, nh / 2), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
                                                                    max_blocks, nh, nkv, scale_log2, window, pro);
     else
