@@ -304,6 +304,56 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write128_kernel(
         *reinterpret_cast<head_chunk*>(k_cache + (((size_t)page * nkv + kvh) * page_size + off) * d + 8 * j) = done;
 }
 
+// k and v alone (q is left to the attention kernels), bfloat16 heads of 128 as above: a
+// workgroup takes 16 consecutive rows of the batch and one kv head, 16 lanes a row.  A value
+// page holds its 16 positions side by side for every entry of the head, so a row's values go
+// to 128 places 32 bytes apart.  When the workgroup's 16 rows fill one page in order (the rows
+// of a prompt do, from a page's first position on), it turns the 16 x 128 values round in
+// LDS and writes the page's 4 KB of this head in one piece; otherwise every row scatters its
+// own.
+__global__ __launch_bounds__(256) void kv_norm_rope_write128_kernel(
+    bf16* __restrict__ qkv, int T_tokens, int nh, int nkv, const float* __restrict__ k_w, float eps,
+    const int* __restrict__ positions, const float* __restrict__ rope_table,
+    bf16* __restrict__ k_cache, bf16* __restrict__ v_cache, const int* __restrict__ slots,
+    int page_size) {
+    constexpr int d = 128, LD = d + 8;            // padded rows: the gather below spreads over the banks
+    __shared__ __attribute__((aligned(16))) bf16 turned[16 * LD];
+    __shared__ int whole;
+    const int t0 = blockIdx.x * 16, kvh = blockIdx.y, g = threadIdx.x >> 4, j = threadIdx.x & 15;
+    const int t = t0 + g, heads = nh + 2 * nkv;
+    const bool live = t < T_tokens;                           // whole groups of 16 lanes
+    const int slot = live ? slots[t] : -1, base = slots[t0];
+    if (threadIdx.x == 0) whole = (page_size == 16 && base >= 0 && base % 16 == 0) ? 1 : 0;
+    __syncthreads();
+    if (j == 0 && slot != base + g) whole = 0;                // (everyone who writes, writes 0)
+    __syncthreads();
+    const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot - page * page_size : 0;
+    head_chunk value;
+    if (live) {
+        bf16* x = qkv + ((size_t)t * heads + nh + kvh) * d + 8 * j;
+        const float* cs = rope_table ? rope_table + (size_t)positions[t] * d : nullptr;
+        const head_chunk key = head128_norm_rope(*reinterpret_cast<const head_chunk*>(x), j, k_w, eps, cs);
+        *reinterpret_cast<head_chunk*>(x) = key;
+        if (slot >= 0)
+            *reinterpret_cast<head_chunk*>(k_cache + (((size_t)page * nkv + kvh) * page_size + off) * d + 8 * j) = key;
+        value = *reinterpret_cast<const head_chunk*>(x + (size_t)nkv * d);
+    }
+    if (whole) {                                              // the same for the whole workgroup
+        *reinterpret_cast<head_chunk*>(&turned[g * LD + 8 * j]) = value;
+        __syncthreads();
+        const int dim = threadIdx.x >> 1, half = threadIdx.x & 1;
+        head_chunk column;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) column[i] = turned[(8 * half + i) * LD + dim];
+        const int first_page = base / 16;
+        *reinterpret_cast<head_chunk*>(v_cache + (((size_t)first_page * nkv + kvh) * d + dim) * 16 + 8 * half) = column;
+    } else if (live && slot >= 0) {
+        bf16* col = v_cache + ((size_t)page * nkv + kvh) * d * page_size + off;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) col[(size_t)(8 * j + e) * page_size] = value[e];
+    }
+}
+
 // ------------------------------------------------------------------------------- SwiGLU
 // gu: [T, 2 I] (gate columns, then up columns) -> out [T, I]
 template <typename T>
@@ -413,6 +463,13 @@ LC_API int lc_qk_norm_rope_write(void* qkv, int dt, int T, int nh, int nkv, int 
     if (!rope_table) rot = 0;
     if (dt == DT_BF16 && d == 128 && (rot == 0 || rot == 128) && (q_w == nullptr) == (k_w == nullptr) &&
         (uintptr_t)qkv % 16 == 0 && (uintptr_t)k_cache % 16 == 0) {
+        if (first_head == nh && k_cache && slots) {
+            kv_norm_rope_write128_kernel<<<dim3((T + 15) / 16, nkv), 256, 0, stream>>>(
+                (bf16*)qkv, T, nh, nkv, k_w, eps, positions, rope_table, (bf16*)k_cache, (bf16*)v_cache,
+                slots, page_size);
+            LC_LAUNCH_CHECK("kv_norm_rope_write128");
+            return 0;
+        }
         const long long groups = (long long)T * (nh + 2 * nkv - first_head);
         qk_norm_rope_write128_kernel<<<(unsigned)((groups + 15) / 16), 256, 0, stream>>>(
             (bf16*)qkv, T, nh, nkv, q_w, k_w, eps, positions, rope_table, (bf16*)k_cache, (bf16*)v_cache,

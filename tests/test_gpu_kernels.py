@@ -465,6 +465,38 @@ def test_attention_mixed_step_with_raw_q(nh, nkv, d, window, rot, normed):
     assert float((got.float() - want.float()).abs().max()) <= 2.0 ** -6 * float(want.float().abs().max())
 
 
+@pytest.mark.parametrize("lengths,new", [([70], [70]), ([102, 33], [70, 33]), ([40 + 50], [50]), ([64, 16, 200], [64, 16, 100]),
+                                         ([2048], [2048])])
+def test_k_and_v_alone_page_by_page(lengths, new):
+    """q left to the attention kernels, heads of 128: where 16 rows of the batch fill one page
+    in order the values are turned round in LDS and written as one piece, elsewhere row by row
+    (a portion that starts in the middle of a page, a second request whose rows do not start
+    at a multiple of 16, the ragged end).  Caches and k in place must equal the plain version's,
+    q must stay raw."""
+    nh, nkv, d, page = 6, 3, 128, 16
+    qkv, batch, kc, vc = paged_case(lengths, new, nh, nkv, d, page, torch.bfloat16, seed=98)
+    kw = 1 + 0.1 * rnd(d, seed=99)
+    qw = 1 + 0.1 * rnd(d, seed=100)
+    ang = torch.arange(4096, dtype=torch.float64)[:, None] * (10000.0 ** (-torch.arange(d // 2, dtype=torch.float64) * 2 / d))
+    table = torch.cat([ang.cos(), ang.sin()], 1).float().to(DEV)
+    pos, req = batch.positions.tolist(), batch.tok_req.tolist()
+    slots = torch.tensor([int(batch.block_table[r, p // page]) * page + p % page for r, p in zip(req, pos)],
+                         dtype=torch.int32, device=DEV)
+    got_qkv, got_k, got_v = qkv.clone(), kc.clone(), vc.clone()
+    ops.qk_norm_rope_write(got_qkv, nh, nkv, d, qw, kw, 1e-6, batch.positions, table, got_k, got_v, slots, page,
+                           skip_q=True)
+    want_qkv, want_k, want_v = qkv.clone(), kc.clone(), vc.clone()
+    ref.qk_norm_rope_write(want_qkv, nh, nkv, d, qw, kw, 1e-6, batch.positions, table, want_k, want_v, slots, page)
+    assert torch.equal(got_qkv[:, :nh * d], qkv[:, :nh * d])
+    assert torch.equal(got_v, want_v)                          # copies
+    close(got_k, want_k, torch.bfloat16)
+    close(got_qkv[:, nh * d:(nh + nkv) * d], want_qkv[:, nh * d:(nh + nkv) * d], torch.bfloat16)
+    # and to the bit what the kernel for all heads writes
+    all_qkv, all_k, all_v = qkv.clone(), kc.clone(), vc.clone()
+    ops.qk_norm_rope_write(all_qkv, nh, nkv, d, qw, kw, 1e-6, batch.positions, table, all_k, all_v, slots, page)
+    assert torch.equal(got_k, all_k) and torch.equal(got_v, all_v)
+
+
 @pytest.mark.parametrize("M,I,K", [(1, 16, 128), (8, 200, 256), (33, 1000, 128), (64, 96, 384), (65, 136, 256),
                                    (300, 520, 128), (2048, 256, 256), (40, 2048, 1024), (64, 12288, 512),
                                    (2, 72, 640), (14, 8200, 256), (16, 8192, 128)])
