@@ -861,7 +861,7 @@ static int launch_bf16(const bf16* x, const bf16* w, TO* out, float* workspace, 
     const int tile = pick_tile(M, N, K);
     const TailPlan tail = tail_plan(tile, M, N, K);
     switch (tile) {
-    case TILE_64x128:  return launch_tiled<64, 128, 4, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
+    case TILE_64x128:  return launch_tiled<64, 128, 3, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     case TILE_128x128: return launch_tiled<128, 128, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     case TILE_256x128: return launch_tiled<256, 128, 3, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     case TILE_256x192: return launch_tiled<256, 192, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
@@ -1023,7 +1023,7 @@ LC_API int lc_gemm_bf16_partials(const void* x, const void* w, float* partials, 
     const bf16* wb = (const bf16*)w;
     if (pick_tile(M, N, K) == TILE_64x128) {
         const int tiles_m = (M + 63) / 64, tiles = tiles_m * ((N + 127) / 128);
-        gemm_tiled_kernel<64, 128, 4, 0, true, float><<<dim3(tiles, shares), 256, 0, stream>>>(
+        gemm_tiled_kernel<64, 128, 3, 0, true, float><<<dim3(tiles, shares), 256, 0, stream>>>(
             xb, wb, nullptr, partials, M, N, K, tiles_m, 0, tiles, 0);
     } else {
         const int tiles_m = (M + 127) / 128, tiles = tiles_m * ((N + 127) / 128);
