@@ -3,8 +3,9 @@
 Default run: the layer sizes of the Qwen3-8B-shaped configuration (36 layers, hidden 4096, 32
 query heads, 8 kv heads, head size 128, intermediate 12288, vocabulary 151936), random
 weights, bfloat16, a batch of 8 requests at a context of 8,192 tokens.  One "step" is one
-decode step of the whole batch through the engine's own step function and sampler (greedy),
-the sampled tokens being fed to the next step.  The cache of the live requests is filled with
+decode step of the whole batch through the engine's own step function and sampler (greedy).
+As in the engine's loop, the sampled tokens reach the next step on the device and the host
+reads them while that step runs (`--run-ahead 0`: the host waits for them first).  The cache of the live requests is filled with
 random keys and values instead of running their 8,191-token prompts (a decode step's cost
 does not depend on what the cache holds); the prefill figure is a real 2,048-token prompt in
 one step.  Prints ONE JSON line.
@@ -43,6 +44,8 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--points", default="1,64", help="further decode batch sizes (comma list, '' for none)")
     ap.add_argument("--block-size", type=int, default=16)
+    ap.add_argument("--run-ahead", type=int, default=1, choices=[0, 1],
+                    help="1: a step is queued before the host has read the tokens of the one before")
     ap.add_argument("--workload", default="decode", choices=["decode", "mixed"],
                     help="decode: the default line; mixed: 64 requests with prompts of 16 to 2,048 "
                          "tokens through the scheduler (Qwen3-0.6B-shaped), chunked prefill beside decode")
@@ -55,7 +58,7 @@ def main() -> int:
 
     import torch
     from lucciola_amd.config.engine_config import EngineConfig
-    from lucciola_amd.engine.batch import StepEntry
+    from lucciola_amd.engine.batch import PENDING, Carry, StepEntry
     from lucciola_amd.engine.loading import random_model
     from lucciola_amd.engine.runner import ModelRunner
     from lucciola_amd.sampling.sampler import Sampler, SamplingParams
@@ -106,16 +109,30 @@ def main() -> int:
         tokens = torch.randint(0, V, (batch,), generator=gen).tolist()
         params = [SamplingParams(max_new_tokens=1 << 30)] * batch
 
+        rows = {n: i for i, n in enumerate(names)}
+        under_way = None        # the step whose tokens the host has not read yet
+
         def one():
-            nonlocal tokens
-            logits = runner.step([StepEntry(n, [t], [0]) for n, t in zip(names, tokens)])
-            tokens = sampler.sample(logits, params, [0] * batch)
+            nonlocal tokens, under_way
+            if under_way is None:
+                logits = runner.step([StepEntry(n, [t], [0]) for n, t in zip(names, tokens)])
+            else:
+                logits = runner.step([StepEntry(n, [PENDING], [0]) for n in names],
+                                     Carry(under_way.ids, rows))
+            sampled = sampler.sample_async(logits, params, [0] * batch)
+            if under_way is not None:
+                tokens = under_way.tokens()
+            under_way = sampled
+            if not args.run_ahead:
+                tokens, under_way = sampled.tokens(), None
         for _ in range(warmup):
             one()
         torch.cuda.synchronize()
         t = time.perf_counter()
         for _ in range(steps):
             one()
+        if under_way is not None:
+            tokens = under_way.tokens()
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t) * 1e3 / steps
         ctx_mid = args.context + warmup + steps / 2.0
@@ -200,7 +217,7 @@ def mixed_workload(args, dtype, dev) -> int:
     blocks = -(-total_tokens // args.block_size) + 64
     engine = LLMEngine.from_random(cfg, 0, EngineConfig(
         dtype=dtype, block_size=args.block_size, max_blocks=blocks, max_seqs=64,
-        max_tokens_per_step=args.max_tokens_per_step, device=dev))
+        max_tokens_per_step=args.max_tokens_per_step, device=dev, run_ahead=bool(args.run_ahead)))
     params = SamplingParams(max_new_tokens=args.new_tokens, ignore_eos=True)
     engine.generate(prompts[:4], SamplingParams(max_new_tokens=4, ignore_eos=True))   # warm-up
     torch.cuda.synchronize()

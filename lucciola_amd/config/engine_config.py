@@ -41,6 +41,7 @@ class EngineConfig:
     use_graphs: bool = True         # replay decode steps from HIP graphs (bfloat16 on the GPU)
     graph_max_batch: int = 256      # largest decode batch that is captured
     graph_cache_size: int = 16      # captured steps kept
+    run_ahead: bool = True          # queue a step before the host has the tokens of the one before
 
     def __post_init__(self) -> None:
         self.dtype = parse_dtype(self.dtype)

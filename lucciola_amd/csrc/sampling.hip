@@ -168,6 +168,16 @@ __global__ __launch_bounds__(SP_THREADS) void sample_pick_kernel(const float* __
     }
 }
 
+// ids[i] = sampled[source[i]] where source[i] >= 0: the tokens a step sampled go into the next
+// step's batch on the device, without a round trip through the host.
+__global__ void feed_tokens_kernel(int* __restrict__ ids, const int* __restrict__ source,
+                                   const int* __restrict__ sampled, int T, int S) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= T) return;
+    int s = source[i];
+    if (s >= 0 && s < S) ids[i] = sampled[s];
+}
+
 }  // namespace lc
 
 using namespace lc;
@@ -197,5 +207,17 @@ LC_API int lc_sample(const float* logits, const float* temperature, const float*
     sample_pick_kernel<<<R, SP_THREADS, 0, stream>>>(logits, temperature, uniform, ws_max, ws_idx,
                                                      ws_sum, out, V);
     LC_LAUNCH_CHECK("sample_pick");
+    return 0;
+}
+
+// ids [T] of a batch: where source[i] >= 0 the id is taken from sampled[source[i]] (S rows of an
+// earlier lc_sample on the same stream); other ids stay.
+LC_API int lc_feed_tokens(int* ids, const int* source, const int* sampled, int T, int S,
+                          hipStream_t stream) {
+    LC_CHECK(T >= 0 && S >= 0, "feed_tokens: bad sizes T=%d S=%d", T, S);
+    if (T == 0 || S == 0) return 0;
+    LC_CHECK(ids && source && sampled, "feed_tokens: null pointer");
+    feed_tokens_kernel<<<(T + 255) / 256, 256, 0, stream>>>(ids, source, sampled, T, S);
+    LC_LAUNCH_CHECK("feed_tokens");
     return 0;
 }

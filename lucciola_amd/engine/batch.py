@@ -18,6 +18,7 @@ from ..cache.manager import CacheManager
 from ..kernels.ops import AttentionBatch
 
 PREFILL_TILE = 64   # query rows of one work item of the prefill attention kernel
+PENDING = -1        # a token that an earlier step has sampled and the host has not seen yet
 
 
 @dataclass
@@ -25,8 +26,17 @@ class StepEntry:
     """A request's next tokens, and the places among them whose logits are wanted."""
 
     request: Hashable
-    tokens: Sequence[int]
+    tokens: Sequence[int]       # [PENDING]: the token comes from the carry given to the step
     want: Sequence[int] = ()
+
+
+@dataclass
+class Carry:
+    """Tokens that an earlier step sampled, still on the device: ``ids[rows[request]]`` is the
+    next token of ``request``."""
+
+    ids: torch.Tensor           # int32 [S]
+    rows: dict
 
 
 @dataclass
@@ -56,6 +66,7 @@ class StepBatch:
     tok_req: torch.Tensor         # int32 [T]
     want_rows: torch.Tensor       # int32 [W] rows of the batch whose logits are wanted
     slot_ids: torch.Tensor        # int32 [R]
+    feed: torch.Tensor            # int32 [T] row of the carry a token is taken from, or -1
     groups: List[AttentionBatch] = field(default_factory=list)
     num_wanted: int = 0
     buffer: Optional[torch.Tensor] = None   # the one device buffer all of the above view
@@ -110,12 +121,14 @@ class _Packer:
 
 def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
                 pad_blocks: Optional[int] = None, into: Optional[torch.Tensor] = None,
-                refresh_only: bool = False) -> Optional[StepBatch]:
+                refresh_only: bool = False, carry_rows: Optional[dict] = None) -> Optional[StepBatch]:
     """Lay the entries out as one flat batch.  Pages for the new tokens must be reserved.
 
     ``pad_blocks``: width of the block tables (at least the longest table), so that batches of
     the same make-up have the same layout; ``into``: the buffer of such an earlier batch;
-    ``refresh_only``: only bring that buffer up to date (its views exist already), return None."""
+    ``refresh_only``: only bring that buffer up to date (its views exist already), return None;
+    ``carry_rows``: for entries whose one token is PENDING, the row of the carry it comes from
+    (the caller copies it in on the device; the host's copy holds token 0 there)."""
     bs = cache.block_size
     R = len(entries)
     requests = [e.request for e in entries]
@@ -166,8 +179,22 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
         tile_list.sort(key=lambda t: -(t[3] + t[2]))
         tiles = [v for t in tile_list for v in t]
 
+    feed = np.full(T, -1, dtype=np.int32)
+    pending = np.nonzero(token_ids == PENDING)[0]
+    if pending.size:
+        starts = {q_start[r]: r for r in range(R) if q_start[r + 1] - q_start[r] == 1}
+        for i in pending.tolist():
+            r = starts.get(i)
+            if r is None or carry_rows is None or requests[r] not in carry_rows:
+                raise ValueError(f"request {requests[int(tok_req[i])]!r}: a pending token must be "
+                                 "an entry's only token and have a row in the step's carry")
+            feed[i] = carry_rows[requests[r]]
+        token_ids = token_ids.copy()
+        token_ids[pending] = 0
+
     pk = _Packer()
     h_tok = pk.add(token_ids)
+    h_feed = pk.add(feed)
     h_pos = pk.add(positions)
     h_req = pk.add(tok_req)
     h_want = pk.add(want_rows)
@@ -214,5 +241,5 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
         first_position=first_pos, slot_list=slot_list,
         max_position=int(positions.max()) if T else 0,
         token_ids=pk.view(h_tok), positions=pk.view(h_pos), tok_req=pk.view(h_req),
-        want_rows=pk.view(h_want), slot_ids=pk.view(h_slot), groups=groups,
+        want_rows=pk.view(h_want), slot_ids=pk.view(h_slot), feed=pk.view(h_feed), groups=groups,
         num_wanted=num_wanted, buffer=buffer)

@@ -1,7 +1,12 @@
-"""The engine: model runner + scheduler + sampler, stepped synchronously.
+"""The engine: model runner + scheduler + sampler.
 
 ``LLMEngine.step`` is one turn of the reference's engine loop (src/async_engine.cc:113-160):
-schedule, run the model, pick tokens, apply the stop rules, free what has finished.
+schedule, run the model, pick tokens, apply the stop rules, free what has finished.  The
+reference waits for a step's tokens before it schedules the next.  Here the next step is
+queued first (``EngineConfig.run_ahead``): the sampled ids stay on the device and feed the
+next step from there, the host reads them one step late, and the GPU does not idle while the
+host schedules.  What the host cannot know a step early is an end-of-sequence token: such a
+request runs one step too many, whose token is thrown away.
 """
 from __future__ import annotations
 
@@ -10,6 +15,7 @@ from typing import Callable, Dict, List, Optional, Sequence as Seq
 
 from ..config.engine_config import EngineConfig
 from ..sampling.sampler import Sampler, SamplingParams
+from .batch import PENDING, Carry
 from .loading import load_model, random_model
 from .runner import ModelRunner
 from .scheduler import ScheduledStep, Scheduler
@@ -21,6 +27,16 @@ class StepOutput:
     seq_id: int
     token: int
     finished: bool
+
+
+@dataclass
+class _QueuedStep:
+    """A step whose tokens the host has not read yet."""
+
+    sampled: object                 # SampledTokens
+    seqs: List[Sequence]            # the requests a token was sampled for, in row order
+    places: List[int]               # where in each request's token list that token goes
+    last: List[bool]                # the request reached max_new_tokens with this token
 
 
 class LLMEngine:
@@ -35,6 +51,7 @@ class LLMEngine:
         self.sampler = Sampler()
         self.sequences: Dict[int, Sequence] = {}
         self._next_id = 1
+        self._queued: Optional[_QueuedStep] = None
         self.eos_token_ids = tuple(getattr(model_config, "eos_token_ids", ()) or ())
 
     @classmethod
@@ -65,26 +82,68 @@ class LLMEngine:
         return seq.seq_id
 
     def has_unfinished_requests(self) -> bool:
-        return self.scheduler.has_unfinished_requests()
+        return self._queued is not None or self.scheduler.has_unfinished_requests()
 
     # ------------------------------------------------------------------ one step
     def step(self) -> List[StepOutput]:
+        """Queue the next step, then hand out the tokens of the step queued before it (without
+        ``run_ahead``: of this very step)."""
+        if not self.config.run_ahead:
+            only = self._launch(None)
+            return self._collect(only) if only is not None else []
+        before = self._queued
+        self._queued = self._launch(before)
+        if before is None:
+            if self._queued is None:
+                return []
+            # nothing was in flight: queue a second step, so that from now on one is always
+            # running while the host reads the tokens of the one before
+            before = self._queued
+            self._queued = self._launch(before)
+        return self._collect(before)
+
+    def _launch(self, before: Optional[_QueuedStep]) -> Optional[_QueuedStep]:
+        """Schedule and queue one step.  Requests whose last token is still on the device
+        (sampled by ``before``) are fed from there."""
         sched: ScheduledStep = self.scheduler.step()
         if sched.num_seqs == 0:
-            if self.scheduler.has_unfinished_requests() and not sched.preempted:
+            if before is None and self.scheduler.has_unfinished_requests() and not sched.preempted:
                 raise RuntimeError("the scheduler has requests but can run none of them")
-            return []
-        logits = self.runner.step(sched.entries)
+            return None
+        carry = None
+        if before is not None and before.sampled is not None:
+            carry = Carry(before.sampled.ids, {s.seq_id: row for row, s in enumerate(before.seqs)})
+        logits = self.runner.step(sched.entries, carry)
         sampling = [seq for seq, s in zip(sched.seqs, sched.samples) if s]
+        if not sampling:
+            return _QueuedStep(None, [], [], [])
+        sampled = self.sampler.sample_async(logits, [s.params for s in sampling],
+                                            [s.num_generated for s in sampling])
+        places, last = [], []
+        for seq in sampling:
+            places.append(seq.get_len())
+            done = self.scheduler.on_token(seq, PENDING)    # the count is known, the token is not
+            if done:
+                self.scheduler.free_sequence(seq)
+            last.append(done)
+        return _QueuedStep(sampled, sampling, places, last)
+
+    def _collect(self, step: _QueuedStep) -> List[StepOutput]:
+        """Read a queued step's tokens, put them where they belong and apply the stop rules
+        that need the token itself."""
         outputs: List[StepOutput] = []
-        if sampling:
-            tokens = self.sampler.sample(logits, [s.params for s in sampling],
-                                         [s.num_generated for s in sampling])
-            for seq, token in zip(sampling, tokens):
-                finished = self.scheduler.on_token(seq, token)
-                if finished:
-                    self.scheduler.free_sequence(seq)
-                outputs.append(StepOutput(seq.seq_id, token, finished))
+        if step.sampled is None:
+            return outputs
+        for seq, place, last, token in zip(step.seqs, step.places, step.last, step.sampled.tokens()):
+            if place >= seq.get_len():
+                continue        # the request ended on an earlier token: this one is thrown away
+            seq.token_ids[place] = token
+            finished = last
+            if not finished and seq.stops_on(token):
+                del seq.token_ids[place + 1:]       # a token queued after the last one
+                self.scheduler.free_sequence(seq)
+                finished = True
+            outputs.append(StepOutput(seq.seq_id, token, finished))
         return outputs
 
     def stats(self) -> Dict[str, int]:

@@ -17,7 +17,8 @@ from ..cache.manager import CacheManager
 from ..cache.page_pool import OutOfPages
 from ..config.engine_config import EngineConfig
 from ..models.causal_lm import CausalLM
-from .batch import SiteView, StepBatch, StepEntry, build_batch
+from ..kernels import ops
+from .batch import PENDING, Carry, SiteView, StepBatch, StepEntry, build_batch
 
 
 class _CapturedStep:
@@ -74,9 +75,14 @@ class ModelRunner:
                 taken[gi] = taken.get(gi, 0) + self.cache.pages_needed(g, have, len(e.tokens))
         return new_requests <= self.cache.slots.num_free()
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], carry: Optional[Carry] = None) -> torch.Tensor:
         """Run the entries as one batch; returns float32 logits [wanted places, vocab] in the
         order of the entries and of each entry's ``want``.
+
+        Nothing here waits for the GPU: the kernels are queued on the current stream and the
+        logits are read in stream order.  An entry whose only token is ``PENDING`` takes the id
+        that ``carry`` holds for its request, on the device: a caller may queue a request's
+        next step before it has seen the token that the last one sampled.
 
         A request that the cache does not know is admitted.  Raises OutOfPages (and changes
         nothing) if the pages or slots for the whole batch are not there."""
@@ -89,10 +95,19 @@ class ModelRunner:
             twice = next(n for n in names if names.count(n) > 1)
             raise ValueError(f"request {twice!r} appears twice in one step")
         limit = self.model.spec.max_positions
-        if all(len(e.tokens) == 1 for e in entries):      # one check for a step of single tokens
-            self._check_ids(np.asarray([e.tokens[0] for e in entries]), entries)
+        fed = [e for e in entries if len(e.tokens) == 1 and e.tokens[0] == PENDING]
+        if fed:
+            if carry is None:
+                raise ValueError(f"request {fed[0].request!r}: a pending token and no carry to take it from")
+            for e in fed:
+                if not 0 <= carry.rows.get(e.request, -1) < carry.ids.shape[0]:
+                    raise ValueError(f"request {e.request!r}: no row in the step's carry")
+        known = [e for e in entries if not (len(e.tokens) == 1 and e.tokens[0] == PENDING)] if fed else entries
+        if all(len(e.tokens) == 1 for e in known):      # one check for a step of single tokens
+            if known:
+                self._check_ids(np.asarray([e.tokens[0] for e in known]), known)
         else:
-            for e in entries:
+            for e in known:
                 self._check_ids(np.asarray(e.tokens), [e])
         if limit:
             for e in entries:
@@ -117,9 +132,12 @@ class ModelRunner:
 
         if self.use_graphs and len(entries) <= self.config.graph_max_batch and all(
                 len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
-            logits, num_tokens = self._graph_step(entries), len(entries)
+            logits, num_tokens = self._graph_step(entries, carry if fed else None), len(entries)
         else:
-            batch = build_batch(entries, self.cache, self.device)
+            batch = build_batch(entries, self.cache, self.device,
+                                carry_rows=carry.rows if fed else None)
+            if fed:
+                ops.feed_tokens(batch.token_ids, batch.feed, carry.ids)
             logits, num_tokens = self.model.forward(batch, self._sites(batch)), batch.num_tokens
         for e in entries:
             self.cache.commit(e.request)
@@ -137,7 +155,7 @@ class ModelRunner:
             raise ValueError(f"request {who!r}: token id {bad} is outside the vocabulary of {V}")
 
     # ------------------------------------------------------------------ graph replay
-    def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def _graph_step(self, entries: Sequence[StepEntry], carry: Optional[Carry]) -> torch.Tensor:
         """A step of single tokens, one per request, each wanting its logits: captured once per
         (number of requests, block-table width) as a HIP graph and replayed afterwards.  Only the
         batch description changes between replays, and it lives in one device buffer that is
@@ -159,7 +177,10 @@ class ModelRunner:
         captured = self._graphs.get(key)
         next_position = max(self.cache.length(e.request) for e in entries)
         if captured is None or not self.model.positions_ready(next_position):
-            batch = build_batch(entries, self.cache, self.device, pad_blocks=pad)
+            batch = build_batch(entries, self.cache, self.device, pad_blocks=pad,
+                                carry_rows=carry.rows if carry else None)
+            if carry:
+                ops.feed_tokens(batch.token_ids, batch.feed, carry.ids)
             sites = self._sites(batch)
             logits = self.model.forward(batch, sites)       # runs the step (and grows tables)
             if self.model.position_epoch() != epoch:
@@ -174,7 +195,9 @@ class ModelRunner:
             self._graphs[key] = _CapturedStep(graph, batch, sites, static_logits)
             return logits[:real]
         build_batch(entries, self.cache, self.device, pad_blocks=pad, into=captured.batch.buffer,
-                    refresh_only=True)
+                    refresh_only=True, carry_rows=carry.rows if carry else None)
+        if carry:       # outside the graph: the carry is at another address every step
+            ops.feed_tokens(captured.batch.token_ids, captured.batch.feed, carry.ids)
         captured.graph.replay()
         self.graph_replays += 1
         return captured.logits[:real].clone()      # the next replay overwrites the graph's own output

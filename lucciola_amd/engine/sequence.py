@@ -63,7 +63,8 @@ class Sequence:
         end-of-sequence id, or max_new_tokens generated."""
         if self.num_generated >= self.params.max_new_tokens:
             return True
-        if self.num_generated and not self.params.ignore_eos \
-                and self.token_ids[-1] in self.params.eos_token_ids:
-            return True
-        return False
+        return bool(self.num_generated) and self.stops_on(self.token_ids[-1])
+
+    def stops_on(self, token: int) -> bool:
+        """Is this generated token an end-of-sequence id that the request heeds."""
+        return not self.params.ignore_eos and token in self.params.eos_token_ids

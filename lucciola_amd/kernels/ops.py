@@ -47,6 +47,7 @@ _SIGNATURES = {
     "lc_swiglu": "ppiiip",
     "lc_sample": "pppppiip",
     "lc_sample_workspace": "i",
+    "lc_feed_tokens": "pppiip",
 }
 
 
@@ -544,3 +545,15 @@ def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,
     _call("lc_sample", _ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(out), _ptr(workspace),
           _c_int(R), _c_int(V), _stream())
     return out
+
+
+def feed_tokens(ids: torch.Tensor, source: torch.Tensor, sampled: torch.Tensor) -> None:
+    """``ids[i] = sampled[source[i]]`` wherever ``source[i] >= 0`` (all int32, on the device):
+    what an earlier step sampled becomes a later step's input without passing the host."""
+    _need(ids, "fed ids", torch.int32, 1)
+    _need(source, "feed source", torch.int32, 1)
+    _need(sampled, "sampled ids", torch.int32, 1)
+    if source.shape[0] != ids.shape[0]:
+        raise KernelError("feed_tokens: one source row per id")
+    _call("lc_feed_tokens", _ptr(ids), _ptr(source), _ptr(sampled), _c_int(ids.shape[0]),
+          _c_int(sampled.shape[0]), _stream())

@@ -50,21 +50,53 @@ class SamplingParams:
         self.eos_token_ids = tuple(int(t) for t in self.eos_token_ids)
 
 
+class SampledTokens:
+    """The tokens one step sampled: ``ids`` (int32, on the logits' device) exists as soon as the
+    kernels are queued, and may feed the next step from there; ``tokens()`` waits for the copy
+    to the host."""
+
+    def __init__(self, ids: torch.Tensor):
+        self.ids = ids
+        self._list = None
+        self._event = None
+        if ids.device.type == "cuda":
+            self._host = torch.empty(ids.shape, dtype=ids.dtype, pin_memory=True)
+            self._host.copy_(ids, non_blocking=True)
+            self._event = torch.cuda.Event()
+            self._event.record()
+        else:
+            self._host = ids
+
+    def tokens(self) -> List[int]:
+        if self._list is None:
+            if self._event is not None:
+                self._event.synchronize()
+            self._list = [int(t) for t in self._host.tolist()]
+        return self._list
+
+
 class Sampler:
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams],
                generated: Sequence[int]) -> List[int]:
         """One token per row of ``logits``; ``generated[i]`` is how many tokens row i's request
         has generated so far (the index of the token drawn now)."""
+        return self.sample_async(logits, params, generated).tokens()
+
+    def sample_async(self, logits: torch.Tensor, params: Sequence[SamplingParams],
+                     generated: Sequence[int]) -> SampledTokens:
+        """As ``sample``, without waiting for the GPU."""
         if logits.shape[0] != len(params):
             raise ValueError("one row of logits per request")
         if logits.shape[0] == 0:
-            return []
+            return SampledTokens(torch.empty(0, dtype=torch.int32))
         if all(p.temperature <= 0 for p in params):
             ids = ops.sample(logits)
         else:
             temps = np.array([p.temperature for p in params], dtype=np.float32)
             us = np.array([uniform_for(p.seed, g) for p, g in zip(params, generated)],
                           dtype=np.float32)
-            both = torch.from_numpy(np.stack([temps, us])).to(logits.device)
+            both = torch.from_numpy(np.stack([temps, us]))
+            if logits.device.type == "cuda":
+                both = both.pin_memory().to(logits.device, non_blocking=True)
             ids = ops.sample(logits, both[0].contiguous(), both[1].contiguous())
-        return [int(t) for t in ids.tolist()]
+        return SampledTokens(ids)

@@ -119,7 +119,12 @@ def sample(logits, temperature=None, uniform=None):
     return out
 
 
-ALL = ("embedding", "rmsnorm", "rmsnorm_act", "gemm", "qk_norm_rope_write", "attention",
+def feed_tokens(ids, source, sampled):
+    take = source >= 0
+    ids[take] = sampled[source[take].long()]
+
+
+ALL = ("feed_tokens", "embedding", "rmsnorm", "rmsnorm_act", "gemm", "qk_norm_rope_write", "attention",
        "swiglu", "sample")
 
 

@@ -46,3 +46,92 @@ def test_step_function_matches_plain(monkeypatch, key, family):
     assert not runner.cache.requests
     for g in runner.cache.groups:
         assert g.pool.num_free() == blocks
+
+
+def host_engine(cfg, weights, page, blocks, **kw):
+    from lucciola_amd.engine.llm_engine import LLMEngine
+    from lucciola_amd.engine.loading import _build
+    from lucciola_amd.weights.loader import DictSource
+    arch = architecture_for(cfg)
+    config = arch.read_config(cfg)
+    model = _build(arch.model_spec(config), DictSource(weights), "float32", "cpu")
+    return LLMEngine(model, config, EngineConfig(dtype="float32", block_size=page,
+                                                 max_blocks=blocks, device="cpu", **kw))
+
+
+@pytest.mark.parametrize("blocks", [200, 11])
+def test_running_ahead_generates_what_waiting_generates(monkeypatch, blocks):
+    """A step queued before the tokens of the one before it are known, fed from the sampler's
+    output: the same tokens as with a wait after every step, with plenty of pages and with so
+    few that requests are preempted while a token of theirs is still under way."""
+    from lucciola_amd.sampling.sampler import SamplingParams
+    reference_ops.install(monkeypatch)
+    cfg, page, seed = configs.ALL["A"]
+    weights = random_weights(cfg, seed, std=0.3)
+    prompts = list(prompts_for(cfg, [9, 14, 6, 11], seed + 40).values())
+    params = [SamplingParams(max_new_tokens=n, temperature=t, seed=i)
+              for i, (n, t) in enumerate([(20, 0.0), (1, 0.0), (17, 0.8), (2, 0.0)])]
+    got = {}
+    for ahead in (False, True):
+        engine = host_engine(cfg, weights, page, blocks, max_tokens_per_step=12, max_seqs=4,
+                             run_ahead=ahead)
+        seen = []
+        got[ahead] = engine.generate(prompts, params, on_token=lambda i, t, f: seen.append((i, t, f)))
+        assert [len(g) for g in got[ahead]] == [20, 1, 17, 2]
+        assert all(t >= 0 for g in got[ahead] for t in g)
+        assert sum(f for _, _, f in seen) == 4 and len(seen) == 40
+        if blocks == 11:
+            assert engine.scheduler.num_preemptions > 0
+        engine.runner.cache.check()
+        assert not engine.runner.cache.requests and not engine.has_unfinished_requests()
+    assert got[True] == got[False]
+    assert got[False][0] == plain_qwen3.greedy(cfg, weights, prompts[0], 20)
+
+
+def test_running_ahead_stops_at_an_end_token_and_drops_the_step_after_it(monkeypatch):
+    from lucciola_amd.sampling.sampler import SamplingParams
+    reference_ops.install(monkeypatch)
+    cfg, page, seed = configs.ALL["B"]
+    weights = random_weights(cfg, seed, std=0.3)
+    prompts = list(prompts_for(cfg, [5, 12, 3], seed + 60).values())
+    free_run = host_engine(cfg, weights, page, 64, max_seqs=4, run_ahead=False).generate(
+        prompts, SamplingParams(max_new_tokens=12))
+    stop = free_run[1][4]               # request 1 meets it at its fifth token at the latest
+    want = []
+    for tokens in free_run:
+        cut = tokens.index(stop) + 1 if stop in tokens else len(tokens)
+        want.append(tokens[:cut])
+    assert len(want[1]) <= 5
+    for ahead in (False, True):
+        engine = host_engine(cfg, weights, page, 64, max_seqs=4, run_ahead=ahead)
+        seen = []
+        got = engine.generate(prompts, SamplingParams(max_new_tokens=12, eos_token_ids=(stop,)),
+                              on_token=lambda i, t, f: seen.append((i, t, f)))
+        assert got == want
+        assert len(seen) == sum(len(w) for w in want) and sum(f for _, _, f in seen) == 3
+        engine.runner.cache.check()
+        assert not engine.runner.cache.requests
+        for g in engine.runner.cache.groups:
+            assert g.pool.num_free() == 64
+
+
+def test_a_pending_token_needs_a_carry(monkeypatch):
+    from lucciola_amd.engine.batch import PENDING, Carry
+    reference_ops.install(monkeypatch)
+    cfg, page, seed = configs.ALL["A"]
+    runner, weights = make(cfg, seed, page, 32)
+    logits = runner.step([StepEntry("a", [3, 4, 5], [2]), StepEntry("b", [7, 8], [1])])
+    sampled = reference_ops.sample(logits)
+    with pytest.raises(ValueError, match="no carry"):
+        runner.step([StepEntry("a", [PENDING], [0])])
+    with pytest.raises(ValueError, match="no row"):
+        runner.step([StepEntry("a", [PENDING], [0])], Carry(sampled, {"b": 1}))
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        runner.step([StepEntry("a", [PENDING, 4], [0])], Carry(sampled, {"a": 0}))
+    # one request fed from the device beside one fed from the host: as both from the host
+    fed = runner.step([StepEntry("b", [int(sampled[1])], [0]), StepEntry("a", [PENDING], [0])],
+                      Carry(sampled, {"a": 0, "b": 1}))
+    ids = {"a": [3, 4, 5, int(sampled[0])], "b": [7, 8, int(sampled[1])]}
+    for row, name in enumerate(["b", "a"]):
+        ref = plain_qwen3.forward(cfg, weights, ids[name])[-1]
+        assert float((fed[row].double() - ref).abs().max() / ref.abs().max()) < 2e-5

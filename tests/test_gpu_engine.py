@@ -282,6 +282,42 @@ def test_graph_replay_matches_eager():
     assert torch.equal(results[True], results[False])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["A", "D"])
+def test_running_ahead_matches_waiting(dtype, key):
+    """The engine queues a step before it has read the tokens of the one before (they reach the
+    next step on the device).  With requests that end at different times, by count and by an
+    end token, with temperature beside greedy, through eager steps (float32) and graph replays
+    (bfloat16): the same tokens as an engine that waits after every step."""
+    cfg, page, seed = configs.ALL[key]
+    weights = random_weights(cfg, seed, std=0.3)
+    prompts = list(prompts_for(cfg, [9, 14, 6, 11, 3], seed + 80).values())
+    counts = [24, 1, 17, 2, 30]
+    got = {}
+    stop = None
+    for ahead in (False, True):
+        engine = engine_for(cfg, weights, page, 256 // page + 8, dtype, max_tokens_per_step=12,
+                            max_seqs=5, run_ahead=ahead)
+        if stop is None:        # an end token that request 4 meets half way
+            stop = engine.generate([prompts[4]], SamplingParams(max_new_tokens=30))[0][14]
+        params = [SamplingParams(max_new_tokens=n, temperature=0.7 if i == 2 else 0.0, seed=i,
+                                 eos_token_ids=(stop,) if i == 4 else ())
+                  for i, n in enumerate(counts)]
+        got[ahead] = engine.generate(prompts, params)
+        assert [len(g) for g in got[ahead]][:4] == counts[:4]
+        last = got[ahead][4]
+        assert stop not in last[:-1] and (last[-1] == stop or len(last) == 30)
+        if dtype == "float32":
+            assert last[-1] == stop and len(last) <= 15
+        engine.runner.cache.check()
+        assert not engine.runner.cache.requests
+        if dtype == "bfloat16":
+            assert engine.runner.graph_replays > 10
+    assert got[True] == got[False]
+    if dtype == "float32":
+        assert got[True][0] == plain_qwen3.greedy(cfg, weights, prompts[0], 24)
+
+
 def test_command_line_and_async_engine(tmp_path):
     """The command line and ``AsyncEngine(model_path, max_blocks, block_size)`` /
     ``generate_async(prompt, max_new_tokens, callback)`` give the plain greedy tokens."""

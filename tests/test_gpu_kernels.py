@@ -598,3 +598,18 @@ def test_norm_sums_the_shares_of_a_product_cut_along_k(M, H, K):
     torch.testing.assert_close(h_got.double(), h_want, rtol=1e-5, atol=1e-5)
     close(got, normed.to(torch.bfloat16), torch.bfloat16)
     close(ops.value(pending), (x.double() @ w.double().T).to(torch.bfloat16), torch.bfloat16, scale=2.0)
+
+
+def test_feed_tokens():
+    gen = torch.Generator().manual_seed(5)
+    ids = torch.randint(0, 1000, (37,), generator=gen, dtype=torch.int32)
+    sampled = torch.randint(0, 1000, (9,), generator=gen, dtype=torch.int32)
+    source = torch.full((37,), -1, dtype=torch.int32)
+    source[[0, 5, 6, 36]] = torch.tensor([3, 8, 3, 0], dtype=torch.int32)
+    want = ids.clone()
+    ref.feed_tokens(want, source, sampled)
+    got = ids.to(DEV)
+    ops.feed_tokens(got, source.to(DEV), sampled.to(DEV))
+    assert torch.equal(got.cpu(), want)
+    with pytest.raises(ops.KernelError):
+        ops.feed_tokens(got, source.to(DEV)[:5], sampled.to(DEV))
