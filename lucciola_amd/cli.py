@@ -51,6 +51,9 @@ def main(argv=None) -> int:
     ap.add_argument("--random-config", help="a config.json to make random weights for")
     ap.add_argument("--write-model", help="with --random-config: the model folder to write")
     ap.add_argument("--device", default="cuda:0")
+    ap.add_argument("--wait-for-tokens", action="store_true",
+                    help="read every step's tokens before the next step is queued (by default the "
+                         "next step is queued first and takes them on the device)")
     args = ap.parse_args(argv)
 
     if args.random_config:
@@ -73,7 +76,7 @@ def main(argv=None) -> int:
     engine = LLMEngine.from_folder(args.model, EngineConfig(
         dtype=args.dtype, block_size=args.block_size, max_blocks=args.max_blocks,
         max_tokens_per_step=args.max_tokens_per_step, max_seqs=args.max_seqs, device=args.device,
-        memory_fraction=args.mem_fraction))
+        memory_fraction=args.mem_fraction, run_ahead=not args.wait_for_tokens))
     print(f"model ready: {len(engine.model.layers)} layers, {engine.runner.cache.num_blocks} pages "
           f"of {args.block_size} tokens", file=sys.stderr, flush=True)
 
