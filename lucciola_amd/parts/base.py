@@ -22,7 +22,7 @@ Interfaces (all tensors on the GPU; "act" is the engine's activation dtype):
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Dict, Optional
+from typing import Any, Dict
 
 import torch
 

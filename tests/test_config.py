@@ -10,7 +10,7 @@ from lucciola_amd.config.engine_config import EngineConfig, parse_dtype
 from lucciola_amd.config.model_config import ConfigError, Qwen3Config, read_config_json
 from lucciola_amd.config.registry import (ARCHITECTURES, MIXERS, Architecture, RegistryError,
                                           architecture_for)
-from lucciola_amd.config.specs import ModelSpec, RunEntry
+from lucciola_amd.config.specs import RunEntry
 
 
 def test_reads_every_key():

@@ -2,7 +2,6 @@
 run with the plain torch versions of the kernels put in their place, and compared with the
 plain whole-sequence implementation.  What these tests cannot see is the kernels themselves
 (the ``gpu`` tests cover those)."""
-import random
 
 import pytest
 import torch
@@ -13,10 +12,6 @@ import reference_ops
 import traces
 from lucciola_amd.config.engine_config import EngineConfig
 from lucciola_amd.engine.batch import StepEntry
-from lucciola_amd.engine.loading import random_model
-from lucciola_amd.engine.runner import ModelRunner
-from lucciola_amd.models.causal_lm import declared_tensors
-from lucciola_amd.weights.random_init import random_tensors
 from lucciola_amd.config.registry import architecture_for
 
 

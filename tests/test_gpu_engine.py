@@ -16,7 +16,7 @@ import traces
 from helpers import compare, make_runner, prompts_for, random_weights, replay
 from lucciola_amd.config.engine_config import EngineConfig
 from lucciola_amd.engine.llm_engine import LLMEngine
-from lucciola_amd.engine.loading import _build, load_model
+from lucciola_amd.engine.loading import _build
 from lucciola_amd.config.registry import architecture_for
 from lucciola_amd.sampling.sampler import SamplingParams, uniform_for
 from lucciola_amd.weights.loader import DictSource

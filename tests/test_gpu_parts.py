@@ -1,7 +1,6 @@
 """Each part of a layer alone against the plain implementation, a run order that names a
 layer twice and lets a site read another site's cache, and a toy architecture with a mixer
 that keeps state of its own: registered, built and stepped from this file alone."""
-import math
 
 import pytest
 import torch
