@@ -677,17 +677,20 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restric
 
 // The tile shapes of the tiled kernel.  TILE_AUTO picks by size; the others are forced through
 // lc_gemm_bf16_force_tile (tests and tuning).
-enum : int { TILE_AUTO = -1, TILE_64x128 = 0, TILE_128x128 = 1, TILE_256x128 = 2, TILE_256x192 = 3, TILE_256x256 = 4, TILE_COUNT = 5 };
+enum : int { TILE_AUTO = -1, TILE_64x128 = 0, TILE_128x128 = 1, TILE_256x128 = 2, TILE_256x192 = 3, TILE_256x256 = 4,
+              TILE_192x128 = 5, TILE_192x256 = 6, TILE_COUNT = 7 };
 static int g_force_tile = TILE_AUTO;
 constexpr int kCUs = 256;
 
-static int tile_bm(int t) { return t == TILE_64x128 ? 64 : t == TILE_128x128 ? 128 : 256; }
-static int tile_bn(int t) { return t == TILE_256x256 ? 256 : t == TILE_256x192 ? 192 : 128; }
+static int tile_bm(int t) {
+    return t == TILE_64x128 ? 64 : t == TILE_128x128 ? 128 : (t == TILE_192x128 || t == TILE_192x256) ? 192 : 256;
+}
+static int tile_bn(int t) { return (t == TILE_256x256 || t == TILE_192x256) ? 256 : t == TILE_256x192 ? 192 : 128; }
 static long long tile_count(int t, int M, int N) {
     return (long long)((M + tile_bm(t) - 1) / tile_bm(t)) * ((N + tile_bn(t) - 1) / tile_bn(t));
 }
 
-// The shapes with 256 rows run one workgroup to a CU, so their tiles go through the CUs in
+// The shapes with 192 or 256 rows run one workgroup to a CU, so their tiles go through the CUs in
 // rounds of kCUs.  When the last round would be less than half full, its tiles are cut along K
 // into `shares` parts each (written tile by tile, summed by tail_reduce_kernel), which fills
 // that round's CUs with shorter pieces: rest tiles, shares parts (0, 1: no such tail).
@@ -696,7 +699,7 @@ struct TailPlan {
 };
 static TailPlan tail_plan(int t, int M, int N, int K) {
     TailPlan none = {0, 1};
-    if (tile_bm(t) != 256) return none;
+    if (tile_bm(t) < 192) return none;
     const long long tiles = tile_count(t, M, N);
     const int rest = (int)(tiles % kCUs), nk = K / TL_K;
     if (tiles < kCUs || rest == 0 || rest > kCUs / 2 || nk < 16) return none;
@@ -707,40 +710,11 @@ static TailPlan tail_plan(int t, int M, int N, int K) {
     return plan;
 }
 
-// The tile for a product with M > 16.  Up to 64 rows: the 64-row tile.  Beyond: the shape with
-// the least estimated time in microseconds.  A CU works through a round of tiles in
-// (tile area) x K x 2 / (4.63 MFLOP/us x the shape's relative rate) (measured at K = 4096: larger
-// tiles move fewer bytes per product); a last round that is cut along K takes its share of
-// that, plus the time to write and read its float32 partial tiles (about 4 TB/s) and to start
-// two more kernels.
-static int pick_tile(int M, int N, int K) {
-    if (g_force_tile != TILE_AUTO) return g_force_tile;
-    if (M <= 64) return TILE_64x128;
-    const double rate[TILE_COUNT] = {0.0, 0.82, 0.90, 0.94, 1.0};
-    int best = TILE_128x128;
-    double best_cost = 0.0;
-    for (int t = TILE_128x128; t < TILE_COUNT; ++t) {
-        const long long tiles = tile_count(t, M, N);
-        const double area = (double)tile_bm(t) * tile_bn(t);
-        const double round_us = area * K * 2.0 / (4.63e6 * rate[t]) + 3.0;
-        const TailPlan tail = tail_plan(t, M, N, K);
-        double cost;
-        if (tail.shares > 1)
-            cost = (double)(tiles / kCUs) * round_us + round_us / tail.shares +
-                   (double)tail.rest * tail.shares * area * 8.0 / 4.0e6 + 10.0;
-        else
-            cost = (double)((tiles + kCUs - 1) / kCUs) * round_us;
-        if (t == TILE_128x128 || cost < best_cost) { best = t; best_cost = cost; }
-    }
-    return best;
-}
-
-// How many shares of K the product of these sizes is cut into (1: no workspace needed): as
-// many as it takes to give every CU a workgroup when whole-K tiles would be too few.  Only the
-// two small tiles are cut as a whole.
-static int splitk_shares(int M, int N, int K) {
-    if (M <= 16) return 1;
-    const int t = pick_tile(M, N, K);
+// Into how many shares of K a product with this tile is cut as a whole (1: not at all): as many
+// as it takes to give every CU about two workgroups when whole-K tiles would be too few.  Only
+// the two small tiles are cut as a whole; the shares are summed by splitk_reduce_kernel, or by
+// whoever takes the partial sums (lc_gemm_bf16_partials).
+static int shares_for(int t, int M, int N, int K) {
     if (t != TILE_64x128 && t != TILE_128x128) return 1;
     const long long tiles = tile_count(t, M, N);
     if (tiles >= 400) return 1;
@@ -748,6 +722,49 @@ static int splitk_shares(int M, int N, int K) {
     int S = (int)((480 + tiles / 2) / tiles);
     if (S > nk / 4) S = nk / 4;
     return S < 1 ? 1 : S;
+}
+
+// The tile for a product with M > 16.  Up to 64 rows: the 64-row tile.  Beyond: the shape with
+// the least estimated time in microseconds.  A CU works through a round of tiles in
+// (tile area) x K x 2 / (4.63 MFLOP/us x the shape's relative rate) (measured at K = 4096: larger
+// tiles move fewer bytes per product) and 3 us to start and end.  A last round of a one-a-CU shape
+// that is cut along K takes its share of that, plus the time to write and read its float32
+// partial tiles (about 4 TB/s) and to start two more kernels.  A small tile cut along K as a
+// whole pays for its partial sums likewise, unless the caller takes them as they are
+// (partials_wanted).
+static int pick_tile(int M, int N, int K, bool partials_wanted = false) {
+    if (g_force_tile != TILE_AUTO) return g_force_tile;
+    if (M <= 64) return TILE_64x128;
+    const double rate[TILE_COUNT] = {0.70, 0.82, 0.90, 0.94, 1.0, 0.87, 0.94};
+    int best = -1;
+    double best_cost = 0.0;
+    for (int t = M <= 128 ? TILE_64x128 : TILE_128x128; t < TILE_COUNT; ++t) {
+        const long long tiles = tile_count(t, M, N);
+        const double area = (double)tile_bm(t) * tile_bn(t);
+        const double work_us = area * K * 2.0 / (4.63e6 * rate[t]);
+        double cost;
+        if (tile_bm(t) >= 192) {
+            const double round_us = work_us + 3.0;
+            const TailPlan tail = tail_plan(t, M, N, K);
+            if (tail.shares > 1)
+                cost = (double)(tiles / kCUs) * round_us + round_us / tail.shares +
+                       (double)tail.rest * tail.shares * area * 8.0 / 4.0e6 + 10.0;
+            else
+                cost = (double)((tiles + kCUs - 1) / kCUs) * round_us;
+        } else {
+            const int S = shares_for(t, M, N, K);
+            cost = (double)((tiles * S + kCUs - 1) / kCUs) * (work_us / S + 3.0);
+            if (S > 1) cost += (double)M * N * S * (partials_wanted ? 4.0 : 8.0) / 4.0e6 + (partials_wanted ? 0.0 : 10.0);
+        }
+        cost += 1e-6 * tiles * area * K / 4.63e6;      // equal otherwise: the shape that covers less beyond M x N
+        if (best < 0 || cost < best_cost) { best = t; best_cost = cost; }
+    }
+    return best;
+}
+
+static int splitk_shares(int M, int N, int K, bool partials_wanted = false) {
+    if (M <= 16) return 1;
+    return shares_for(pick_tile(M, N, K, partials_wanted), M, N, K);
 }
 
 // float32 words of workspace that the product needs (0: none)
@@ -824,7 +841,7 @@ static int launch_tiled(const bf16* x, const bf16* w, TO* out, float* workspace,
         return 0;
     }
     LC_CHECK(workspace, "gemm_bf16: M=%d N=%d K=%d needs a workspace", M, N, K);
-    if constexpr (BM == 256) {
+    if constexpr (BM >= 192) {
         LC_CHECK(shares == 1 && tail.rest > 0 && tail.rest < tiles, "gemm_bf16: bad tail for tile %dx%d", BM, BN);
         const int whole = tiles - tail.rest;
         gemm_tiled_kernel<BM, BN, STAGES, EPI, false, TO><<<whole, 256, 0, s>>>(
@@ -865,6 +882,8 @@ static int launch_bf16(const bf16* x, const bf16* w, TO* out, float* workspace, 
     case TILE_128x128: return launch_tiled<128, 128, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     case TILE_256x128: return launch_tiled<256, 128, 3, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     case TILE_256x192: return launch_tiled<256, 192, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
+    case TILE_192x128: return launch_tiled<192, 128, 3, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
+    case TILE_192x256: return launch_tiled<192, 256, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     default:           return launch_tiled<256, 256, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     }
 }
@@ -1007,7 +1026,7 @@ LC_API int lc_gemm_bf16_scaled_rows(const void* x, const void* w, void* out, int
 // Number of shares that lc_gemm_bf16_partials writes for these sizes (0: this product is not cut).
 LC_API int lc_gemm_bf16_shares(int M, int N, int K) {
     if (!lc_gemm_bf16_supported(M, N, K) || M <= 16) return 0;
-    const int shares = splitk_shares(M, N, K);
+    const int shares = splitk_shares(M, N, K, true);
     return shares > 1 ? shares : 0;
 }
 
@@ -1021,7 +1040,7 @@ LC_API int lc_gemm_bf16_partials(const void* x, const void* w, float* partials, 
              "gemm_bf16_partials: operands must be 16-byte aligned");
     const bf16* xb = (const bf16*)x;
     const bf16* wb = (const bf16*)w;
-    if (pick_tile(M, N, K) == TILE_64x128) {
+    if (pick_tile(M, N, K, true) == TILE_64x128) {
         const int tiles_m = (M + 63) / 64, tiles = tiles_m * ((N + 127) / 128);
         gemm_tiled_kernel<64, 128, 3, 0, true, float><<<dim3(tiles, shares), 256, 0, stream>>>(
             xb, wb, nullptr, partials, M, N, K, tiles_m, 0, tiles, 0);

@@ -246,7 +246,7 @@ def test_gemm_bf16_matrix_cores(out_dtype, M, N, K):
     close(got, want, out_dtype, scale=K ** 0.5)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("M,N,K", [(1, 16, 128), (70, 130, 128), (257, 300, 256), (300, 1000, 640),
                                    (513, 257, 384), (64, 128, 1024), (1000, 520, 2048), (100, 400, 128)])
 def test_gemm_bf16_every_tile_shape(tile, M, N, K):
@@ -273,7 +273,7 @@ def test_gemm_bf16_every_tile_shape(tile, M, N, K):
 
 
 @pytest.mark.parametrize("tile,M,N,K", [(4, 2000, 10200, 1024), (2, 2048, 10240, 1024), (3, 1990, 6520, 2048),
-                                        (-1, 2048, 10240, 5120)])
+                                        (-1, 2048, 10240, 5120), (6, 570, 24500, 1024), (5, 760, 12000, 1024)])
 def test_gemm_bf16_last_round_cut_along_k(tile, M, N, K):
     """Sizes whose tiles fill the CUs once or twice and leave a small rest: the rest's tiles
     are cut along K and summed by a second kernel.  Plain and with the SwiGLU epilogue,
