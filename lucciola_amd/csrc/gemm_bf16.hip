@@ -100,7 +100,7 @@ template <int MT, int NT, int WAVES, int UNROLL, int EPI, bool SCALE, int XR, ty
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __restrict__ x,
                                                                  const bf16* __restrict__ w,
                                                                  TO* __restrict__ out, int M, int N,
-                                                                 int K, SkinnyFuse fuse) {
+                                                                 int K, int rows, SkinnyFuse fuse) {
     static_assert(WAVES == 16, "the epilogues lay 1024 threads over a workgroup's results");
     static_assert(MT == 1, "up to 16 rows of x");
     static_assert(!(SCALE && EPI == 2), "both would use the same words of LDS");
@@ -112,7 +112,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
     __shared__ float pieces[WAVES][16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, g = lane >> 4;
-    const int tiles = (N + 16 * NT - 1) / (16 * NT);
+    // a work item ("tile" below) is `rows` <= 16 NT rows of w; with fewer than 16 NT the last of
+    // its blocks of 16 is partly idle, which costs nothing here (the kernel waits for memory) and
+    // lets the host cut N into as many equal items as fill the CUs evenly
+    const int tiles = (N + rows - 1) / rows;
     const int kblocks = K / SK_KBLOCK;
 
     // loads whose values are wanted only after the products; issued first, they are back
@@ -169,7 +172,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
     bool first = true;
     // one tile: its rows of w are in a_use (XR > 0 with AHEAD) or loaded here; a_fill takes the next tile's
     auto one_tile = [&](const int tile, bf16x8 (&a_use)[XR > 0 ? XR : 1][4], bf16x8 (&a_fill)[XR > 0 ? XR : 1][4]) {
-        const int n0 = tile * (16 * NT);
+        const int n0 = tile * rows, n_end = min(N, n0 + rows);
         // The epilogue's layout: wave q and lane (row m = lane % 16, quarter = lane / 16) add up,
         // over the waves 4 quarter .. 4 quarter + 3, the sums for row m and column
         // n0 + 16 nt + 4 (q % 4) + q / 4; the quarters then meet by two lane exchanges, and the
@@ -179,7 +182,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
         if (EPI == 2) {
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                const bool mine = g == 0 && r < M && e_n + nt * 16 < N;
+                const bool mine = g == 0 && r < M && e_n + nt * 16 < n_end;
                 e_resid[nt] = mine ? fuse.resid[(size_t)r * N + e_n + nt * 16] : 0.f;
                 e_w[nt] = mine ? fuse.next_w[e_n + nt * 16] : 0.f;
             }
@@ -187,7 +190,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 
         const bf16* wp[NT];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) wp[nt] = w + (size_t)min(n0 + nt * 16 + r, N - 1) * K + g * 8;
+        for (int nt = 0; nt < NT; ++nt) wp[nt] = w + (size_t)min(n0 + nt * 16 + r, n_end - 1) * K + g * 8;
 
         floatx4 acc[NT][MT];
 #pragma unroll
@@ -199,8 +202,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
             if (!AHEAD) load_w_blocks<XR, WAVES>(a_use, wp[0], wave, kblocks);
             if (AHEAD && tile + gridDim.x < tiles) {
                 // the next tile's rows of w are on their way while this tile's sums meet in LDS
-                const int n_next = (tile + gridDim.x) * 16;
-                load_w_blocks<XR, WAVES>(a_fill, w + (size_t)min(n_next + r, N - 1) * K + g * 8, wave, kblocks);
+                const int n_next = (tile + gridDim.x) * rows;
+                load_w_blocks<XR, WAVES>(a_fill, w + (size_t)min(n_next + r, min(N, n_next + rows) - 1) * K + g * 8, wave, kblocks);
             }
 #pragma unroll
             for (int i = 0; i < XR; ++i) {
@@ -255,7 +258,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const float t = total_of(nt, e_mine);
-                if (g == 0 && r < M && e_n + nt * 16 < N) {
+                if (g == 0 && r < M && e_n + nt * 16 < n_end) {
                     const float v = e_resid[nt] + t;
                     fuse.resid[(size_t)r * N + e_n + nt * 16] = v;
                     fuse.next_x[(size_t)r * N + e_n + nt * 16] = static_cast<bf16>(v * e_w[nt]);
@@ -278,7 +281,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
                 for (int nt = 0; nt < NT; ++nt) {
                     const float t = total_of(nt, e_mine);
                     const int n = e_n + nt * 16;
-                    if (g == 0 && r < M && n < N) store_out<TO>(out + (size_t)r * N + n, t * factor);
+                    if (g == 0 && r < M && n < n_end) store_out<TO>(out + (size_t)r * N + n, t * factor);
                 }
             } else {
                 // rows of w come in blocks of 16: 8 gate rows, then their 8 up rows; out has N / 2
@@ -290,7 +293,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
                         const float gate = total_of(nt, e_mine), up = total_of(nt, e_mine + 32);
                         const int n = e_n + nt * 16;
                         const int col = (n >> 4) * 8 + (n & 7);
-                        if (g == 0 && r < M && n < N)
+                        if (g == 0 && r < M && n < n_end)
                             store_out<TO>(out + (size_t)r * (N / 2) + col, swiglu_f(gate * factor, up * factor));
                     }
                 }
@@ -302,7 +305,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
         // two sets of registers take turns, so that no value has to be moved (a move would
         // wait for the loads that are meant to stay in flight)
         int tile = blockIdx.x;
-        if (tile < tiles) load_w_blocks<XR, WAVES>(a_now, w + (size_t)min(tile * 16 + r, N - 1) * K + g * 8, wave, kblocks);
+        if (tile < tiles)
+            load_w_blocks<XR, WAVES>(a_now, w + (size_t)min(tile * rows + r, min(N, (tile + 1) * rows) - 1) * K + g * 8, wave, kblocks);
         while (tile < tiles) {
             one_tile(tile, a_now, a_next);
             tile += gridDim.x;
@@ -779,10 +783,10 @@ static long long workspace_words(int M, int N, int K) {
 }
 
 template <int MT, int NT, int WAVES, int UNROLL, int EPI, bool SCALE, int XR, typename TO>
-static void launch_skinny(const bf16* x, const bf16* w, TO* out, int M, int N, int K, SkinnyFuse fuse,
-                          int workgroups, hipStream_t s) {
+static void launch_skinny(const bf16* x, const bf16* w, TO* out, int M, int N, int K, int rows,
+                          SkinnyFuse fuse, int workgroups, hipStream_t s) {
     gemm_skinny_kernel<MT, NT, WAVES, UNROLL, EPI, SCALE, XR, TO><<<workgroups, WAVES * 64, 0, s>>>(
-        x, w, out, M, N, K, fuse);
+        x, w, out, M, N, K, rows, fuse);
 }
 
 // The skinny kernel's shape for M <= 16 rows.  Measured: with one or two rows of x a deeper
@@ -804,28 +808,55 @@ static int skinny_shape(int M, int N, int K) {
     if (M >= 12 && N >= 32 * 2 * kCUs) return SKINNY_WIDE;
     return SKINNY_PLAIN;
 }
-// number of tiles, which is also the number of pieces that epilogue 2 writes
-static int skinny_tiles(int M, int N, int K) {
-    const int rows = skinny_shape(M, N, K) == SKINNY_WIDE ? 32 : 16;
-    return (N + rows - 1) / rows;
+// How a product of up to 16 rows is laid over the GPU: the kernel's shape, the rows of w of a
+// work item, the number of items (also the number of pieces that epilogue 2 writes) and the
+// number of workgroups.  A workgroup streams its rows of w at the pace of memory, so what
+// counts is that every CU gets the same number of rows.  Items of 16 (or 32) rows do that when
+// their number is a multiple of the CUs or many times it; at 320 items for 256 CUs a quarter of
+// the CUs would work twice as long as the rest.  Then N is cut into items of fewer rows, as
+// many as give every CU the same number (the SwiGLU epilogue needs whole blocks of 16 rows and
+// keeps them).
+struct SkinnyPlan {
+    int shape, rows, items, groups;
+};
+static int g_even_rows = 1;
+static SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
+    SkinnyPlan p;
+    p.shape = skinny_shape(M, N, K);
+    p.rows = p.shape == SKINNY_WIDE ? 32 : 16;
+    p.items = (N + p.rows - 1) / p.rows;
+    const bool keep = p.shape == SKINNY_KEEP_X;
+    if (g_even_rows && g_force_skinny < 0 && epilogue != 1 && p.items > kCUs && p.items % kCUs != 0) {
+        const int per_cu = (p.items + kCUs - 1) / kCUs;            // items of the busiest CU as it is
+        if (keep && per_cu <= 4) {
+            p.rows = (N + kCUs * per_cu - 1) / (kCUs * per_cu);    // x stays in registers: small items cost nothing
+        } else if (!keep && p.shape != SKINNY_WIDE && per_cu == 2 && M > 2) {
+            p.shape = SKINNY_WIDE;                                 // one item a CU, of up to 32 rows: x is fetched once a CU
+            p.rows = (N + kCUs - 1) / kCUs;
+        } else if (!keep && p.shape != SKINNY_WIDE && per_cu <= 4) {
+            p.rows = (N + kCUs * per_cu - 1) / (kCUs * per_cu);
+        }
+        p.items = (N + p.rows - 1) / p.rows;
+    }
+    p.groups = keep ? (p.items < kCUs ? p.items : kCUs) : p.items;   // keep-x: one workgroup a CU fits
+    return p;
 }
+static int skinny_tiles(int M, int N, int K, int epilogue) { return skinny_plan(M, N, K, epilogue).items; }
 
 template <int EPI, bool SCALE, typename TO>
 static void launch_skinny_any(const bf16* x, const bf16* w, TO* out, int M, int N, int K, SkinnyFuse fuse,
                               hipStream_t s) {
-    const int tiles = skinny_tiles(M, N, K);
-    switch (skinny_shape(M, N, K)) {
-    case SKINNY_DEEP: launch_skinny<1, 1, 16, 4, EPI, SCALE, 0, TO>(x, w, out, M, N, K, fuse, tiles, s); break;
-    case SKINNY_WIDE: launch_skinny<1, 2, 16, 2, EPI, SCALE, 0, TO>(x, w, out, M, N, K, fuse, tiles, s); break;
-    case SKINNY_KEEP_X: {
-        const int groups = tiles < kCUs ? tiles : kCUs, per_wave = (K / SK_KBLOCK + 15) / 16;   // one a CU fits
-
-        if (per_wave == 1) launch_skinny<1, 1, 16, 1, EPI, SCALE, 1, TO>(x, w, out, M, N, K, fuse, groups, s);
-        else if (per_wave == 2) launch_skinny<1, 1, 16, 1, EPI, SCALE, 2, TO>(x, w, out, M, N, K, fuse, groups, s);
-        else launch_skinny<1, 1, 16, 1, EPI, SCALE, 3, TO>(x, w, out, M, N, K, fuse, groups, s);
+    const SkinnyPlan p = skinny_plan(M, N, K, EPI);
+    const int per_wave = (K / SK_KBLOCK + 15) / 16;
+    switch (p.shape) {
+    case SKINNY_DEEP: launch_skinny<1, 1, 16, 4, EPI, SCALE, 0, TO>(x, w, out, M, N, K, p.rows, fuse, p.groups, s); break;
+    case SKINNY_WIDE: launch_skinny<1, 2, 16, 2, EPI, SCALE, 0, TO>(x, w, out, M, N, K, p.rows, fuse, p.groups, s); break;
+    case SKINNY_KEEP_X:
+        if (per_wave == 1) launch_skinny<1, 1, 16, 1, EPI, SCALE, 1, TO>(x, w, out, M, N, K, p.rows, fuse, p.groups, s);
+        else if (per_wave == 2) launch_skinny<1, 1, 16, 1, EPI, SCALE, 2, TO>(x, w, out, M, N, K, p.rows, fuse, p.groups, s);
+        else launch_skinny<1, 1, 16, 1, EPI, SCALE, 3, TO>(x, w, out, M, N, K, p.rows, fuse, p.groups, s);
         break;
-    }
-    default:          launch_skinny<1, 1, 16, 2, EPI, SCALE, 0, TO>(x, w, out, M, N, K, fuse, tiles, s); break;
+    default:          launch_skinny<1, 1, 16, 2, EPI, SCALE, 0, TO>(x, w, out, M, N, K, p.rows, fuse, p.groups, s); break;
     }
 }
 
@@ -954,6 +985,13 @@ LC_API int lc_gemm_bf16(const void* x, const void* w, void* out, int out_dt, int
 // missing is each row's factor rsqrt(mean(h^2) + eps), which a product can apply to its sums.
 // The pieces of row m lie at [piece][m] with lc_gemm_bf16_piece_stride(M) floats per piece.
 
+// 0: work items of 16 or 32 rows whatever N is; 1 (the default): N cut into equal items where
+// that gives every CU the same number of rows.  For tests and tuning.
+LC_API int lc_gemm_bf16_even_rows(int on) {
+    g_even_rows = on ? 1 : 0;
+    return 0;
+}
+
 LC_API int lc_gemm_bf16_piece_stride(int M) {
     int stride = 1;
     while (stride < M) stride *= 2;
@@ -965,7 +1003,7 @@ LC_API int lc_gemm_bf16_piece_stride(int M) {
 // pieces than a scaled product reads).
 LC_API int lc_gemm_bf16_residual_pieces(int M, int N, int K) {
     if (!lc_gemm_bf16_supported(M, N, K) || M > 16 || g_force_tile != TILE_AUTO) return 0;
-    const int pieces = skinny_tiles(M, N, K);
+    const int pieces = skinny_tiles(M, N, K, 2);
     return pieces <= SK_MAX_PIECES ? pieces : 0;
 }
 

@@ -30,6 +30,7 @@ _SIGNATURES = {
     "lc_gemm_bf16_supported": "iii",
     "lc_gemm_bf16_force_tile": "i",
     "lc_gemm_bf16_force_skinny": "i",
+    "lc_gemm_bf16_even_rows": "i",
     "lc_gemm_bf16_residual_pieces": "iii",
     "lc_gemm_bf16_piece_stride": "i",
     "lc_gemm_bf16_shares": "iii",
@@ -346,6 +347,12 @@ def force_gemm_tile(tile: int) -> None:
     """Make the tiled bfloat16 product use one tile shape for every size (0: 64x128, 1: 128x128,
     2: 256x128, 3: 256x192, 4: 256x256, 5: 192x128, 6: 192x256; -1: choose by size again).  For tests and tuning."""
     _call("lc_gemm_bf16_force_tile", _c_int(tile))
+
+
+def gemm_even_rows(on: bool) -> None:
+    """Whether the bfloat16 product of up to 16 rows may cut N into work items of fewer than 16
+    rows so that every CU gets the same number (on by default).  For tests and tuning."""
+    _call("lc_gemm_bf16_even_rows", _c_int(1 if on else 0))
 
 
 def force_gemm_skinny(shape: int) -> None:

@@ -296,7 +296,8 @@ def test_gemm_bf16_last_round_cut_along_k(tile, M, N, K):
     close(fused, (g / (1 + torch.exp(-g)) * u).to(torch.bfloat16), torch.bfloat16, scale=K ** 0.5)
 
 
-@pytest.mark.parametrize("M,H,K,N2", [(1, 128, 128, 48), (2, 384, 256, 1000), (5, 256, 640, 272), (8, 4096, 512, 2064),
+@pytest.mark.parametrize("M,H,K,N2", [(1, 5120, 128, 6160), (8, 5120, 256, 10250), (16, 6272, 384, 5130),
+                                      (1, 128, 128, 48), (2, 384, 256, 1000), (5, 256, 640, 272), (8, 4096, 512, 2064),
                                       (11, 640, 128, 16), (12, 16384, 6272, 16416), (12, 8192, 128, 48), (16, 1152, 384, 130)])
 def test_norm_folded_into_the_products_around_it(M, H, K, N2):
     """Up to 16 rows: the product before a norm adds its result to the stream and leaves
@@ -552,6 +553,20 @@ def test_gemm_bf16_few_rows_every_shape(M, N, K, shape):
         few_rows_case(M, N, K)
     finally:
         ops.force_gemm_skinny(-1)
+
+
+@pytest.mark.parametrize("even", [True, False])
+@pytest.mark.parametrize("M,N,K", [(1, 5120, 256), (2, 6150, 384), (8, 5120, 8192), (16, 5136, 128), (5, 6150, 4096),
+                                   (9, 10250, 5120), (3, 4100, 128), (12, 7170, 6272), (8, 16001, 256)])
+def test_gemm_bf16_few_rows_cut_evenly(M, N, K, even):
+    """Numbers of columns that items of 16 rows of w would spread unevenly over the CUs (one and
+    a quarter a CU, one and a half, two and a half): N is cut into equal items of fewer rows, whose
+    last block of 16 is partly idle; with and without that, every epilogue."""
+    ops.gemm_even_rows(even)
+    try:
+        few_rows_case(M, N, K)
+    finally:
+        ops.gemm_even_rows(True)
 
 
 def few_rows_case(M, N, K):
