@@ -34,6 +34,7 @@ class AsyncEngine:
         self._pending: List[Tuple[int, List[int], SamplingParams]] = []
         self._callbacks: Dict[int, Callable[[int, bool], None]] = {}
         self._engine_ids: Dict[int, int] = {}
+        self._aborts: List[int] = []
         self._next_req_id = 1
         self._error: Optional[BaseException] = None
         self._thread = threading.Thread(target=self._engine_loop, name="lucciola-engine", daemon=True)
@@ -54,6 +55,13 @@ class AsyncEngine:
             self._pending.append((req_id, [int(t) for t in prompt], params))
             self._cv.notify()
         return req_id
+
+    def abort(self, req_id: int) -> None:
+        """End a request: the engine thread frees what it holds and calls its callback once
+        more with ``(-1, True)``.  (The reference has no way to end a request early.)"""
+        with self._cv:
+            self._aborts.append(req_id)
+            self._cv.notify()
 
     def stop(self) -> None:
         with self._cv:
@@ -77,11 +85,13 @@ class AsyncEngine:
         try:
             while True:
                 with self._cv:
-                    while not self._stop and not self._pending and not eng.has_unfinished_requests():
+                    while not self._stop and not self._pending and not self._aborts \
+                            and not eng.has_unfinished_requests():
                         self._cv.wait()
                     if self._stop:
                         return
                     pending, self._pending = self._pending, []
+                    aborts, self._aborts = self._aborts, []
                 for req_id, prompt, params in pending:
                     try:
                         engine_id = eng.add_request(prompt, params)
@@ -93,6 +103,17 @@ class AsyncEngine:
                         continue
                     with self._mu:
                         self._engine_ids[engine_id] = req_id
+                for req_id in aborts:
+                    with self._mu:
+                        engine_id = next((e for e, r in self._engine_ids.items() if r == req_id), None)
+                        cb = self._callbacks.pop(req_id, None) if engine_id is not None else None
+                        if engine_id is not None:
+                            del self._engine_ids[engine_id]
+                    if engine_id is not None:
+                        eng.abort_request(engine_id)
+                        eng.sequences.pop(engine_id, None)
+                        if cb:
+                            cb(-1, True)
                 for out in eng.step():
                     with self._mu:
                         req_id = self._engine_ids.get(out.seq_id)

@@ -81,6 +81,18 @@ class LLMEngine:
         self.sequences[seq.seq_id] = seq
         return seq.seq_id
 
+    def abort_request(self, seq_id: int) -> bool:
+        """End a request now, wherever it is (waiting, partly fed, running, with a token under
+        way): its pages and its slot go back, tokens that the host has not read yet are
+        dropped.  Returns False if there is no such live request."""
+        seq = self.sequences.get(seq_id)
+        if seq is None or seq.is_finished():
+            return False
+        while seq.get_len() > seq.get_prompt_len() and seq.token_ids[-1] == PENDING:
+            seq.token_ids.pop()        # `_collect` skips a place beyond the request's end
+        self.scheduler.free_sequence(seq)
+        return True
+
     def has_unfinished_requests(self) -> bool:
         return self._queued is not None or self.scheduler.has_unfinished_requests()
 

@@ -130,3 +130,47 @@ def test_a_pending_token_needs_a_carry(monkeypatch):
     for row, name in enumerate(["b", "a"]):
         ref = plain_qwen3.forward(cfg, weights, ids[name])[-1]
         assert float((fed[row].double() - ref).abs().max() / ref.abs().max()) < 2e-5
+
+
+@pytest.mark.parametrize("ahead", [False, True])
+def test_a_request_is_ended_early_and_gives_everything_back(monkeypatch, ahead):
+    """Requests ended from outside while waiting, while their prompt is partly fed, and while
+    running with a token under way: what they hold goes back at once, the others generate
+    what they generate alone, and no token of an ended request comes out afterwards."""
+    from lucciola_amd.sampling.sampler import SamplingParams
+    reference_ops.install(monkeypatch)
+    cfg, page, seed = configs.ALL["A"]
+    weights = random_weights(cfg, seed, std=0.3)
+    prompts = list(prompts_for(cfg, [9, 30, 6, 11], seed + 90).values())
+    engine = host_engine(cfg, weights, page, 40, max_tokens_per_step=12, max_seqs=3, run_ahead=ahead)
+    ids = [engine.add_request(p, SamplingParams(max_new_tokens=16)) for p in prompts]
+    seen = {i: [] for i in ids}
+    ended = set()
+    steps = 0
+    while engine.has_unfinished_requests():
+        for out in engine.step():
+            assert out.seq_id not in ended
+            seen[out.seq_id].append(out.token)
+        steps += 1
+        if steps == 1:
+            assert engine.abort_request(ids[3])                 # still waiting (max_seqs is 3)
+            ended.add(ids[3])
+        if steps == 2:
+            assert 0 < engine.sequences[ids[1]].prefill_offset < 30
+            assert engine.abort_request(ids[1])                 # its prompt is partly fed
+            ended.add(ids[1])
+        if steps == 6:
+            assert engine.abort_request(ids[2])                 # running, a token may be under way
+            ended.add(ids[2])
+            assert not engine.abort_request(ids[2])
+            engine.runner.cache.check()
+            assert set(engine.runner.cache.requests) == {ids[0]}
+    assert seen[ids[0]] == plain_qwen3.greedy(cfg, weights, prompts[0], 16)
+    assert 0 < len(seen[ids[2]]) < 16 and seen[ids[1]] == [] and seen[ids[3]] == []
+    assert seen[ids[2]] == plain_qwen3.greedy(cfg, weights, prompts[2], 16)[:len(seen[ids[2]])]
+    assert all(t >= 0 for t in engine.sequences[ids[2]].token_ids)
+    engine.runner.cache.check()
+    assert not engine.runner.cache.requests
+    for g in engine.runner.cache.groups:
+        assert g.pool.num_free() == 40
+    assert not engine.abort_request(12345)

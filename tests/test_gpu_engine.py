@@ -354,13 +354,27 @@ def test_command_line_and_async_engine(tmp_path):
             if finished:
                 done[i].set()
         return cb
+    long_one, over = [], threading.Event()
+
+    def until_three(token, finished):       # ends its own request after three tokens
+        long_one.append((token, finished))
+        if len(long_one) == 3:
+            engine.abort(long_id[0])
+        if finished:
+            over.set()
+    long_id = [None]
     try:
         for i, p in enumerate(prompts):
             engine.generate_async(p, 6, callback(i))
         assert all(d.wait(120) for d in done)
+        long_id[0] = engine.generate_async(prompts[0], 150, until_three)
+        assert over.wait(120)
     finally:
         engine.stop()
     assert [got[0], got[1]] == want
+    assert long_one[-1] == (-1, True) and 3 <= len(long_one) < 20
+    assert [t for t, _ in long_one[:3]] == want[0][:3]
+    assert not engine.engine.runner.cache.requests
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
