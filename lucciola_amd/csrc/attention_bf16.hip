@@ -324,20 +324,17 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     }
 }
 
-// Joins the shares of a request's pages: out = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).
-// The factors are worked out once (one thread per share) and left in LDS, so that the sum over
-// the shares is a run of independent loads.
+// Joins the shares of a row's keys: out = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m), the
+// shares of (row, head) lying at part_o[base + s][D] and part_ml[base + s][2].  The factors are
+// worked out once (one thread per share) and left in LDS, so that the sum over the shares is a
+// run of independent loads.  128 threads; at most 64 shares.
 template <int D>
-__global__ __launch_bounds__(128) void attn_decode_join_kernel(const float* __restrict__ part_o,
-                                                               const float* __restrict__ part_ml,
-                                                               const int* __restrict__ decode_tokens,
-                                                               bf16* __restrict__ out, int nh,
-                                                               int splits) {
+__device__ __forceinline__ void join_shares(const float* __restrict__ part_o,
+                                            const float* __restrict__ part_ml, size_t base,
+                                            int splits, bf16* __restrict__ out_row) {
     __shared__ float f[64];
     __shared__ float inv_l;
-    const int di = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
-    const int t = decode_tokens[di];
-    const size_t base = ((size_t)di * nh + h) * splits;
+    const int tid = threadIdx.x;
     if (tid < 64) {
         const float ms = tid < splits ? part_ml[(base + tid) * 2] : -INFINITY;
         const float ls = tid < splits ? part_ml[(base + tid) * 2 + 1] : 0.f;
@@ -352,8 +349,33 @@ __global__ __launch_bounds__(128) void attn_decode_join_kernel(const float* __re
         float o = 0.f;
 #pragma unroll 8
         for (int s = 0; s < splits; ++s) o += f[s] * part_o[(base + s) * D + dim];
-        out[((size_t)t * nh + h) * D + dim] = static_cast<bf16>(o * inv_l);
+        out_row[dim] = static_cast<bf16>(o * inv_l);
     }
+}
+
+template <int D>
+__global__ __launch_bounds__(128) void attn_decode_join_kernel(const float* __restrict__ part_o,
+                                                               const float* __restrict__ part_ml,
+                                                               const int* __restrict__ decode_tokens,
+                                                               bf16* __restrict__ out, int nh,
+                                                               int splits) {
+    const int di = blockIdx.x, h = blockIdx.y;
+    const int t = decode_tokens[di];
+    join_shares<D>(part_o, part_ml, ((size_t)di * nh + h) * splits, splits, out + ((size_t)t * nh + h) * D);
+}
+
+// The same for the rows of prefill tiles, whose shares lie at the rows' places in the batch.
+template <int D>
+__global__ __launch_bounds__(128) void attn_prefill_join_kernel(const float* __restrict__ part_o,
+                                                                const float* __restrict__ part_ml,
+                                                                const int* __restrict__ tiles,
+                                                                bf16* __restrict__ out, int nh,
+                                                                int splits) {
+    const int* tile = tiles + (size_t)(blockIdx.x >> 6) * 4;
+    const int r = blockIdx.x & 63, h = blockIdx.y;
+    if (r >= tile[2]) return;
+    const int t = tile[1] + r;
+    join_shares<D>(part_o, part_ml, ((size_t)t * nh + h) * splits, splits, out + ((size_t)t * nh + h) * D);
 }
 
 // ------------------------------------------------------------------------------- prefill
@@ -377,7 +399,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     const bf16* __restrict__ qkv, int q_stride, const bf16* __restrict__ k_cache,
     const bf16* __restrict__ v_cache, bf16* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ block_table, int max_blocks, int nh, int nkv, float scale_log2,
-    int window, DecodePrologue pro) {
+    int window, DecodePrologue pro, int splits, float* __restrict__ part_o,
+    float* __restrict__ part_ml) {
     constexpr int QT = HPW, NP = PF_NP;
     constexpr int KLD = D + 8;
     constexpr int KPAGE = PAGE * KLD, VPAGE = D * PAGE;   // elements of a page in LDS
@@ -396,7 +419,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     const int total = gridDim.x * gridDim.y, number = blockIdx.y * gridDim.x + blockIdx.x;
     const int half = (total + 1) / 2;
     const int task = (total <= 2 * 256 && number >= half) ? total - 1 - (number - half) : number;
-    const int tile_index = task / gridDim.y, heads_index = task - tile_index * gridDim.y;
+    // with few tiles and many keys, a tile's pages are cut into `splits` shares (x counts tile
+    // and share), each a workgroup of its own whose sums a second kernel joins
+    const int tile_share = task / gridDim.y, heads_index = task - tile_share * gridDim.y;
+    const int tile_index = tile_share / splits, split = tile_share - tile_index * splits;
     const int* tile = tiles + (size_t)tile_index * 4;
     const int req = tile[0], row0 = tile[1], rows = tile[2], pos0 = tile[3];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -469,7 +495,12 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     }
     // pages the workgroup walks, and the part of them this wave needs
     const int t_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
-    const int first = t_lo / PAGE, last = (pos0 + rows - 1) / PAGE;
+    int first = t_lo / PAGE, last = (pos0 + rows - 1) / PAGE;
+    if (splits > 1) {       // this workgroup's share of them, in whole groups of pages
+        const int per = ((last - first + splits) / splits + NP - 1) / NP * NP;
+        first += split * per;
+        last = min(last, first + per - 1);
+    }
     const int w_min = pos0 + min(wrow, rows - 1), w_max = pos0 + min(wrow + 16 * QT - 1, rows - 1);
     const int w_lo = (window > 0 && w_min - window + 1 > 0) ? w_min - window + 1 : 0;
     const int w_first = w_lo / PAGE, w_last = w_max / PAGE;
@@ -608,6 +639,23 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
                     st.o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[c][n / 2], st.o[c][t], 0, 0, 0);
             }
     }
+    if (splits > 1) {       // sums as they are, with their reference point in the units of the exponent
+#pragma unroll
+        for (int c = 0; c < QT; ++c) {
+            float l = st.l[c];
+            l = column_sum(l);
+            if (!valid[c]) continue;
+            const size_t slot = ((size_t)(row0 + wrow + c * 16 + q) * nh + h) * splits + split;
+            float* po = part_o + slot * D + kg * 4;
+#pragma unroll
+            for (int tt = 0; tt < D / 16; ++tt) *reinterpret_cast<floatx4*>(po + tt * 16) = st.o[c][tt];
+            if (kg == 0) {
+                part_ml[slot * 2] = st.m[c] == -INFINITY ? -INFINITY : st.m[c] * scale_log2;
+                part_ml[slot * 2 + 1] = l;
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int c = 0; c < QT; ++c) {
         float l = st.l[c];
@@ -644,19 +692,31 @@ static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* 
     return 0;
 }
 
+// pairs of heads share the keys and values they read; with so few tiles that half of the CUs
+// would get nothing to do, single heads and twice the workgroups are faster (measured)
+// (where the keys are shared out, the shares fill the CUs, and pairs stay)
+static bool prefill_head_pairs(int NT, int nh, int nkv, int splits) {
+    return (nh / nkv) % 2 == 0 && ((long long)NT * (nh / 2) > 128 || splits > 1);
+}
+
 template <int D>
 static int launch_prefill(const bf16* qkv, int q_stride, const bf16* k, const bf16* v, bf16* out,
                           const int* tiles, const int* table, int max_blocks, int NT, int nh,
-                          int nkv, float scale_log2, int window, DecodePrologue pro, hipStream_t s) {
-    // pairs of heads share the keys and values they read; with so few tiles that half of the CUs
-    // would get nothing to do, single heads and twice the workgroups are faster (measured)
-    if ((nh / nkv) % 2 == 0 && (long long)NT * (nh / 2) > 128)
-        attn_prefill_kernel<D, 2><<<dim3(NT, nh / 2), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
-                                                                   max_blocks, nh, nkv, scale_log2, window, pro);
+                          int nkv, float scale_log2, int window, DecodePrologue pro, int splits,
+                          float* part_o, float* part_ml, hipStream_t s) {
+    if (prefill_head_pairs(NT, nh, nkv, splits))
+        attn_prefill_kernel<D, 2><<<dim3(NT * splits, nh / 2), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
+                                                                            max_blocks, nh, nkv, scale_log2, window, pro,
+                                                                            splits, part_o, part_ml);
     else
-        attn_prefill_kernel<D, 1><<<dim3(NT, nh), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
-                                                               max_blocks, nh, nkv, scale_log2, window, pro);
+        attn_prefill_kernel<D, 1><<<dim3(NT * splits, nh), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
+                                                                        max_blocks, nh, nkv, scale_log2, window, pro,
+                                                                        splits, part_o, part_ml);
     LC_LAUNCH_CHECK("attn_prefill");
+    if (splits > 1) {
+        attn_prefill_join_kernel<D><<<dim3(NT * 64, nh), 128, 0, s>>>(part_o, part_ml, tiles, out, nh, splits);
+        LC_LAUNCH_CHECK("attn_prefill_join");
+    }
     return 0;
 }
 
@@ -723,19 +783,39 @@ LC_API int lc_attn_decode_bf16(const void* qkv, int q_stride, void* k_cache, voi
     return 0;
 }
 
+// Into how many shares the prefill kernel cuts the keys of every tile: more than one when the
+// tiles are so few that CUs would stand idle while each workgroup walks a long history (a
+// portion of a prompt that follows thousands of cached tokens); a share has at least 1,024 keys
+// (measured: with fewer, writing and joining the shares costs more than the idle CUs).
+LC_API int lc_attn_prefill_splits(int num_tiles, int nh, int nkv, int max_ctx) {
+    if (num_tiles <= 0 || nkv <= 0) return 1;
+    const long long groups = (long long)num_tiles * ((nh / nkv) % 2 == 0 ? nh / 2 : nh);
+    if (groups >= 256) return 1;
+    long long splits = 512 / groups;                      // no more workgroups than run at once
+    const int most = (max_ctx + PAGE - 1) / PAGE / 64;
+    if (splits > most) splits = most;
+    if (splits > 16) splits = 16;
+    return splits < 1 ? 1 : (int)splits;
+}
+
 // Whether the prefill kernel can norm and rotate q itself for this head size and rotary width
 // (whole heads of 128 that rotate whole or not at all).
 LC_API int lc_attn_prefill_prepares_q(int d, int rot) { return d == 128 && (rot == 0 || rot == 128); }
 
 // prologue != 0 (lc_attn_prefill_prepares_q(d, rot) must hold): q in qkv is raw; the kernel norms
 // (q_w may be null) and rotates it itself (rope_table may be null).  The step's keys and values
-// are in the cache either way.
+// are in the cache either way.  splits > 1 (at most 64): every tile's keys are cut into that
+// many shares; part_o [T rows of the batch][nh][splits][d] and part_ml [T][nh][splits][2] float32.
 LC_API int lc_attn_prefill_bf16(const void* qkv, int q_stride, const void* k_cache, const void* v_cache,
                                 void* out, const int* tiles, const int* block_table, int max_blocks,
                                 int num_tiles, int nh, int nkv, int d, int page_size, float scale,
                                 int window, int prologue, const float* q_w, float eps,
-                                const float* rope_table, int rot, hipStream_t stream) {
+                                const float* rope_table, int rot, int splits, float* part_o,
+                                float* part_ml, hipStream_t stream) {
     if (num_tiles == 0) return 0;
+    LC_CHECK(splits >= 1 && splits <= 64 && (splits == 1 || (part_o && part_ml)),
+             "attn_prefill_bf16: %d shares (1 to 64; more than one need a workspace)", splits);
+    LC_CHECK((long long)num_tiles * splits <= 0x7fffffff / 64, "attn_prefill_bf16: too many tiles (%d)", num_tiles);
     LC_CHECK(lc_attn_bf16_supported(nh, nkv, d, page_size),
              "attn_prefill_bf16: unsupported sizes nh=%d nkv=%d d=%d page=%d", nh, nkv, d, page_size);
     LC_CHECK(qkv && k_cache && v_cache && out && tiles && block_table, "attn_prefill_bf16: null pointer");
@@ -746,7 +826,8 @@ LC_API int lc_attn_prefill_bf16(const void* qkv, int q_stride, const void* k_cac
     const float sl2 = scale * 1.4426950408889634f;
     DecodePrologue pro = {q_w, nullptr, rope_table, eps, rot, 0, prologue};
 #define CALL(DD) launch_prefill<DD>((const bf16*)qkv, q_stride, (const bf16*)k_cache, (const bf16*)v_cache, \
-        (bf16*)out, tiles, block_table, max_blocks, num_tiles, nh, nkv, sl2, window, pro, stream)
+        (bf16*)out, tiles, block_table, max_blocks, num_tiles, nh, nkv, sl2, window, pro, splits,       \
+        part_o, part_ml, stream)
     LC_DISPATCH_D(d, CALL)
 #undef CALL
     return 0;

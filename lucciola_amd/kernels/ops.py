@@ -43,7 +43,8 @@ _SIGNATURES = {
     "lc_attn_bf16_supported": "iiii",
     "lc_attn_decode_splits": "iii",
     "lc_attn_decode_bf16": "pippppppppp" + "iiiiii" + "f" + "ii" + "ippfpii" + "p",
-    "lc_attn_prefill_bf16": "pippppp" + "iiiiii" + "f" + "i" + "ipfpi" + "p",
+    "lc_attn_prefill_bf16": "pippppp" + "iiiiii" + "f" + "i" + "ipfpi" + "ipp" + "p",
+    "lc_attn_prefill_splits": "iiii",
     "lc_attn_prefill_prepares_q": "ii",
     "lc_swiglu": "ppiiip",
     "lc_sample": "pppppiip",
@@ -515,12 +516,17 @@ def attention(qkv: torch.Tensor, batch: AttentionBatch, k_cache: torch.Tensor,
                   1 if all_in_decode and prologue.slots is not None else 0, _stream())
         nt = batch.prefill_tiles.shape[0]
         if nt > 0:
+            pf_splits = lib.lc_attn_prefill_splits(nt, nh, nkv, batch.max_ctx)
+            pf_o = pf_ml = None
+            if pf_splits > 1:      # few tiles after a long history: the keys are shared out
+                pf_o = torch.empty((T * nh * pf_splits * d,), dtype=torch.float32, device=qkv.device)
+                pf_ml = torch.empty((T * nh * pf_splits * 2,), dtype=torch.float32, device=qkv.device)
             _call("lc_attn_prefill_bf16", _ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
                   _ptr(out), _ptr(batch.prefill_tiles), _ptr(batch.block_table), mb, nt, nh, nkv, d,
                   page_size, scale, window, 1 if own_q else 0,
                   _ptr(prologue.q_weight if own_q else None),
                   _c_float(prologue.eps if own_q else 0.0), _ptr(rope if own_q else None),
-                  rot if own_q else 0, _stream())
+                  rot if own_q else 0, pf_splits, _ptr(pf_o), _ptr(pf_ml), _stream())
         return out
     _call("lc_attention_generic", _ptr(qkv), _c_int(qkv.shape[1]), _ptr(k_cache), _ptr(v_cache),
           _ptr(out), _c_int(_dt(qkv)), _ptr(batch.tok_req), _ptr(batch.positions),

@@ -628,3 +628,24 @@ def test_feed_tokens():
     assert torch.equal(got.cpu(), want)
     with pytest.raises(ops.KernelError):
         ops.feed_tokens(got, source.to(DEV)[:5], sampled.to(DEV))
+
+
+@pytest.mark.parametrize("nh,nkv,d,window,lengths,new", [
+    (32, 8, 128, 0, [8192], [576]),               # pairs of heads, four shares
+    (32, 8, 128, 0, [5000, 1], [100, 1]),         # single heads, eight shares, a decode token beside
+    (8, 2, 64, 0, [5000, 3000], [100, 70]),
+    (4, 4, 96, 1000, [6000], [130]),              # a window: the shares cover its pages only
+    (16, 1, 32, 0, [4100, 700], [64, 3]),
+    (32, 8, 128, 0, [900], [576])])               # no more than a share's worth of keys: not cut
+def test_attention_prefill_shares_of_the_keys(nh, nkv, d, window, lengths, new):
+    """A portion of a prompt after a long history is few tiles with many keys each: the tiles'
+    pages are shared out over several workgroups and joined, as the decode kernel does it."""
+    qkv, batch, kc, vc = paged_case(lengths, new, nh, nkv, d, 16, torch.bfloat16, seed=77)
+    nt = batch.prefill_tiles.shape[0]
+    splits = ops.library().lc_attn_prefill_splits(nt, nh, nkv, batch.max_ctx)
+    assert (splits > 1) == (max(lengths) >= 2048)
+    got = ops.attention(qkv, batch, kc, vc, nh, nkv, d, 16, d ** -0.5, window)
+    want = ref.attention(qkv.cpu(), AttentionBatch(batch.tok_req.cpu(), batch.positions.cpu(),
+                                                   batch.block_table.cpu()),
+                         kc.cpu(), vc.cpu(), nh, nkv, d, 16, d ** -0.5, window)
+    close(got, want, torch.bfloat16, atol=attention_atol(torch.bfloat16, vc))
