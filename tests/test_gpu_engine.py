@@ -318,6 +318,34 @@ def test_running_ahead_matches_waiting(dtype, key):
         assert got[True][0] == plain_qwen3.greedy(cfg, weights, prompts[0], 24)
 
 
+@pytest.mark.parametrize("trial", range(8))
+def test_running_ahead_under_random_workloads(trial):
+    """Random requests (lengths, counts, end tokens, temperature), budgets and pool sizes, some so
+    tight that requests are preempted: running ahead and waiting generate the same."""
+    import random
+    rng = random.Random(1000 + trial)
+    cfg, page, seed = configs.ALL[rng.choice("ABCD")]
+    dtype = rng.choice(["float32", "bfloat16"])
+    weights = random_weights(cfg, seed + trial, std=0.3)
+    n = rng.randint(2, 6)
+    prompts = [[rng.randrange(cfg["vocab_size"]) for _ in range(rng.randint(1, 40))] for _ in range(n)]
+    counts = [rng.randint(1, 30) for _ in range(n)]
+    eos = tuple(rng.sample(range(cfg["vocab_size"]), 12))
+    roomy = sum(len(p) + c for p, c in zip(prompts, counts)) // page + n + 2
+    tight = max((len(p) + c) // page + 2 for p, c in zip(prompts, counts)) + rng.randint(1, 6)
+    blocks, budget = rng.choice([roomy, tight]), rng.choice([8, 16, 64])
+    got = {}
+    for ahead in (False, True):
+        engine = engine_for(cfg, weights, page, blocks, dtype, max_tokens_per_step=budget, max_seqs=4,
+                            run_ahead=ahead)
+        params = [SamplingParams(max_new_tokens=c, temperature=0.8 if i % 3 == 1 else 0.0, seed=i,
+                                 eos_token_ids=eos if i % 2 == 0 else ()) for i, c in enumerate(counts)]
+        got[ahead] = engine.generate(prompts, params)
+        engine.runner.cache.check()
+        assert not engine.runner.cache.requests
+    assert got[True] == got[False]
+
+
 def test_command_line_and_async_engine(tmp_path):
     """The command line and ``AsyncEngine(model_path, max_blocks, block_size)`` /
     ``generate_async(prompt, max_new_tokens, callback)`` give the plain greedy tokens."""
