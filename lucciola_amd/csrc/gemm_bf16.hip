@@ -682,14 +682,16 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restric
 // The tile shapes of the tiled kernel.  TILE_AUTO picks by size; the others are forced through
 // lc_gemm_bf16_force_tile (tests and tuning).
 enum : int { TILE_AUTO = -1, TILE_64x128 = 0, TILE_128x128 = 1, TILE_256x128 = 2, TILE_256x192 = 3, TILE_256x256 = 4,
-              TILE_192x128 = 5, TILE_192x256 = 6, TILE_COUNT = 7 };
+              TILE_192x128 = 5, TILE_192x256 = 6, TILE_64x64 = 7, TILE_COUNT = 8 };
 static int g_force_tile = TILE_AUTO;
 constexpr int kCUs = 256;
 
 static int tile_bm(int t) {
-    return t == TILE_64x128 ? 64 : t == TILE_128x128 ? 128 : (t == TILE_192x128 || t == TILE_192x256) ? 192 : 256;
+    return (t == TILE_64x128 || t == TILE_64x64) ? 64 : t == TILE_128x128 ? 128 : (t == TILE_192x128 || t == TILE_192x256) ? 192 : 256;
 }
-static int tile_bn(int t) { return (t == TILE_256x256 || t == TILE_192x256) ? 256 : t == TILE_256x192 ? 192 : 128; }
+static int tile_bn(int t) {
+    return (t == TILE_256x256 || t == TILE_192x256) ? 256 : t == TILE_256x192 ? 192 : t == TILE_64x64 ? 64 : 128;
+}
 static long long tile_count(int t, int M, int N) {
     return (long long)((M + tile_bm(t) - 1) / tile_bm(t)) * ((N + tile_bn(t) - 1) / tile_bn(t));
 }
@@ -728,7 +730,7 @@ static int shares_for(int t, int M, int N, int K) {
     return S < 1 ? 1 : S;
 }
 
-// The tile for a product with M > 16.  Up to 64 rows: the 64-row tile.  Beyond: the shape with
+// The tile for a product with M > 16.  Up to 64 rows: a 64-row tile.  Beyond: the shape with
 // the least estimated time in microseconds.  A CU works through a round of tiles in
 // (tile area) x K x 2 / (4.63 MFLOP/us x the shape's relative rate) (measured at K = 4096: larger
 // tiles move fewer bytes per product) and 3 us to start and end.  A last round of a one-a-CU shape
@@ -738,11 +740,20 @@ static int shares_for(int t, int M, int N, int K) {
 // (partials_wanted).
 static int pick_tile(int M, int N, int K, bool partials_wanted = false) {
     if (g_force_tile != TILE_AUTO) return g_force_tile;
-    if (M <= 64) return TILE_64x128;
-    const double rate[TILE_COUNT] = {0.70, 0.82, 0.90, 0.94, 1.0, 0.87, 0.94};
+    if (M <= 64) {
+        // The 64-row tile, cut along K where its tiles are few.  Where tiles of 64 columns and
+        // whole K fill the CUs once to three times, or K is so short that a second kernel to
+        // sum the shares costs more than idle CUs, those are faster (measured: 64 x 24576 x 4096
+        // with SwiGLU 47 instead of 52 us, 64 x 6144 x 1024 9 instead of 11).
+        const long long tiles64 = tile_count(TILE_64x64, M, N);
+        if (!partials_wanted && ((tiles64 >= kCUs && tiles64 <= 3 * kCUs) || (K <= 2048 && tiles64 >= 48)))
+            return TILE_64x64;
+        return TILE_64x128;
+    }
+    const double rate[TILE_COUNT] = {0.70, 0.82, 0.90, 0.94, 1.0, 0.87, 0.94, 0.5};
     int best = -1;
     double best_cost = 0.0;
-    for (int t = M <= 128 ? TILE_64x128 : TILE_128x128; t < TILE_COUNT; ++t) {
+    for (int t = M <= 128 ? TILE_64x128 : TILE_128x128; t < TILE_64x64; ++t) {
         const long long tiles = tile_count(t, M, N);
         const double area = (double)tile_bm(t) * tile_bn(t);
         const double work_us = area * K * 2.0 / (4.63e6 * rate[t]);
@@ -915,6 +926,7 @@ static int launch_bf16(const bf16* x, const bf16* w, TO* out, float* workspace, 
     case TILE_256x192: return launch_tiled<256, 192, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     case TILE_192x128: return launch_tiled<192, 128, 3, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     case TILE_192x256: return launch_tiled<192, 256, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
+    case TILE_64x64:   return launch_tiled<64, 64, 3, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     default:           return launch_tiled<256, 256, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     }
 }
