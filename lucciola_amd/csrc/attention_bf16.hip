@@ -187,16 +187,18 @@ struct DecodePrologue {
 // Every workgroup prepares the q heads of its group itself (into LDS); the one whose share of
 // the pages holds the token's own position also prepares k and v and writes them to the
 // cache before anyone in the workgroup reads that page.
-template <int D>
-__global__ __launch_bounds__(256) void attn_decode_kernel(
+// NW waves take the pages of the workgroup's share in turn, each with one page in flight beside
+// the one it works on: a workgroup draws on memory at NW times a wave's pace.
+template <int D, int NW>
+__global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
     const bf16* __restrict__ qkv, int q_stride, bf16* k_cache, bf16* v_cache,
     bf16* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const int* __restrict__ decode_tokens,
     const int* __restrict__ tok_req, const int* __restrict__ positions,
     const int* __restrict__ block_table, int max_blocks, int nh, int nkv, float scale_log2,
     int window, int splits, DecodePrologue pro) {
-    __shared__ float sm_o[4][D * 16];
-    __shared__ float sm_m[4][16], sm_l[4][16];
+    __shared__ float sm_o[NW][D * 16];
+    __shared__ float sm_m[NW][16], sm_l[NW][16];
     __shared__ __attribute__((aligned(16))) bf16 sm_q[16 * D];
 
     const int split = blockIdx.x, kvh = blockIdx.y, di = blockIdx.z;
@@ -222,7 +224,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
         if (D == 128 && (pro.rot == 128 || pro.rot == 0)) {
             // 16 lanes a head, as the separate kernel does it (and to the same bits)
             const int j = threadIdx.x & 15;
-            for (int task = threadIdx.x >> 4; task < ntask; task += 16) {
+            for (int task = threadIdx.x >> 4; task < ntask; task += 4 * NW) {
                 if (task == G + 1) {                      // v: copied, transposed into the page
                     const head_chunk raw = *reinterpret_cast<const head_chunk*>(row + (size_t)(nh + nkv + kvh) * D + 8 * j);
                     bf16* col = v_cache + ((size_t)table[last_page] * nkv + kvh) * D * PAGE + (p % PAGE);
@@ -239,7 +241,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
                 *reinterpret_cast<head_chunk*>(dst + 8 * j) = done;
             }
         } else {
-            for (int task = wave; task < ntask; task += 4) {
+            for (int task = wave; task < ntask; task += NW) {
                 if (task == G + 1) {                          // v: copied, transposed into the page
                     const bf16* x = row + (size_t)(nh + nkv + kvh) * D;
                     bf16* col = v_cache + ((size_t)table[last_page] * nkv + kvh) * D * PAGE + (p % PAGE);
@@ -288,7 +290,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     AttnState<D, 1> st;
     init_state<D, 1>(st);
     const int lo[1] = {j_lo}, hi[1] = {p};
-    attend_range<D, 1>(st, bq, k_cache, v_cache, table, begin + wave, end, 4, nkv, kvh, lo, hi,
+    attend_range<D, 1>(st, bq, k_cache, v_cache, table, begin + wave, end, NW, nkv, kvh, lo, hi,
                        scale_log2, lane);
 
     // the waves' results meet in LDS
@@ -300,14 +302,16 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 #pragma unroll
         for (int v = 0; v < 4; ++v) sm_o[wave][(tt * 16 + kg * 4 + v) * 16 + q] = st.o[0][tt][v];
     __syncthreads();
-    for (int idx = threadIdx.x; idx < D * 16; idx += 256) {
+    for (int idx = threadIdx.x; idx < D * 16; idx += 64 * NW) {
         const int dim = idx >> 4, qq = idx & 15;
         if (qq >= G) continue;
-        float m_all = fmaxf(fmaxf(sm_m[0][qq], sm_m[1][qq]), fmaxf(sm_m[2][qq], sm_m[3][qq]));
+        float m_all = sm_m[0][qq];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) m_all = fmaxf(m_all, sm_m[w][qq]);
         float o = 0.f, lsum = 0.f;
         if (m_all != -INFINITY) {
 #pragma unroll
-            for (int w = 0; w < 4; ++w) {
+            for (int w = 0; w < NW; ++w) {
                 const float f = (sm_m[w][qq] == -INFINITY) ? 0.f : exp2f(sm_m[w][qq] - m_all);
                 o += f * sm_o[w][idx];
                 lsum += f * sm_l[w][qq];
@@ -673,6 +677,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     }
 }
 
+static int g_decode_waves = 0;   // 0: by the launch's shape
+
 template <int D>
 static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* out,
                          float* part_o, float* part_ml, const int* decode_tokens, const int* tok_req,
@@ -680,9 +686,19 @@ static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* 
                          int nkv, float scale_log2, int window, int splits, DecodePrologue pro,
                          hipStream_t s) {
     dim3 grid(splits, nkv, ND);
-    attn_decode_kernel<D><<<grid, 256, 0, s>>>(qkv, q_stride, k, v, out, part_o, part_ml,
-                                               decode_tokens, tok_req, positions, table, max_blocks,
-                                               nh, nkv, scale_log2, window, splits, pro);
+    // One workgroup per request and kv head (no shares): requests of unequal length leave the
+    // long ones running alone at the end, each at the pace its waves draw on memory; eight
+    // waves double that (64 requests of 16 to 2,176 tokens: 59 instead of 65 us; equal lengths
+    // take the same time either way, short shares are slower with eight).
+    const int waves = g_decode_waves ? g_decode_waves : (splits == 1 && max_blocks >= 32 ? 8 : 4);
+    if (waves == 8)
+        attn_decode_kernel<D, 8><<<grid, 512, 0, s>>>(qkv, q_stride, k, v, out, part_o, part_ml,
+                                                      decode_tokens, tok_req, positions, table, max_blocks,
+                                                      nh, nkv, scale_log2, window, splits, pro);
+    else
+        attn_decode_kernel<D, 4><<<grid, 256, 0, s>>>(qkv, q_stride, k, v, out, part_o, part_ml,
+                                                      decode_tokens, tok_req, positions, table, max_blocks,
+                                                      nh, nkv, scale_log2, window, splits, pro);
     LC_LAUNCH_CHECK("attn_decode");
     if (splits > 1) {
         attn_decode_join_kernel<D><<<dim3(ND, nh), 128, 0, s>>>(
@@ -729,6 +745,13 @@ LC_API int lc_attn_bf16_supported(int nh, int nkv, int d, int page_size) {
     if (page_size != PAGE || nkv <= 0 || nh % nkv != 0) return 0;
     if (nh / nkv > 16 || nh > 65535 || nkv > 65535) return 0;
     return d == 32 || d == 64 || d == 96 || d == 128;
+}
+
+// Waves of a decode workgroup (4 or 8; 0: chosen by the launch's shape).  For tests and tuning.
+LC_API int lc_attn_decode_waves(int waves) {
+    LC_CHECK(waves == 0 || waves == 4 || waves == 8, "attn_decode: %d waves (0, 4 or 8)", waves);
+    g_decode_waves = waves;
+    return 0;
 }
 
 // Into how many shares the decode kernel cuts a request's pages.

@@ -42,6 +42,7 @@ _SIGNATURES = {
     "lc_attention_generic": "pipppipppiiiiiifip",
     "lc_attn_bf16_supported": "iiii",
     "lc_attn_decode_splits": "iii",
+    "lc_attn_decode_waves": "i",
     "lc_attn_decode_bf16": "pippppppppp" + "iiiiii" + "f" + "ii" + "ippfpii" + "p",
     "lc_attn_prefill_bf16": "pippppp" + "iiiiii" + "f" + "i" + "ipfpi" + "ipp" + "p",
     "lc_attn_prefill_splits": "iiii",

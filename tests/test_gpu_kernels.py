@@ -393,11 +393,21 @@ def test_attention_bf16_long_contexts(nh, nkv, d, window):
 @pytest.mark.parametrize("nh,nkv,d,window,rot,normed", [(32, 8, 128, 0, 128, True), (6, 2, 96, 24, 96, True),
                                                         (8, 1, 64, 0, 32, False), (4, 4, 32, 0, 0, True),
                                                         (16, 1, 32, 0, 32, True)])
-def test_attention_decode_with_prologue_in_the_kernel(nh, nkv, d, window, rot, normed):
+@pytest.mark.parametrize("waves", [0, 4, 8])
+def test_attention_decode_with_prologue_in_the_kernel(nh, nkv, d, window, rot, normed, waves):
     """A step of single tokens with raw q, k, v: the decode kernel norms, rotates and writes
     the cache itself.  Output and cache must equal those of the separate kernel followed by
     the plain decode kernel, for short and long contexts (one or many shares of the pages),
-    a token at a page's first and last place, part of the head rotated or none."""
+    a token at a page's first and last place, part of the head rotated or none; with workgroups
+    of four and of eight waves."""
+    ops.library().lc_attn_decode_waves(waves)
+    try:
+        decode_prologue_case(nh, nkv, d, window, rot, normed)
+    finally:
+        ops.library().lc_attn_decode_waves(0)
+
+
+def decode_prologue_case(nh, nkv, d, window, rot, normed):
     lengths = [1, 16, 17, 300, 2049, 5000, 33]
     qkv, batch, kc, vc = paged_case(lengths, [1] * len(lengths), nh, nkv, d, 16, torch.bfloat16, seed=90)
     assert ops.library().lc_attn_bf16_supported(nh, nkv, d, 16)
@@ -644,6 +654,22 @@ def test_attention_prefill_shares_of_the_keys(nh, nkv, d, window, lengths, new):
     nt = batch.prefill_tiles.shape[0]
     splits = ops.library().lc_attn_prefill_splits(nt, nh, nkv, batch.max_ctx)
     assert (splits > 1) == (max(lengths) >= 2048)
+    got = ops.attention(qkv, batch, kc, vc, nh, nkv, d, 16, d ** -0.5, window)
+    want = ref.attention(qkv.cpu(), AttentionBatch(batch.tok_req.cpu(), batch.positions.cpu(),
+                                                   batch.block_table.cpu()),
+                         kc.cpu(), vc.cpu(), nh, nkv, d, 16, d ** -0.5, window)
+    close(got, want, torch.bfloat16, atol=attention_atol(torch.bfloat16, vc))
+
+
+@pytest.mark.parametrize("nh,nkv,d,window", [(32, 8, 128, 0), (6, 2, 96, 700), (8, 1, 64, 0)])
+def test_attention_decode_of_many_requests_of_unequal_length(nh, nkv, d, window):
+    """So many requests that each gets one workgroup per kv head (of eight waves then), lengths
+    from one token to thousands."""
+    rng = random.Random(5)
+    lengths = [rng.choice([1, 15, 16, 17, 100, 700, 2100, 3000]) for _ in range(70)]
+    qkv, batch, kc, vc = paged_case(lengths, [1] * len(lengths), nh, nkv, d, 16, torch.bfloat16, seed=95)
+    if nkv >= 8:
+        assert ops.library().lc_attn_decode_splits(len(lengths), nkv, max(lengths)) == 1
     got = ops.attention(qkv, batch, kc, vc, nh, nkv, d, 16, d ** -0.5, window)
     want = ref.attention(qkv.cpu(), AttentionBatch(batch.tok_req.cpu(), batch.positions.cpu(),
                                                    batch.block_table.cpu()),
