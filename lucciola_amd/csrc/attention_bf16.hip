@@ -754,13 +754,19 @@ LC_API int lc_attn_decode_waves(int waves) {
     return 0;
 }
 
-// Into how many shares the decode kernel cuts a request's pages.
+// Into how many shares the decode kernel cuts a request's pages.  Two workgroups fit on a CU
+// (measured to beat four), 512 on the GPU, and from about 384 on they draw all that memory
+// gives.  So: as many shares as keep the workgroups within 512 (one more, and a second round
+// of workgroups has to wait for the first: 3 requests in 22 shares each took 31 us, in 21 26);
+// with 257 to 383 workgroups of whole requests, three shares each (40 requests: 252 instead
+// of 282 us), with 384 to 447 two (48 requests: 291 instead of 305); from 448 on none.  A share has
+// 8 pages or more, and there are at most 32.
 LC_API int lc_attn_decode_splits(int num_decode, int nkv, int max_ctx) {
     if (num_decode <= 0) return 1;
     const int pages = (max_ctx + PAGE - 1) / PAGE;
     const long long base = (long long)num_decode * nkv;
-    long long splits = (512 + base - 1) / base;           // two workgroups a CU: measured to beat four
-    const int most = (pages + 7) / 8;                     // at least 8 pages per workgroup
+    long long splits = base >= 448 ? 1 : base >= 384 ? 2 : base > 256 ? 3 : 512 / base;
+    const int most = (pages + 7) / 8;
     if (splits > most) splits = most;
     if (splits > 32) splits = 32;
     if (splits < 1) splits = 1;
