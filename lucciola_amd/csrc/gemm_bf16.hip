@@ -720,8 +720,12 @@ static TailPlan tail_plan(int t, int M, int N, int K) {
 // as it takes to give every CU about two workgroups when whole-K tiles would be too few.  Only
 // the two small tiles are cut as a whole; the shares are summed by splitk_reduce_kernel, or by
 // whoever takes the partial sums (lc_gemm_bf16_partials).
+// products of up to 64 rows whose shares someone else sums: tiles of 64 x 64 make half as many
+// shares as tiles of 64 x 128 for the same number of workgroups (64 x 4096 x 4096 and the norm
+// after it: 17.8 instead of 23.5 us)
+static int g_small_partials = 1;
 static int shares_for(int t, int M, int N, int K) {
-    if (t != TILE_64x128 && t != TILE_128x128) return 1;
+    if (t != TILE_64x128 && t != TILE_128x128 && !(t == TILE_64x64 && g_small_partials)) return 1;
     const long long tiles = tile_count(t, M, N);
     if (tiles >= 400) return 1;
     const int nk = K / TL_K;
@@ -748,6 +752,7 @@ static int pick_tile(int M, int N, int K, bool partials_wanted = false) {
         const long long tiles64 = tile_count(TILE_64x64, M, N);
         if (!partials_wanted && ((tiles64 >= kCUs && tiles64 <= 3 * kCUs) || (K <= 2048 && tiles64 >= 48)))
             return TILE_64x64;
+        if (partials_wanted && g_small_partials) return TILE_64x64;
         return TILE_64x128;
     }
     const double rate[TILE_COUNT] = {0.70, 0.82, 0.90, 0.94, 1.0, 0.87, 0.94, 0.5};
@@ -1004,6 +1009,9 @@ LC_API int lc_gemm_bf16_even_rows(int on) {
     return 0;
 }
 
+// 0: shares that are handed on come from tiles of 64 x 128 also for up to 64 rows.  For tests and tuning.
+LC_API int lc_gemm_bf16_small_partials(int on) { g_small_partials = on; return 0; }
+
 LC_API int lc_gemm_bf16_piece_stride(int M) {
     int stride = 1;
     while (stride < M) stride *= 2;
@@ -1090,7 +1098,11 @@ LC_API int lc_gemm_bf16_partials(const void* x, const void* w, float* partials, 
              "gemm_bf16_partials: operands must be 16-byte aligned");
     const bf16* xb = (const bf16*)x;
     const bf16* wb = (const bf16*)w;
-    if (pick_tile(M, N, K, true) == TILE_64x128) {
+    if (pick_tile(M, N, K, true) == TILE_64x64) {
+        const int tiles_m = (M + 63) / 64, tiles = tiles_m * ((N + 63) / 64);
+        gemm_tiled_kernel<64, 64, 3, 0, true, float><<<dim3(tiles, shares), 256, 0, stream>>>(
+            xb, wb, nullptr, partials, M, N, K, tiles_m, 0, tiles, 0);
+    } else if (pick_tile(M, N, K, true) == TILE_64x128) {
         const int tiles_m = (M + 63) / 64, tiles = tiles_m * ((N + 127) / 128);
         gemm_tiled_kernel<64, 128, 3, 0, true, float><<<dim3(tiles, shares), 256, 0, stream>>>(
             xb, wb, nullptr, partials, M, N, K, tiles_m, 0, tiles, 0);

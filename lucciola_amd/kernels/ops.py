@@ -31,6 +31,7 @@ _SIGNATURES = {
     "lc_gemm_bf16_force_tile": "i",
     "lc_gemm_bf16_force_skinny": "i",
     "lc_gemm_bf16_even_rows": "i",
+    "lc_gemm_bf16_small_partials": "i",
     "lc_gemm_bf16_residual_pieces": "iii",
     "lc_gemm_bf16_piece_stride": "i",
     "lc_gemm_bf16_shares": "iii",

@@ -598,10 +598,19 @@ def few_rows_case(M, N, K):
 
 
 @pytest.mark.parametrize("M,H,K", [(40, 512, 2048), (64, 4096, 4096), (100, 384, 1024), (17, 1152, 1536)])
-def test_norm_sums_the_shares_of_a_product_cut_along_k(M, H, K):
+@pytest.mark.parametrize("small", [1, 0])
+def test_norm_sums_the_shares_of_a_product_cut_along_k(M, H, K, small):
     """More than 16 rows and few tiles: the product before a norm is cut along K; its shares
     stay float32 and the norm kernel adds them to the stream itself (all rows, and chosen rows
     with the stream left alone)."""
+    ops.library().lc_gemm_bf16_small_partials(small)     # up to 64 rows: tiles of 64 x 64 or of 64 x 128
+    try:
+        norm_of_shares_case(M, H, K)
+    finally:
+        ops.library().lc_gemm_bf16_small_partials(1)
+
+
+def norm_of_shares_case(M, H, K):
     eps = 1e-6
     h = rnd(M, H, seed=90, scale=2.0)
     x = rnd(M, K, dtype=torch.bfloat16, seed=91)
