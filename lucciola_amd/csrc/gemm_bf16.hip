@@ -718,14 +718,20 @@ static TailPlan tail_plan(int t, int M, int N, int K) {
 
 // Into how many shares of K a product with this tile is cut as a whole (1: not at all): as many
 // as it takes to give every CU about two workgroups when whole-K tiles would be too few.  Only
-// the two small tiles are cut as a whole; the shares are summed by splitk_reduce_kernel, or by
-// whoever takes the partial sums (lc_gemm_bf16_partials).
-// products of up to 64 rows whose shares someone else sums: tiles of 64 x 64 make half as many
-// shares as tiles of 64 x 128 for the same number of workgroups (64 x 4096 x 4096 and the norm
-// after it: 17.8 instead of 23.5 us)
-static int g_small_partials = 1;
-static int shares_for(int t, int M, int N, int K) {
-    if (t != TILE_64x128 && t != TILE_128x128 && !(t == TILE_64x64 && g_small_partials)) return 1;
+// the small tiles are cut as a whole; the shares are summed by splitk_reduce_kernel, or by
+// whoever takes the partial sums (lc_gemm_bf16_partials).  The tile of 64 x 64 is for up to 64
+// rows: cut, it makes half as many shares as the tile of 64 x 128 for the same number of
+// workgroups (64 x 4096 x 4096 and the norm that sums its shares: 17.8 instead of 23.5 us;
+// 64 x 6144 x 4096 and the sum of its shares: 16.4 instead of 19.6); whole, it saves the kernel
+// that sums (see pick_tile).
+static int g_small_partials = 1;   // 0: shares that are handed on come from 64 x 128 tiles (tests, tuning)
+static bool whole_k_64x64(int M, int N, int K) {
+    const long long tiles64 = tile_count(TILE_64x64, M, N);
+    return (tiles64 >= kCUs && tiles64 <= 3 * kCUs) || (K <= 2048 && tiles64 >= 48);
+}
+static int shares_for(int t, int M, int N, int K, bool partials_wanted = false) {
+    if (t != TILE_64x128 && t != TILE_128x128 && t != TILE_64x64) return 1;
+    if (t == TILE_64x64 && g_force_tile == TILE_AUTO && !partials_wanted && whole_k_64x64(M, N, K)) return 1;
     const long long tiles = tile_count(t, M, N);
     if (tiles >= 400) return 1;
     const int nk = K / TL_K;
@@ -745,14 +751,13 @@ static int shares_for(int t, int M, int N, int K) {
 static int pick_tile(int M, int N, int K, bool partials_wanted = false) {
     if (g_force_tile != TILE_AUTO) return g_force_tile;
     if (M <= 64) {
-        // The 64-row tile, cut along K where its tiles are few.  Where tiles of 64 columns and
-        // whole K fill the CUs once to three times, or K is so short that a second kernel to
-        // sum the shares costs more than idle CUs, those are faster (measured: 64 x 24576 x 4096
-        // with SwiGLU 47 instead of 52 us, 64 x 6144 x 1024 9 instead of 11).
-        const long long tiles64 = tile_count(TILE_64x64, M, N);
-        if (!partials_wanted && ((tiles64 >= kCUs && tiles64 <= 3 * kCUs) || (K <= 2048 && tiles64 >= 48)))
-            return TILE_64x64;
-        if (partials_wanted && g_small_partials) return TILE_64x64;
+        // Tiles of 64 x 64 and whole K where they fill the CUs once to three times, or where K
+        // is so short that a second kernel to sum shares costs more than idle CUs (measured:
+        // 64 x 24576 x 4096 with SwiGLU 47 instead of 52 us, 64 x 6144 x 1024 9 instead of 11);
+        // tiles of 64 x 64 cut along K where there are few of them, and for shares that are
+        // handed on; else tiles of 64 x 128, cut where they are few.
+        if (partials_wanted) return g_small_partials ? TILE_64x64 : TILE_64x128;
+        if (whole_k_64x64(M, N, K) || tile_count(TILE_64x64, M, N) <= 128) return TILE_64x64;
         return TILE_64x128;
     }
     const double rate[TILE_COUNT] = {0.70, 0.82, 0.90, 0.94, 1.0, 0.87, 0.94, 0.5};
@@ -784,7 +789,7 @@ static int pick_tile(int M, int N, int K, bool partials_wanted = false) {
 
 static int splitk_shares(int M, int N, int K, bool partials_wanted = false) {
     if (M <= 16) return 1;
-    return shares_for(pick_tile(M, N, K, partials_wanted), M, N, K);
+    return shares_for(pick_tile(M, N, K, partials_wanted), M, N, K, partials_wanted);
 }
 
 // float32 words of workspace that the product needs (0: none)
