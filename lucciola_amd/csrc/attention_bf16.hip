@@ -182,6 +182,12 @@ struct DecodePrologue {
     int rot;
     int write_kv;
     int enabled;
+    // the raw q, k, v as the shares of a product cut along K (float32 [num_shares][rows][width],
+    // summed in their order and rounded to bfloat16 as the kernel that sums them would), or null
+    const float* shares;
+    int num_shares;
+    int width;
+    long long share_stride;
 };
 
 // Every workgroup prepares the q heads of its group itself (into LDS); the one whose share of
@@ -224,19 +230,36 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
         if (D == 128 && (pro.rot == 128 || pro.rot == 0)) {
             // 16 lanes a head, as the separate kernel does it (and to the same bits)
             const int j = threadIdx.x & 15;
+            // eight entries of the token's row of q, k, v from column `col` on
+            auto chunk_at = [&](size_t col) -> head_chunk {
+                if (!pro.shares) return *reinterpret_cast<const head_chunk*>(row + col);
+                const float* src = pro.shares + (size_t)t * pro.width + col;
+                floatx4 lo4 = {0.f, 0.f, 0.f, 0.f}, hi4 = {0.f, 0.f, 0.f, 0.f};
+                for (int sh = 0; sh < pro.num_shares; ++sh) {
+                    lo4 += *reinterpret_cast<const floatx4*>(src + (size_t)sh * pro.share_stride);
+                    hi4 += *reinterpret_cast<const floatx4*>(src + (size_t)sh * pro.share_stride + 4);
+                }
+                head_chunk out8;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    out8[e] = static_cast<bf16>(lo4[e]);
+                    out8[4 + e] = static_cast<bf16>(hi4[e]);
+                }
+                return out8;
+            };
             for (int task = threadIdx.x >> 4; task < ntask; task += 4 * NW) {
                 if (task == G + 1) {                      // v: copied, transposed into the page
-                    const head_chunk raw = *reinterpret_cast<const head_chunk*>(row + (size_t)(nh + nkv + kvh) * D + 8 * j);
+                    const head_chunk raw = chunk_at((size_t)(nh + nkv + kvh) * D + 8 * j);
                     bf16* col = v_cache + ((size_t)table[last_page] * nkv + kvh) * D * PAGE + (p % PAGE);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) col[(size_t)(8 * j + e) * PAGE] = raw[e];
                     continue;
                 }
                 const bool is_k = task == G;
-                const bf16* x = row + (size_t)(is_k ? nh + kvh : kvh * G + task) * D + 8 * j;
+                const size_t col = (size_t)(is_k ? nh + kvh : kvh * G + task) * D + 8 * j;
                 bf16* dst = is_k ? k_cache + (((size_t)table[last_page] * nkv + kvh) * PAGE + (p % PAGE)) * D
                                  : sm_q + task * D;
-                const head_chunk done = head128_norm_rope(*reinterpret_cast<const head_chunk*>(x), j,
+                const head_chunk done = head128_norm_rope(chunk_at(col), j,
                                                           is_k ? pro.k_w : pro.q_w, pro.eps, cs);
                 *reinterpret_cast<head_chunk*>(dst + 8 * j) = done;
             }
@@ -782,6 +805,11 @@ LC_API int lc_attn_decode_splits(int num_decode, int nkv, int max_ctx) {
         default: LC_CHECK(false, "attention_bf16: head size %d has no matrix-core kernel", d); \
     }
 
+// Whether lc_attn_decode_bf16 takes the raw q, k, v as the float32 shares of a product cut along K
+// (qkv_shares [num_shares][share_rows][q_stride], summed in their order and rounded to bfloat16 as
+// the kernel that sums shares does): with its own preparation of whole heads of 128.
+LC_API int lc_attn_decode_takes_shares(int d, int rot) { return d == 128 && (rot == 0 || rot == 128); }
+
 // prologue != 0: qkv holds the raw projections; the kernel norms and rotates q and k itself
 // (q_w, k_w, rope_table may be null; rot entries of a head rotate) and, if write_kv != 0, writes
 // the tokens' k and v to the cache.  Otherwise qkv is ready and the cache holds the tokens.
@@ -791,13 +819,21 @@ LC_API int lc_attn_decode_bf16(const void* qkv, int q_stride, void* k_cache, voi
                                int max_blocks, int num_decode, int nh, int nkv, int d, int page_size,
                                float scale, int window, int splits, int prologue, const float* q_w,
                                const float* k_w, float eps, const float* rope_table, int rot,
-                               int write_kv, hipStream_t stream) {
+                               int write_kv, const float* qkv_shares, int num_shares, int share_rows,
+                               hipStream_t stream) {
     if (num_decode == 0) return 0;
     LC_CHECK(!prologue || (rot >= 0 && rot <= d && rot % 2 == 0 && (q_w == nullptr) == (k_w == nullptr)),
              "attn_decode_bf16: bad prologue (rot=%d of %d)", rot, d);
-    DecodePrologue pro = {q_w, k_w, rope_table, eps, rope_table ? rot : 0, write_kv, prologue};
+    DecodePrologue pro = {q_w, k_w, rope_table, eps, rope_table ? rot : 0, write_kv, prologue,
+                          qkv_shares, num_shares, q_stride, (long long)share_rows * q_stride};
     LC_CHECK(lc_attn_bf16_supported(nh, nkv, d, page_size),
              "attn_decode_bf16: unsupported sizes nh=%d nkv=%d d=%d page=%d", nh, nkv, d, page_size);
+    LC_CHECK(!qkv_shares || lc_attn_decode_takes_shares(d, prologue ? pro.rot : -1),
+             "attn_decode_bf16: q, k, v as shares of a product need the kernel's own preparation of heads of 128 "
+             "(d=%d, %d rotary entries)", d, pro.rot);
+    LC_CHECK(!qkv_shares || (num_shares >= 1 && share_rows >= 1 && q_stride % 4 == 0 && (uintptr_t)qkv_shares % 16 == 0),
+             "attn_decode_bf16: bad shares (%d of %d rows)", num_shares, share_rows);
+    if (qkv_shares && !qkv) qkv = qkv_shares;      // never read, but not null
     LC_CHECK(qkv && k_cache && v_cache && out && decode_tokens && tok_req && positions && block_table,
              "attn_decode_bf16: null pointer");
     LC_CHECK(splits >= 1 && splits <= 65535 && (splits == 1 || (part_o && part_ml)),

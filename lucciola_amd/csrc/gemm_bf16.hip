@@ -1120,3 +1120,18 @@ LC_API int lc_gemm_bf16_partials(const void* x, const void* w, float* partials, 
     return 0;
 }
 
+
+// out [M, N] (dt: bfloat16 or float32) = the sum of partials [shares][M][N] in their order: what
+// lc_gemm_bf16 itself does with the shares of a product that it cuts along K.
+LC_API int lc_gemm_bf16_sum_shares(const float* partials, void* out, int dt, int M, int N, int shares,
+                                   hipStream_t stream) {
+    LC_CHECK(partials && out && M >= 0 && N > 0 && shares >= 1, "gemm_bf16_sum_shares: bad arguments");
+    if (M == 0) return 0;
+    const size_t work = (size_t)M * N;
+    const int blocks = (int)((work + 255) / 256 < 65535 * 16 ? (work + 255) / 256 : 65535 * 16);
+    if (dt == DT_BF16) splitk_reduce_kernel<0, bf16><<<blocks, 256, 0, stream>>>(partials, (bf16*)out, M, N, shares);
+    else if (dt == DT_F32) splitk_reduce_kernel<0, float><<<blocks, 256, 0, stream>>>(partials, (float*)out, M, N, shares);
+    else LC_CHECK(false, "gemm_bf16_sum_shares: unknown dtype %d", dt);
+    LC_LAUNCH_CHECK("splitk_reduce");
+    return 0;
+}

@@ -44,7 +44,9 @@ _SIGNATURES = {
     "lc_attn_bf16_supported": "iiii",
     "lc_attn_decode_splits": "iii",
     "lc_attn_decode_waves": "i",
-    "lc_attn_decode_bf16": "pippppppppp" + "iiiiii" + "f" + "ii" + "ippfpii" + "p",
+    "lc_attn_decode_bf16": "pippppppppp" + "iiiiii" + "f" + "ii" + "ippfpii" + "pii" + "p",
+    "lc_attn_decode_takes_shares": "ii",
+    "lc_gemm_bf16_sum_shares": "ppiiiip",
     "lc_attn_prefill_bf16": "pippppp" + "iiiiii" + "f" + "i" + "ipfpi" + "ipp" + "p",
     "lc_attn_prefill_splits": "iiii",
     "lc_attn_prefill_prepares_q": "ii",
@@ -183,9 +185,31 @@ class ScaledRows:
         return rmsnorm(self.h, None, self.weight, self.eps, self.x.dtype)
 
 
+@dataclass
+class ProductShares:
+    """``x . w^T`` as the float32 shares [S, M, N] of a product that was cut along K: their sum
+    in this order, rounded to ``out_dtype``, is the product.  Handed only to code that asked for
+    it (``gemm(..., shares=True)``) and sums the shares itself, which saves the kernel that
+    would."""
+
+    partials: torch.Tensor
+    out_dtype: torch.dtype
+
+    @property
+    def shape(self):
+        return self.partials.shape[1:]
+
+    def value(self) -> torch.Tensor:
+        S, M, N = self.partials.shape
+        out = torch.empty((M, N), dtype=self.out_dtype, device=self.partials.device)
+        _call("lc_gemm_bf16_sum_shares", _ptr(self.partials), _ptr(out), _c_int(_dt(out)), _c_int(M),
+              _c_int(N), _c_int(S), _stream())
+        return out
+
+
 def value(t):
     """The tensor that ``t`` stands for (``t`` itself if it is one)."""
-    return t.value() if isinstance(t, (PendingProduct, ScaledRows)) else t
+    return t.value() if isinstance(t, (PendingProduct, ScaledRows, ProductShares)) else t
 
 
 def rmsnorm(h: torch.Tensor, delta, weight: torch.Tensor, eps: float,
@@ -272,12 +296,14 @@ def _scaled_product(x: "ScaledRows", w: torch.Tensor, epilogue: int) -> Optional
     return out
 
 
-def gemm(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None, defer: bool = False):
+def gemm(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None, defer: bool = False,
+         shares: bool = False):
     """``x`` [M, K] times ``w`` [N, K] transposed -> [M, N]; float32 accumulation.
 
     ``x`` may be ScaledRows.  ``defer``: the result is a branch's output that goes to the
     residual stream; where the kernel that computes it can add it there itself, a
-    PendingProduct comes back instead of a tensor."""
+    PendingProduct comes back instead of a tensor.  ``shares``: the caller sums the shares of
+    a product that is cut along K itself; where this one is, ProductShares come back."""
     if isinstance(x, ScaledRows):
         if out_dtype in (None, torch.bfloat16) and not defer:
             out = _scaled_product(x, w, 0)
@@ -294,6 +320,13 @@ def gemm(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None, defer: boo
     if (defer and out_dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
             and (library().lc_gemm_bf16_residual_pieces(M, N, K) or library().lc_gemm_bf16_shares(M, N, K))):
         return PendingProduct(x, w, out_dtype)
+    if shares and out_dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+        count = library().lc_gemm_bf16_shares(M, N, K)
+        if count:
+            partials = torch.empty((count, M, N), dtype=torch.float32, device=x.device)
+            _call("lc_gemm_bf16_partials", _ptr(x), _ptr(w), _ptr(partials), _c_int(M), _c_int(N),
+                  _c_int(K), _stream())
+            return ProductShares(partials, out_dtype)
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     if M == 0:
         return out
@@ -460,17 +493,41 @@ class QKPrologue:
     slots: Optional[torch.Tensor]
 
 
-def attention(qkv: torch.Tensor, batch: AttentionBatch, k_cache: torch.Tensor,
+def attention_takes_shares(batch: AttentionBatch, T: int, nh: int, nkv: int, d: int, page_size: int,
+                           dtype: torch.dtype, rot: int) -> bool:
+    """Whether ``attention`` can take the raw q, k, v of this step as ProductShares: a step of
+    single tokens in bfloat16, whose decode kernel prepares whole heads of 128 itself and sums
+    the shares as it reads them."""
+    lib = library()
+    return bool(dtype == torch.bfloat16 and batch.decode_tokens is not None
+                and batch.prefill_tiles is not None and batch.num_decode == T and T > 0
+                and lib.lc_attn_bf16_supported(nh, nkv, d, page_size)
+                and lib.lc_attn_decode_takes_shares(d, rot))
+
+
+def attention(qkv, batch: AttentionBatch, k_cache: torch.Tensor,
               v_cache: torch.Tensor, nh: int, nkv: int, d: int, page_size: int, scale: float,
               window: int = 0, prologue: Optional[QKPrologue] = None) -> torch.Tensor:
     """Causal attention of the q heads in ``qkv`` [T, (nh + 2 nkv) d] over the cached keys and
     values -> [T, nh d].  Without ``prologue`` the step's own keys and values have been written
     already and q is ready; with it, ``qkv`` is raw, and what is left raw in it afterwards is
     not defined (q stays raw where the attention kernels prepare it on the fly)."""
+    shares = None
+    if isinstance(qkv, ProductShares):
+        # asked for by a caller who had attention_takes_shares say yes; anything else gets the sum
+        rope0 = prologue.rope_table if prologue is not None else None
+        if (prologue is not None and qkv.out_dtype == torch.bfloat16
+                and attention_takes_shares(batch, qkv.shape[0], nh, nkv, d, page_size, qkv.out_dtype,
+                                           rope0.shape[1] if rope0 is not None else 0)
+                and (prologue.q_weight is None) == (prologue.k_weight is None)):
+            shares = qkv.partials
+            qkv = torch.empty((0, shares.shape[2]), dtype=torch.bfloat16, device=shares.device)
+        else:
+            qkv = qkv.value()
     _need(qkv, "qkv", None, 2)
     _need(k_cache, "k cache", qkv.dtype, 4)
     _need(v_cache, "v cache", qkv.dtype, 4)
-    T = qkv.shape[0]
+    T = qkv.shape[0] if shares is None else shares.shape[1]
     out = torch.empty((T, nh * d), dtype=qkv.dtype, device=qkv.device)
     if T == 0:
         return out
@@ -506,7 +563,7 @@ def attention(qkv: torch.Tensor, batch: AttentionBatch, k_cache: torch.Tensor,
             if splits > 1:
                 part_o = torch.empty((nd * nh * splits * d,), dtype=torch.float32, device=qkv.device)
                 part_ml = torch.empty((nd * nh * splits * 2,), dtype=torch.float32, device=qkv.device)
-            _call("lc_attn_decode_bf16", _ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
+            _call("lc_attn_decode_bf16", _ptr(qkv if shares is None else None), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
                   _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(batch.decode_tokens),
                   _ptr(batch.tok_req), _ptr(batch.positions), _ptr(batch.block_table), mb, nd, nh,
                   nkv, d, page_size, scale, window, splits,
@@ -515,7 +572,9 @@ def attention(qkv: torch.Tensor, batch: AttentionBatch, k_cache: torch.Tensor,
                   _ptr(prologue.k_weight if in_kernel else None),
                   _c_float(prologue.eps if in_kernel else 0.0), _ptr(rope if in_kernel else None),
                   rot if in_kernel else 0,
-                  1 if all_in_decode and prologue.slots is not None else 0, _stream())
+                  1 if all_in_decode and prologue.slots is not None else 0,
+                  _ptr(shares), shares.shape[0] if shares is not None else 0,
+                  shares.shape[1] if shares is not None else 0, _stream())
         nt = batch.prefill_tiles.shape[0]
         if nt > 0:
             pf_splits = lib.lc_attn_prefill_splits(nt, nh, nkv, batch.max_ctx)

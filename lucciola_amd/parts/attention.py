@@ -71,7 +71,6 @@ class Attention(Part):
         return PagedKV(self.nkv, self.d, self.window)
 
     def forward(self, x: torch.Tensor, site) -> torch.Tensor:
-        qkv = ops.gemm(x, self.qkv, self.dtype)
         attn = site.attn
         q_w = k_w = None
         eps = 0.0
@@ -81,8 +80,15 @@ class Attention(Part):
         table = None
         if self.position is not None:
             table = self.position.rotary_table(site.batch.max_position)
-            if table is None:
-                self.position.apply(qkv, self.nh, self.nkv, self.d, attn.positions)
+        # where the q/k/v product is cut along K and the attention kernel can sum its shares
+        # as it reads them, the kernel that would sum them is saved
+        rows = x.x.shape[0] if isinstance(x, ops.ScaledRows) else x.shape[0]
+        as_shares = ((table is not None or self.position is None)
+                     and ops.attention_takes_shares(attn, rows, self.nh, self.nkv, self.d, site.page_size,
+                                                    self.dtype, table.shape[1] if table is not None else 0))
+        qkv = ops.gemm(x, self.qkv, self.dtype, shares=as_shares)
+        if self.position is not None and table is None:
+            self.position.apply(qkv, self.nh, self.nkv, self.d, attn.positions)
         k_cache, v_cache = site.kv
         prologue = ops.QKPrologue(q_w, k_w, eps, table, attn.slots if site.writes_cache else None)
         o = ops.attention(qkv, attn, k_cache, v_cache, self.nh, self.nkv, self.d, site.page_size,

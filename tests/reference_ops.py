@@ -33,7 +33,7 @@ def rmsnorm_act(x, weight, eps):
     return (v * inv * weight.to(F64)).to(x.dtype)
 
 
-def gemm(x, w, out_dtype=None, defer=False):   # never defers
+def gemm(x, w, out_dtype=None, defer=False, shares=False):   # never defers, never hands out shares
     return (x.to(F64) @ w.to(F64).T).to(out_dtype or x.dtype)
 
 
@@ -119,12 +119,16 @@ def sample(logits, temperature=None, uniform=None):
     return out
 
 
+def attention_takes_shares(*args, **kwargs):
+    return False
+
+
 def feed_tokens(ids, source, sampled):
     take = source >= 0
     ids[take] = sampled[source[take].long()]
 
 
-ALL = ("feed_tokens", "embedding", "rmsnorm", "rmsnorm_act", "gemm", "qk_norm_rope_write", "attention",
+ALL = ("feed_tokens", "attention_takes_shares", "embedding", "rmsnorm", "rmsnorm_act", "gemm", "qk_norm_rope_write", "attention",
        "swiglu", "sample")
 
 

@@ -427,3 +427,43 @@ def test_layers_of_the_8b_size(dtype):
         got = replay(runner, steps)
         worst = compare(got, cfg, weights, prompts, TOL[dtype], refs)
         print(f"8B-size layers {dtype}: worst relative error {worst:.3e}")
+
+
+@pytest.mark.parametrize("requests", [20, 40])
+def test_many_requests_decode_together(requests):
+    """More than 16 requests decode in one step (heads of 128, bfloat16): the products go through
+    the tiled kernels, cut along K; the norms sum the shares of the output and down products, the
+    attention kernel those of q, k, v; the steps are replayed from graphs.  Every logit row
+    against the plain implementation."""
+    cfg = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 1024,
+           "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 128,
+           "intermediate_size": 1536, "vocab_size": 300, "rope_theta": 100000.0,
+           "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 4096,
+           "initializer_range": 0.03}
+    rng = __import__("random").Random(requests)
+    weights = random_weights(cfg, 21)
+    prompts = prompts_for(cfg, [rng.randint(2, 40) for _ in range(requests)], 22)
+    tail = 5
+    steps = []
+    names = list(prompts)
+    for i in range(0, requests, 8):      # prompts less their last tokens, eight requests a step
+        steps.append(([(n, prompts[n][:-tail], []) for n in names[i:i + 8] if len(prompts[n]) > tail], []))
+    for k in range(tail):                # then everybody's next token, all in one step
+        entries = []
+        for n in names:
+            ids = prompts[n]
+            at = len(ids) - tail + k if len(ids) > tail else k
+            if at < len(ids):
+                entries.append((n, [ids[at]], [0]))
+        steps.append((entries, []))
+    steps[-1] = (steps[-1][0], names)
+    runner = make_runner(cfg, weights, 16, 4 * requests, "bfloat16", DEV, max_seqs=requests)
+    got = replay(runner, steps)
+    assert runner.graph_replays >= 2
+    assert ops_library().lc_gemm_bf16_shares(requests, (4 + 2 * 2) * 128, 1024) > 1
+    compare(got, cfg, weights, prompts, TOL["bfloat16"])
+
+
+def ops_library():
+    from lucciola_amd.kernels import ops
+    return ops.library()

@@ -684,3 +684,48 @@ def test_attention_decode_of_many_requests_of_unequal_length(nh, nkv, d, window)
                                                    batch.block_table.cpu()),
                          kc.cpu(), vc.cpu(), nh, nkv, d, 16, d ** -0.5, window)
     close(got, want, torch.bfloat16, atol=attention_atol(torch.bfloat16, vc))
+
+
+@pytest.mark.parametrize("nh,nkv,window,rot,normed,count", [(32, 8, 0, 128, True, 5), (12, 4, 40, 128, True, 1),
+                                                            (4, 4, 0, 0, False, 3), (16, 2, 0, 128, False, 8)])
+def test_attention_decode_takes_q_k_v_as_shares_of_a_product(nh, nkv, window, rot, normed, count):
+    """A step of single tokens whose q/k/v product was cut along K: the decode kernel sums the
+    float32 shares as it reads them.  Output and caches equal, to the bit, those of summing the
+    shares first (in their order, rounded to bfloat16) and handing the kernel the sum."""
+    d = 128
+    lengths = [1, 16, 17, 300, 2049, 5000, 33]
+    T = len(lengths)
+    _, batch, kc, vc = paged_case(lengths, [1] * T, nh, nkv, d, 16, torch.bfloat16, seed=97)
+    width = (nh + 2 * nkv) * d
+    partials = rnd(count, T, width, seed=98, scale=count ** -0.5)
+    shares = ops.ProductShares(partials, torch.bfloat16)
+    summed = shares.value()
+    plain = torch.zeros(T, width, device=DEV)
+    for s in range(count):
+        plain += partials[s]
+    assert torch.equal(summed, plain.to(torch.bfloat16))
+    qw = (1 + 0.1 * rnd(d, seed=91)) if normed else None
+    kw = (1 + 0.1 * rnd(d, seed=92)) if normed else None
+    table = make_rope_table(6000, rot, 10000.0) if rot else None
+    slots = torch.tensor([int(batch.block_table[r, (n - 1) // 16]) * 16 + (n - 1) % 16
+                          for r, n in enumerate(lengths)], dtype=torch.int32, device=DEV)
+    assert ops.attention_takes_shares(batch, T, nh, nkv, d, 16, torch.bfloat16, rot)
+    kc1, vc1 = kc.clone(), vc.clone()
+    want = ops.attention(summed.clone(), batch, kc1, vc1, nh, nkv, d, 16, d ** -0.5, window,
+                         ops.QKPrologue(qw, kw, 1e-6, table, slots))
+    kc2, vc2 = kc.clone(), vc.clone()
+    got = ops.attention(shares, batch, kc2, vc2, nh, nkv, d, 16, d ** -0.5, window,
+                        ops.QKPrologue(qw, kw, 1e-6, table, slots))
+    assert torch.equal(got, want)
+    assert torch.equal(kc2, kc1) and torch.equal(vc2, vc1)
+    # where the kernel cannot (a prompt portion in the step), the shares are summed first
+    _, mixed, kc3, vc3 = paged_case([40, 9], [1, 4], nh, nkv, d, 16, torch.bfloat16, seed=99)
+    assert not ops.attention_takes_shares(mixed, 5, nh, nkv, d, 16, torch.bfloat16, rot)
+    part5 = rnd(2, 5, width, seed=100)
+    slots5 = torch.tensor([int(mixed.block_table[0, 2]) * 16 + 7] +
+                          [int(mixed.block_table[1, 0]) * 16 + i for i in range(5, 9)], dtype=torch.int32, device=DEV)
+    a = ops.attention(ops.ProductShares(part5, torch.bfloat16), mixed, kc3.clone(), vc3.clone(), nh, nkv, d, 16,
+                      d ** -0.5, window, ops.QKPrologue(qw, kw, 1e-6, table, slots5))
+    b = ops.attention(ops.ProductShares(part5, torch.bfloat16).value(), mixed, kc3.clone(), vc3.clone(), nh, nkv, d,
+                      16, d ** -0.5, window, ops.QKPrologue(qw, kw, 1e-6, table, slots5))
+    assert torch.equal(a, b)
