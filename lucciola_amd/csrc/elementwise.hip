@@ -101,8 +101,11 @@ template <> struct Pack8<bf16> {
 
 constexpr int RN_THREADS = 256, RN_CHUNKS = 4;   // 256 threads x 4 chunks x 8 entries = 8192
 
-template <typename T>
-__global__ __launch_bounds__(RN_THREADS) void rmsnorm_vec_kernel(
+// THREADS x CHUNKS x 8 entries at most.  Few rows (a decode step) leave most CUs without a
+// workgroup, and the ones that have one are bound by what its waves keep in flight: 1024 threads
+// with one chunk each then, 256 with four for many rows.
+template <typename T, int THREADS, int CHUNKS>
+__global__ __launch_bounds__(THREADS) void rmsnorm_vec_kernel(
     float* __restrict__ h, const T* __restrict__ delta, const int* __restrict__ rows,
     const float* __restrict__ w, float eps, T* __restrict__ out, int n, int write_h,
     float* __restrict__ sumsq, int shares, size_t share_stride) {
@@ -113,11 +116,11 @@ __global__ __launch_bounds__(RN_THREADS) void rmsnorm_vec_kernel(
     const T* dr = (delta && !shares) ? delta + (size_t)src * n : nullptr;
     const float* pr = shares ? reinterpret_cast<const float*>(delta) + (size_t)src * n : nullptr;
     const int chunks = n / 8;
-    Pack8<float> hv[RN_CHUNKS];
-    Pack8<T> dv[RN_CHUNKS];
+    Pack8<float> hv[CHUNKS];
+    Pack8<T> dv[CHUNKS];
 #pragma unroll
-    for (int c = 0; c < RN_CHUNKS; ++c) {
-        const int chunk = threadIdx.x + c * RN_THREADS;
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int chunk = threadIdx.x + c * THREADS;
         if (chunk < chunks) {
             hv[c] = *reinterpret_cast<const Pack8<float>*>(hr + chunk * 8);
             if (dr) dv[c] = *reinterpret_cast<const Pack8<T>*>(dr + chunk * 8);
@@ -125,8 +128,8 @@ __global__ __launch_bounds__(RN_THREADS) void rmsnorm_vec_kernel(
     }
     if (pr) {   // the shares of the branch's product, in their order, then the stream
 #pragma unroll
-        for (int c = 0; c < RN_CHUNKS; ++c) {
-            const int chunk = threadIdx.x + c * RN_THREADS;
+        for (int c = 0; c < CHUNKS; ++c) {
+            const int chunk = threadIdx.x + c * THREADS;
             if (chunk < chunks) {
                 Pack8<float> sum = *reinterpret_cast<const Pack8<float>*>(pr + chunk * 8);
                 for (int s = 1; s < shares; ++s) {
@@ -141,8 +144,8 @@ __global__ __launch_bounds__(RN_THREADS) void rmsnorm_vec_kernel(
     }
     float ss = 0.f;
 #pragma unroll
-    for (int c = 0; c < RN_CHUNKS; ++c) {
-        const int chunk = threadIdx.x + c * RN_THREADS;
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int chunk = threadIdx.x + c * THREADS;
         if (chunk < chunks) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -159,8 +162,8 @@ __global__ __launch_bounds__(RN_THREADS) void rmsnorm_vec_kernel(
     if (sumsq && threadIdx.x == 0) sumsq[r] = ss;
     T* o = out + (size_t)r * n;
 #pragma unroll
-    for (int c = 0; c < RN_CHUNKS; ++c) {
-        const int chunk = threadIdx.x + c * RN_THREADS;
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int chunk = threadIdx.x + c * THREADS;
         if (chunk < chunks) {
             const Pack8<float> wv = *reinterpret_cast<const Pack8<float>*>(w + chunk * 8);
             Pack8<T> ov;
@@ -407,16 +410,23 @@ LC_API int lc_rmsnorm(float* h, const void* delta, const int* rows, const float*
     const bool vec = n % 8 == 0 && n >= 512 && n <= RN_THREADS * RN_CHUNKS * 8 &&
                      (uintptr_t)h % 16 == 0 && (uintptr_t)delta % 16 == 0 && (uintptr_t)out % 16 == 0 &&
                      (uintptr_t)w % 16 == 0;
+    const bool few = R <= 128 && n > 2048 && n <= 8192;
     if (dt == DT_F32) {
-        if (vec)
-            rmsnorm_vec_kernel<float><<<R, RN_THREADS, 0, stream>>>(h, (const float*)delta, rows, w, eps,
+        if (vec && few)
+            rmsnorm_vec_kernel<float, 1024, 1><<<R, 1024, 0, stream>>>(h, (const float*)delta, rows, w, eps,
+                                                                       (float*)out, n, write_h, sumsq, shares, share_stride);
+        else if (vec)
+            rmsnorm_vec_kernel<float, RN_THREADS, RN_CHUNKS><<<R, RN_THREADS, 0, stream>>>(h, (const float*)delta, rows, w, eps,
                                                                     (float*)out, n, write_h, sumsq, shares, share_stride);
         else
             rmsnorm_kernel<float><<<R, threads, 0, stream>>>(h, (const float*)delta, rows, w, eps,
                                                              (float*)out, n, write_h, sumsq, shares, share_stride);
     } else if (dt == DT_BF16) {
-        if (vec)
-            rmsnorm_vec_kernel<bf16><<<R, RN_THREADS, 0, stream>>>(h, (const bf16*)delta, rows, w, eps,
+        if (vec && few)
+            rmsnorm_vec_kernel<bf16, 1024, 1><<<R, 1024, 0, stream>>>(h, (const bf16*)delta, rows, w, eps,
+                                                                      (bf16*)out, n, write_h, sumsq, shares, share_stride);
+        else if (vec)
+            rmsnorm_vec_kernel<bf16, RN_THREADS, RN_CHUNKS><<<R, RN_THREADS, 0, stream>>>(h, (const bf16*)delta, rows, w, eps,
                                                                    (bf16*)out, n, write_h, sumsq, shares, share_stride);
         else
             rmsnorm_kernel<bf16><<<R, threads, 0, stream>>>(h, (const bf16*)delta, rows, w, eps,
