@@ -1,10 +1,12 @@
 """A plain, slow implementation of the Qwen3 dense decoder: whole sequences, no cache, one
 function for each part, float64 on the CPU.  Written from the formulas of the reference's
-kernels (each function cites file:line of /root/reference); it shares no code with the
+kernels (each function cites file:line of the reference's tree); it shares no code with the
 engine under ``lucciola_amd`` and is what the engine is compared with.
 """
+import hashlib
 import math
 
+import numpy as np
 import torch
 
 F64 = torch.float64
@@ -178,3 +180,35 @@ def sample_token(logits, temperature, u):
     p = torch.exp(z - z.max())
     cdf = torch.cumsum(p, 0)
     return int(torch.searchsorted(cdf, torch.tensor(u, dtype=F64) * cdf[-1], right=True).clamp(max=len(p) - 1))
+
+
+def random_weight(seed, name, shape, std, plus_one=False):
+    """The engine's random weights, computed again in numpy (the reference has no random
+    weights, src/qwen.cc:69-84; the recipe is the engine's own and is written out here from
+    its description, not from its code): a value depends on (seed, tensor name, element
+    index) only.  key = mix(seed xor first 8 bytes of sha256(name), little-endian);
+    h_j = mix(key + (3 i + j + 1) * G) for j = 0..2; z = (sum of the twelve 16-bit fields of
+    the h_j - 6 * 65535) / 65536; value = float32(z * std) (+ 1), mix being splitmix64's
+    finaliser and G its increment.  Returns float32."""
+    G, M1, M2 = np.uint64(0x9E3779B97F4A7C15), np.uint64(0xBF58476D1CE4E5B9), np.uint64(0x94D049BB133111EB)
+
+    def mix(x):
+        x = x + G
+        x = (x ^ (x >> np.uint64(30))) * M1
+        x = (x ^ (x >> np.uint64(27))) * M2
+        return x ^ (x >> np.uint64(31))
+
+    with np.errstate(over="ignore"):
+        start = (int(seed) % (1 << 64)) ^ int.from_bytes(hashlib.sha256(name.encode()).digest()[:8], "little")
+        key = mix(np.array([start], dtype=np.uint64))[0]
+        count = int(np.prod(shape)) if len(shape) else 1
+        i = np.arange(count, dtype=np.uint64)
+        total = np.zeros(count, dtype=np.int64)
+        for j in (1, 2, 3):
+            h = mix(key + (i * np.uint64(3) + np.uint64(j)) * G)
+            for shift in (0, 16, 32, 48):
+                total += ((h >> np.uint64(shift)) & np.uint64(0xFFFF)).astype(np.int64)
+    z = ((total - 6 * 65535).astype(np.float32) / np.float32(65536.0)) * np.float32(std)
+    if plus_one:
+        z = z + np.float32(1.0)
+    return z.astype(np.float32).reshape(shape)

@@ -4,10 +4,12 @@ import json
 import os
 import struct
 
+import numpy as np
 import pytest
 import torch
 
 import configs
+import plain_qwen3
 from lucciola_amd import models  # noqa: F401
 from lucciola_amd.config.registry import architecture_for
 from lucciola_amd.engine.loading import load_model
@@ -142,6 +144,57 @@ def test_random_model_folder(tmp_path, key):
     model, config = load_model(folder, "float32", "cpu")
     assert len(model.layers) == cfg["num_hidden_layers"]
     assert (model.head is model.embedding) == cfg["tie_word_embeddings"]
+
+
+@pytest.mark.parametrize("key", ["A", "C"])
+def test_random_weights_are_a_function_of_seed_name_and_index(key):
+    """Every value again from the written recipe, in numpy: bit for bit."""
+    cfg, _, seed = configs.ALL[key]
+    arch = architecture_for(cfg)
+    declared = declared_tensors(arch.model_spec(arch.read_config(cfg)))
+    std = cfg["initializer_range"]
+    for name, t in random_tensors(declared, seed, std, torch.float32):
+        again = plain_qwen3.random_weight(seed, name, declared[name].shape, std,
+                                          plus_one=declared[name].init == "ones_plus_normal")
+        assert t.dtype == torch.float32 and np.array_equal(t.numpy(), again), name
+    # rounded once to bfloat16; a value does not depend on how many come before or after it
+    name = "model.layers.1.mlp.down_proj.weight"
+    whole = dict(random_tensors({name: declared[name]}, seed, std, torch.bfloat16))[name]
+    assert torch.equal(whole, torch.from_numpy(
+        plain_qwen3.random_weight(seed, name, declared[name].shape, std)).to(torch.bfloat16))
+    from lucciola_amd.weights.random_init import tensor_key, unit_normal
+    part = unit_normal(tensor_key(seed, name), 1000, 50, "cpu") * torch.tensor(std)
+    assert torch.equal(part.to(torch.bfloat16), whole.reshape(-1)[1000:1050])
+    # twelve uniform numbers less six: unit variance, nothing beyond six
+    z = unit_normal(tensor_key(seed, "any"), 0, 1 << 18, "cpu")
+    assert abs(float(z.mean())) < 0.01 and abs(float(z.std()) - 1) < 0.01 and float(z.abs().max()) <= 6
+
+
+@pytest.mark.gpu
+def test_random_weights_do_not_depend_on_the_device(tmp_path):
+    """A model made on the GPU from (configuration, seed) holds the tensors of the folder
+    written on the CPU from the same two."""
+    from lucciola_amd.engine.loading import random_model
+    cfg, _, seed = configs.ALL["B"]
+    folder = write_model_folder(str(tmp_path / "m"), cfg, seed)
+    arch = architecture_for(cfg)
+    declared = declared_tensors(arch.model_spec(arch.read_config(cfg)))
+    on_gpu = dict(random_tensors(declared, seed, cfg["initializer_range"], torch.bfloat16, device="cuda:0"))
+    as_f32 = dict(random_tensors(declared, seed, cfg["initializer_range"], torch.float32, device="cuda:0"))
+    with SafetensorsFile(os.path.join(folder, "model.safetensors")) as f:
+        for name in declared:
+            assert torch.equal(f.get(name), on_gpu[name].cpu()), name
+            assert np.array_equal(as_f32[name].cpu().numpy(), plain_qwen3.random_weight(
+                seed, name, declared[name].shape, cfg["initializer_range"],
+                plus_one=declared[name].init == "ones_plus_normal")), name
+    made, _ = random_model(cfg, seed, "bfloat16", "cuda:0")
+    loaded, _ = load_model(folder, "bfloat16", "cuda:0")
+    assert torch.equal(made.embedding, loaded.embedding) and torch.equal(made.head, loaded.head)
+    for a, b in zip(made.layers, loaded.layers):
+        assert torch.equal(a.mixer.qkv, b.mixer.qkv) and torch.equal(a.mixer.o, b.mixer.o)
+        assert torch.equal(a.feed_forward.gate_up, b.feed_forward.gate_up)
+        assert torch.equal(a.feed_forward.down, b.feed_forward.down)
+        assert torch.equal(a.mixer_norm.weight, b.mixer_norm.weight)
 
 
 def test_folder_with_wrong_weights(tmp_path):
