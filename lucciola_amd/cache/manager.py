@@ -89,6 +89,17 @@ class CacheManager:
             total += len(g.sites) * 2 * g.spec.num_kv_heads * self.block_size * g.spec.head_dim * size
         return total
 
+    def state_bytes(self) -> int:
+        """Bytes of the per-request state tensors of all state sites."""
+        total = 0
+        for site in self.state_sites:
+            spec = self.site_specs[site]
+            count = self.max_seqs
+            for n in spec.shape:
+                count *= int(n)
+            total += count * torch.empty((), dtype=spec.dtype).element_size()
+        return total
+
     def allocate_tensors(self, dtype: torch.dtype, device) -> None:
         """Per paged site: keys [num_blocks, kv_heads, block_size, head_dim] and values
         [num_blocks, kv_heads, head_dim, block_size] (transposed inside a page);
@@ -156,6 +167,19 @@ class CacheManager:
             need = self.pages_needed(g, have, new_tokens)
             g.tables[request].extend(g.pool.allocate_many(need))
         st.pending += new_tokens
+
+    def cancel(self, request: Hashable) -> None:
+        """The reserved tokens will not be written after all: the pages taken for them go
+        back."""
+        st = self.requests[request]
+        keep = _ceil_div(st.length, self.block_size)
+        for g in self.groups:
+            table = g.tables[request]
+            while len(table) > keep:
+                page = table.pop()
+                if page >= 0:
+                    g.pool.free(page)
+        st.pending = 0
 
     def commit(self, request: Hashable) -> None:
         """The reserved tokens have been written.  Pages that a window has passed go back."""

@@ -410,7 +410,9 @@ LC_API int lc_rmsnorm(float* h, const void* delta, const int* rows, const float*
     const bool vec = n % 8 == 0 && n >= 512 && n <= RN_THREADS * RN_CHUNKS * 8 &&
                      (uintptr_t)h % 16 == 0 && (uintptr_t)delta % 16 == 0 && (uintptr_t)out % 16 == 0 &&
                      (uintptr_t)w % 16 == 0;
-    const bool few = R <= 128 && n > 2048 && n <= 8192;
+    // float32 results must not depend on how many rows share a step: there the shape of the
+    // kernel, and with it the grouping of a row's sum of squares, follows from n alone
+    const bool few = dt == DT_BF16 && R <= 128 && n > 2048 && n <= 8192;
     if (dt == DT_F32) {
         if (vec && few)
             rmsnorm_vec_kernel<float, 1024, 1><<<R, 1024, 0, stream>>>(h, (const float*)delta, rows, w, eps,

@@ -125,7 +125,11 @@ class LLMEngine:
         carry = None
         if before is not None and before.sampled is not None:
             carry = Carry(before.sampled.ids, {s.seq_id: row for row, s in enumerate(before.seqs)})
-        logits = self.runner.step(sched.entries, carry)
+        try:
+            logits = self.runner.step(sched.entries, carry)
+        except BaseException:
+            self.scheduler.undo(sched)      # the runner has put the cache back as it was
+            raise
         sampling = [seq for seq, s in zip(sched.seqs, sched.samples) if s]
         if not sampling:
             return _QueuedStep(None, [], [], [])

@@ -26,6 +26,26 @@ class _CapturedStep:
         self.graph, self.batch, self.sites, self.logits = graph, batch, sites, logits
 
 
+def blocks_from_free_memory(free: int, bytes_per_block: int, state_bytes: int,
+                            config: EngineConfig, max_positions: int = 0) -> int:
+    """Pages for the cache when none are asked for, as the reference sizes its pools
+    (src/qwen.cc:527-543): ``memory_fraction`` of the free memory less a reserve, divided by
+    what a page costs over all layers.  Beyond the reference: the per-request state tensors
+    come off first, and the count is capped at what ``max_seqs`` requests of the model's
+    longest context can hold and at what a 32-bit slot id (page * block_size + offset) can
+    name."""
+    per_block = max(1, int(bytes_per_block))
+    usable = int(max(0, free - config.memory_reserve) * config.memory_fraction) - int(state_bytes)
+    blocks = usable // per_block
+    if blocks <= 0:
+        raise RuntimeError(f"no memory for the cache: {free} bytes free, a page of all "
+                           f"layers takes {per_block}")
+    blocks = min(blocks, (2 ** 31 - 1) // config.block_size)
+    if max_positions:
+        blocks = min(blocks, config.max_seqs * -(-max_positions // config.block_size))
+    return int(blocks)
+
+
 class ModelRunner:
     def __init__(self, model: CausalLM, config: EngineConfig, num_blocks: Optional[int] = None):
         self.model = model
@@ -48,17 +68,11 @@ class ModelRunner:
 
     # ------------------------------------------------------------------ sizing
     def _blocks_from_free_memory(self, needs) -> int:
-        """As the reference sizes its pools: a fraction of the free memory less a reserve
-        (src/qwen.cc:527-543)."""
-        probe = CacheManager(needs, self.config.block_size, 1, 1)
-        per_block = max(1, probe.bytes_per_block(self.config.dtype))
+        probe = CacheManager(needs, self.config.block_size, 1, self.config.max_seqs)
         free, _ = torch.cuda.mem_get_info(self.device)
-        usable = int((free - self.config.memory_reserve) * self.config.memory_fraction)
-        blocks = usable // per_block
-        if blocks <= 0:
-            raise RuntimeError(f"no memory for the cache: {free} bytes free, a page of all "
-                               f"layers takes {per_block}")
-        return int(blocks)
+        return blocks_from_free_memory(
+            free, probe.bytes_per_block(self.config.dtype), probe.state_bytes(), self.config,
+            self.model.spec.max_positions)
 
     # ------------------------------------------------------------------ the step
     def can_run(self, entries: Sequence[StepEntry]) -> bool:
@@ -84,8 +98,9 @@ class ModelRunner:
         that ``carry`` holds for its request, on the device: a caller may queue a request's
         next step before it has seen the token that the last one sampled.
 
-        A request that the cache does not know is admitted.  Raises OutOfPages (and changes
-        nothing) if the pages or slots for the whole batch are not there."""
+        A request that the cache does not know is admitted.  Raises OutOfPages if the pages or
+        slots for the whole batch are not there.  Whatever is raised, by the checks or by the
+        model, the cache's bookkeeping is left as it was before the call."""
         entries = [e for e in entries if len(e.tokens) > 0]
         V = self.model.vocab_size
         if not entries:
@@ -120,25 +135,38 @@ class ModelRunner:
                              f" tokens of {len(entries)} requests; "
                              f"{self.cache.num_free_blocks()} pages free)")
         fresh: List[int] = []
-        for e in entries:
-            if not self.cache.has(e.request):
-                self.cache.admit(e.request)
-            if self.cache.length(e.request) == 0:
-                fresh.append(self.cache.slot(e.request))
-            self.cache.reserve(e.request, len(e.tokens))
-        for site, state in self.cache.state.items():
-            for slot in fresh:
-                state[slot].zero_()
+        admitted: List[Hashable] = []
+        try:
+            for e in entries:
+                if not self.cache.has(e.request):
+                    self.cache.admit(e.request)
+                    admitted.append(e.request)
+                if self.cache.length(e.request) == 0:
+                    fresh.append(self.cache.slot(e.request))
+                self.cache.reserve(e.request, len(e.tokens))
+            for site, state in self.cache.state.items():
+                for slot in fresh:
+                    state[slot].zero_()
 
-        if self.use_graphs and len(entries) <= self.config.graph_max_batch and all(
-                len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
-            logits, num_tokens = self._graph_step(entries, carry if fed else None), len(entries)
-        else:
-            batch = build_batch(entries, self.cache, self.device,
-                                carry_rows=carry.rows if fed else None)
-            if fed:
-                ops.feed_tokens(batch.token_ids, batch.feed, carry.ids)
-            logits, num_tokens = self.model.forward(batch, self._sites(batch)), batch.num_tokens
+            if self.use_graphs and len(entries) <= self.config.graph_max_batch and all(
+                    len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+                logits, num_tokens = self._graph_step(entries, carry if fed else None), len(entries)
+            else:
+                batch = build_batch(entries, self.cache, self.device,
+                                    carry_rows=carry.rows if fed else None)
+                if fed:
+                    ops.feed_tokens(batch.token_ids, batch.feed, carry.ids)
+                logits, num_tokens = self.model.forward(batch, self._sites(batch)), batch.num_tokens
+        except BaseException:
+            # nothing of this step counts: reserved pages go back, requests that it admitted
+            # leave again (what kernels may already have written lies beyond every length)
+            for e in entries:
+                if self.cache.has(e.request):
+                    if e.request in admitted:
+                        self.cache.release(e.request)
+                    else:
+                        self.cache.cancel(e.request)
+            raise
         for e in entries:
             self.cache.commit(e.request)
         self.steps += 1

@@ -37,6 +37,7 @@ class ScheduledStep:
     entries: List[StepEntry] = field(default_factory=list)
     seqs: List[Sequence] = field(default_factory=list)
     samples: List[bool] = field(default_factory=list)   # does this entry yield a new token
+    portions: List[int] = field(default_factory=list)   # prompt tokens fed by this entry (0: a decode)
     num_decode_seqs: int = 0
     num_prefill_seqs: int = 0
     num_prefill_tokens: int = 0
@@ -147,6 +148,7 @@ class Scheduler:
             out.entries.append(StepEntry(seq.seq_id, [seq.token_ids[-1]], [0]))
             out.seqs.append(seq)
             out.samples.append(True)
+            out.portions.append(0)
             out.num_decode_seqs += 1
             budget -= 1
 
@@ -180,6 +182,7 @@ class Scheduler:
             out.entries.append(StepEntry(seq.seq_id, tokens, [chunk - 1] if last else []))
             out.seqs.append(seq)
             out.samples.append(last)
+            out.portions.append(chunk)
             out.num_prefill_seqs += 1
             out.num_prefill_tokens += chunk
             seq.prefill_offset += chunk
@@ -191,6 +194,19 @@ class Scheduler:
             else:
                 break   # the budget or the pages are used up
         return out
+
+    def undo(self, step: ScheduledStep) -> None:
+        """The step was not run: its prompt portions are waiting again, in their order.
+        Requests that the step preempted stay preempted (they hold nothing, which is a state
+        like any other)."""
+        for seq, chunk, last in reversed(list(zip(step.seqs, step.portions, step.samples))):
+            if chunk == 0:
+                continue
+            seq.prefill_offset -= chunk
+            if last:
+                self.running.remove(seq)
+                self.waiting.appendleft(seq)
+                seq.status = SequenceStatus.WAITING
 
     def on_token(self, seq: Sequence, token: int) -> bool:
         """Record a generated token; returns True if the request has finished."""

@@ -15,11 +15,14 @@ from lucciola_amd.weights.loader import DictSource
 from lucciola_amd.weights.random_init import random_tensors
 
 
-def random_weights(cfg, seed, std=None, dtype=torch.bfloat16):
+def random_weights(cfg, seed, std=None, dtype=torch.bfloat16, device="cpu"):
+    """The random weights of (cfg, seed); made on ``device`` (the values are the same on every
+    device), returned on the CPU."""
     arch = architecture_for(cfg)
     spec = arch.model_spec(arch.read_config(cfg))
-    return dict(random_tensors(declared_tensors(spec), seed,
-                               cfg["initializer_range"] if std is None else std, dtype))
+    return {name: t.cpu() for name, t in random_tensors(
+        declared_tensors(spec), seed, cfg["initializer_range"] if std is None else std, dtype,
+        device=device)}
 
 
 def make_runner(cfg, weights, page, blocks, dtype, device, max_seqs=4):

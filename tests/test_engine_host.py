@@ -174,3 +174,63 @@ def test_a_request_is_ended_early_and_gives_everything_back(monkeypatch, ahead):
     for g in engine.runner.cache.groups:
         assert g.pool.num_free() == 40
     assert not engine.abort_request(12345)
+
+
+def test_a_step_that_raises_leaves_the_cache_and_the_queues_as_they_were(monkeypatch):
+    """The model raises in the middle of a step (a kernel error, say): pages reserved for the
+    step go back, a request that the step admitted leaves again, the scheduler's portions are
+    waiting again, and the same work then runs to the plain implementation's tokens."""
+    from lucciola_amd.sampling.sampler import SamplingParams
+    reference_ops.install(monkeypatch)
+    cfg, page, seed = configs.ALL["A"]
+    weights = random_weights(cfg, seed, std=0.3)
+
+    # the runner alone: a known request beside a new one
+    runner = make_runner(cfg, weights, page, 16, "float32", "cpu")
+    runner.step([StepEntry("a", [3, 4, 5, 6, 7], [4])])
+    before = (runner.cache.length("a"), runner.cache.block_table(0, "a"), runner.cache.num_free_blocks())
+    real_forward = runner.model.forward
+    def broken(batch, sites):
+        raise RuntimeError("injected")
+    runner.model.forward = broken
+    with pytest.raises(RuntimeError, match="injected"):
+        runner.step([StepEntry("a", [8, 9, 10, 11, 12], [4]), StepEntry("b", [1, 2, 3], [2])])
+    runner.cache.check()
+    assert not runner.cache.has("b") and runner.cache.requests["a"].pending == 0
+    assert (runner.cache.length("a"), runner.cache.block_table(0, "a"), runner.cache.num_free_blocks()) == before
+    with pytest.raises(ValueError, match="outside its"):
+        runner.step([StepEntry("a", [8, 9], [5])])       # raised while the batch is laid out
+    runner.cache.check()
+    assert runner.cache.requests["a"].pending == 0 and runner.cache.num_free_blocks() == before[2]
+    runner.model.forward = real_forward
+    got = runner.step([StepEntry("a", [8, 9, 10, 11, 12], [4])])[0].double()
+    ref = plain_qwen3.forward(cfg, weights, [3, 4, 5, 6, 7, 8, 9, 10, 11, 12])[-1]
+    assert float((got - ref).abs().max() / ref.abs().max()) < 2e-5
+
+    # through the engine: the third step fails once, then everything goes on
+    prompts = list(prompts_for(cfg, [9, 20, 6], seed + 7).values())
+    engine = host_engine(cfg, weights, page, 40, max_tokens_per_step=12, max_seqs=3, run_ahead=False)
+    ids = [engine.add_request(p, SamplingParams(max_new_tokens=6)) for p in prompts]
+    real = engine.runner.model.forward
+    calls = {"n": 0}
+    def flaky(batch, sites):
+        calls["n"] += 1
+        if calls["n"] == 3:
+            raise RuntimeError("injected")
+        return real(batch, sites)
+    engine.runner.model.forward = flaky
+    seen = {i: [] for i in ids}
+    failures = 0
+    while engine.has_unfinished_requests():
+        try:
+            for out in engine.step():
+                seen[out.seq_id].append(out.token)
+        except RuntimeError:
+            failures += 1
+            engine.runner.cache.check()
+            assert all(st.pending == 0 for st in engine.runner.cache.requests.values())
+    assert failures == 1
+    for i, p in zip(ids, prompts):
+        assert seen[i] == plain_qwen3.greedy(cfg, weights, p, 6)
+    engine.runner.cache.check()
+    assert not engine.runner.cache.requests

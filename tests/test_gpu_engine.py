@@ -172,19 +172,41 @@ def test_greedy_generation_through_the_engine(key):
     assert not engine.runner.cache.requests
 
 
-def test_generation_survives_preemption():
-    """With so few pages that running requests are preempted and recomputed, the generated
-    tokens are those of an engine with plenty of pages."""
+@pytest.mark.parametrize("ahead", [False, True])
+def test_generation_survives_preemption(ahead):
+    """With so few pages that running requests are preempted and recomputed, every request's
+    tokens are those of the plain implementation (greedy ones, and the temperature draws too:
+    a draw depends on the request's seed and the token's index alone)."""
     cfg, page, seed = configs.ALL["A"]
     weights = random_weights(cfg, seed, std=0.3)
     prompts = list(prompts_for(cfg, [9, 14, 6, 11], seed + 40).values())
-    roomy = engine_for(cfg, weights, page, 200, "float32", max_tokens_per_step=12, max_seqs=4)
-    want = roomy.generate(prompts, SamplingParams(max_new_tokens=20))
-    tight = engine_for(cfg, weights, page, 18, "float32", max_tokens_per_step=12, max_seqs=4)
+    tight = engine_for(cfg, weights, page, 18, "float32", max_tokens_per_step=12, max_seqs=4,
+                       run_ahead=ahead)
     got = tight.generate(prompts, SamplingParams(max_new_tokens=20))
     assert tight.scheduler.num_preemptions > 0
-    assert got == want
+    for prompt, tokens in zip(prompts, got):
+        assert tokens == plain_qwen3.greedy(cfg, weights, prompt, 20)
     tight.runner.cache.check()
+    assert not tight.runner.cache.requests
+    params = [SamplingParams(max_new_tokens=20, temperature=0.7 if i % 2 else 0.0, seed=50 + i)
+              for i in range(4)]
+    got = tight.generate(prompts, params)
+    assert tight.scheduler.num_preemptions > 1
+    for prompt, p, tokens in zip(prompts, params, got):
+        check_sampled(cfg, weights, prompt, p, tokens)
+
+
+def check_sampled(cfg, weights, prompt, params, tokens):
+    """Every token of a request against the plain implementation's pick at its place."""
+    ids = list(prompt)
+    for i, tok in enumerate(tokens):
+        logits = plain_qwen3.forward(cfg, weights, ids)[-1]
+        want = plain_qwen3.sample_token(logits, params.temperature, uniform_for(params.seed, i))
+        if tok != want:   # only a rounding neighbour of the CDF boundary may differ
+            assert params.temperature > 0
+            pr = torch.softmax(logits / params.temperature, 0).cumsum(0)
+            assert abs(float(pr[min(tok, want)]) - uniform_for(params.seed, i)) < 1e-4
+        ids.append(tok)
 
 
 def test_temperature_sampling_through_the_engine():
@@ -314,8 +336,9 @@ def test_running_ahead_matches_waiting(dtype, key):
         if dtype == "bfloat16":
             assert engine.runner.graph_replays > 10
     assert got[True] == got[False]
-    if dtype == "float32":
-        assert got[True][0] == plain_qwen3.greedy(cfg, weights, prompts[0], 24)
+    if dtype == "float32":      # every request against the plain implementation
+        for prompt, p, tokens in zip(prompts, params, got[True]):
+            check_sampled(cfg, weights, prompt, p, tokens)
 
 
 @pytest.mark.parametrize("trial", range(8))
@@ -405,28 +428,137 @@ def test_command_line_and_async_engine(tmp_path):
     assert not engine.engine.runner.cache.requests
 
 
+_8B = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 4096,
+       "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+       "intermediate_size": 12288, "vocab_size": 151936, "rope_theta": 1000000.0,
+       "rms_norm_eps": 1e-6, "tie_word_embeddings": False, "max_position_embeddings": 40960,
+       "initializer_range": 0.02}
+
+
+def case_8b():
+    if "8b" not in _cache:
+        weights = random_weights(_8B, 11, device=DEV)
+        prompts = prompts_for(_8B, [150, 37], 12)
+        refs = {n: plain_qwen3.forward(_8B, weights, ids) for n, ids in prompts.items()}
+        _cache["8b"] = (weights, prompts, refs)
+    return _cache["8b"]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_layers_of_the_8b_size(dtype):
-    """Two layers with the sizes of the Qwen3-8B-shaped configuration (hidden 4096, 32 query and
-    8 kv heads of 128, feed-forward 12288; the vocabulary is cut to 2048 to keep the plain
-    float64 run short): the kernels chosen for real sizes (matrix-core products, vector norms,
-    matrix-core attention in bfloat16; FMA kernels in float32) against the plain implementation,
-    whole, in portions and token by token."""
-    cfg = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 4096,
-           "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
-           "intermediate_size": 12288, "vocab_size": 2048, "rope_theta": 1000000.0,
-           "rms_norm_eps": 1e-6, "tie_word_embeddings": False, "max_position_embeddings": 40960,
-           "initializer_range": 0.02}
-    weights = random_weights(cfg, 11)
-    prompts = prompts_for(cfg, [150, 37], 12)
-    refs = {n: plain_qwen3.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    """Two of the 36 layers of the Qwen3-8B-shaped configuration, every size as it is there
+    (hidden 4096, 32 query and 8 kv heads of 128, feed-forward 12288, the whole vocabulary of
+    151,936 with a head of its own; src/qwen.cc:875-882 is the head): the kernels chosen for
+    real sizes (matrix-core products, vector norms, matrix-core attention in bfloat16; FMA
+    kernels in float32) against the plain implementation, whole, in portions and token by
+    token."""
+    weights, prompts, refs = case_8b()
     for family in (traces.whole, lambda p: traces.chunked(p, sizes=(70, 2, 33, 5)),
                    lambda p: traces.tail_decode(p, tail=8)):
         steps = family(prompts)
-        runner = make_runner(cfg, weights, 16, traces.max_live_tokens(steps, 16) // 16, dtype, DEV)
+        runner = make_runner(_8B, weights, 16, traces.max_live_tokens(steps, 16) // 16, dtype, DEV)
         got = replay(runner, steps)
-        worst = compare(got, cfg, weights, prompts, TOL[dtype], refs)
+        assert len(got) == 187 and next(iter(got.values())).shape[0] == 151936
+        worst = compare(got, _8B, weights, prompts, TOL[dtype], refs)
         print(f"8B-size layers {dtype}: worst relative error {worst:.3e}")
+        del runner
+
+
+def test_float32_logits_do_not_depend_on_the_cut():
+    """In float32 the logits at a position are the same bits however the tokens are cut into
+    steps, whatever else is in the batch, whichever pages are used and whatever the page size
+    is: every reduction's order is a function of the row alone.  At the 8B-shaped sizes (norm
+    rows of 4096, where the kernel's shape once depended on the number of rows) and at tiny C."""
+    for cfg, weights, page, lengths in ((_8B, case_8b()[0], 16, [90, 37, 20]),
+                                        (configs.TINY_C, random_weights(configs.TINY_C, 2), 16, [70, 33, 50])):
+        prompts = prompts_for(cfg, lengths, 77)
+        results = []
+        for family, pg, shuffle in ((traces.whole, page, False),
+                                    (lambda p: traces.chunked(p, sizes=(7, 2, 16, 3, 33)), page, True),
+                                    (lambda p: traces.tail_decode(p, tail=6), page, False),
+                                    (lambda p: traces.mixed(p, seed=3, decode_tail=4), page, True),
+                                    (traces.whole, 4, True)):
+            steps = family(prompts)
+            blocks = traces.max_live_tokens(steps, 64) // pg + 7
+            runner = make_runner(cfg, weights, pg, blocks, "float32", DEV)
+            if shuffle:     # other pages, in another order
+                import random
+                for g in runner.cache.groups:
+                    order = list(g.pool._free)
+                    random.Random(5).shuffle(order)
+                    g.pool._free.clear()
+                    g.pool._free.extend(order)
+            got = replay(runner, steps)
+            results.append({k: v.float() for k, v in got.items()})
+            del runner
+        for other in results[1:]:
+            assert other.keys() == results[0].keys()
+            for place, row in results[0].items():
+                assert torch.equal(row, other[place]), f"logits at {place} differ between cuts"
+
+
+def test_cache_sized_from_free_memory():
+    """``max_blocks=0`` (the default of the command line and of AsyncEngine): the page count is
+    the reference's (src/qwen.cc:527-543: a share of the free memory less 500 MiB over the bytes
+    of a page in all layers), capped at what max_seqs requests of the longest context hold."""
+    cfg, page, seed = configs.ALL["A"]
+    weights = random_weights(cfg, seed, std=0.3)
+    arch = architecture_for(cfg)
+    config = arch.read_config(cfg)
+    model = _build(arch.model_spec(config), DictSource(weights), "float32", DEV)
+    torch.cuda.synchronize()
+    per_page = 2 * cfg["num_hidden_layers"] * cfg["num_key_value_heads"] * cfg["head_dim"] * 4 * page
+    for fraction in (2e-6, 0.5):
+        free, _ = torch.cuda.mem_get_info(DEV)
+        engine = LLMEngine(model, config, EngineConfig(dtype="float32", block_size=page, max_blocks=0,
+                                                       memory_fraction=fraction, device=DEV, max_seqs=4,
+                                                       max_tokens_per_step=16))
+        by_memory = int((free - (500 << 20)) * fraction) // per_page
+        cap = 4 * (cfg["max_position_embeddings"] // page)
+        assert engine.runner.cache.num_blocks == min(by_memory, cap)
+        assert (by_memory < cap) == (fraction < 0.1) and by_memory > 20
+        assert engine.runner.cache.kv[0][0].shape[0] == engine.runner.cache.num_blocks
+        prompts = list(prompts_for(cfg, [5, 11, 17], seed + 30).values())
+        got = engine.generate(prompts, SamplingParams(max_new_tokens=8))
+        assert got == [plain_qwen3.greedy(cfg, weights, p, 8) for p in prompts]
+        del engine
+
+
+def test_position_table_grows_under_captured_steps():
+    """Decode steps replayed from graphs while the rotary table is made anew because a
+    position beyond it shows up (a real model's table starts at 16,384 rows; here at 256, so
+    that a short run crosses its end twice): logits on both sides of the crossings against
+    the plain implementation."""
+    from dataclasses import replace
+    cfg, page, seed = configs.ALL["D"]
+    weights = random_weights(cfg, seed)
+    arch = architecture_for(cfg)
+    config = arch.read_config(cfg)
+    spec = arch.model_spec(config)
+    layers = []
+    for layer in spec.layers:
+        position = layer.mixer.params["position"]
+        assert position.params["max_positions"] >= 2048
+        layers.append(replace(layer, mixer=layer.mixer.with_params(
+            position=position.with_params(max_positions=0, theta=position.params["theta"] + 1))))
+    spec = replace(spec, layers=layers)     # theta + 1: a table of its own, not another test's
+    cfg = dict(cfg, rope_theta=cfg["rope_theta"] + 1)
+    model = _build(spec, DictSource(weights), "bfloat16", DEV)
+    from lucciola_amd.engine.runner import ModelRunner
+    runner = ModelRunner(model, EngineConfig(dtype="bfloat16", block_size=page, max_blocks=80,
+                                             max_seqs=4, device=DEV))
+    prompts = prompts_for(cfg, [600, 530], seed + 3)
+    refs = {n: plain_qwen3.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    steps = [([(n, ids[:200], []) for n, ids in prompts.items()], [])]
+    for i in range(200, 600):
+        entries = [(n, [ids[i]], [0]) for n, ids in prompts.items() if i < len(ids)]
+        steps.append((entries, []))
+    position = model.layers[0].mixer.position
+    assert position.capacity() == 0
+    got = replay(runner, steps)
+    assert position.capacity() >= 600 and position.generation >= 3
+    assert runner.graph_replays > 300
+    compare(got, cfg, weights, prompts, TOL["bfloat16"], refs)
 
 
 @pytest.mark.parametrize("requests", [20, 40])

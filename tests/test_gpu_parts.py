@@ -309,6 +309,42 @@ def test_toy_architecture_with_a_stateful_mixer():
         ARCHITECTURES.unregister("ToyForCausalLM")
 
 
+def test_toy_architecture_through_the_engine_with_preemption():
+    """The toy model (state slots beside pages) through LLMEngine and the scheduler, with so few
+    pages that running requests are preempted and fed again: a preempted request's state
+    starts from zero again, and every request's tokens are the plain implementation's."""
+    from lucciola_amd.engine.llm_engine import LLMEngine
+    from lucciola_amd.sampling.sampler import SamplingParams
+    MIXERS.register("toy_decay", ToyDecay, replace=True)
+    FEED_FORWARDS.register("toy_scale", ToyScale, replace=True)
+    ARCHITECTURES.register("ToyForCausalLM", Architecture("ToyForCausalLM", read_config=dict,
+                                                          model_spec=toy_spec), replace=True)
+    try:
+        spec = toy_spec(TOY)
+        weights = dict(random_tensors(declared_tensors(spec), 5, 0.6, torch.float32))
+        model = _build(spec, DictSource(weights), "float32", "cuda:0")
+        prompts = list(prompts_for({"vocab_size": 50}, [9, 14, 6, 11], 8).values())
+        for ahead in (False, True):
+            engine = LLMEngine(model, TOY, EngineConfig(dtype="float32", block_size=4, max_blocks=18,
+                                                        max_seqs=4, max_tokens_per_step=12,
+                                                        device="cuda:0", run_ahead=ahead))
+            for state in engine.runner.cache.state.values():
+                state.fill_(3.0)
+            got = engine.generate(prompts, SamplingParams(max_new_tokens=20))
+            assert engine.scheduler.num_preemptions > 0
+            for prompt, tokens in zip(prompts, got):
+                ids = list(prompt)
+                for tok in tokens:
+                    assert tok == int(torch.argmax(toy_plain(TOY, weights, ids)[-1]))
+                    ids.append(tok)
+            engine.runner.cache.check()
+            assert not engine.runner.cache.requests
+    finally:
+        MIXERS.unregister("toy_decay")
+        FEED_FORWARDS.unregister("toy_scale")
+        ARCHITECTURES.unregister("ToyForCausalLM")
+
+
 # ------------------------------------------------------------------ routing and another position encoding
 class ToyRouted(Part):
     """A feed-forward with routing: a float32 router picks the top 2 of E one-matrix experts per
