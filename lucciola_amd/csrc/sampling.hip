@@ -13,11 +13,41 @@
 //   pass 3  per row: pick (greedy: the best part's index; sampled: the part that holds
 //           u * total, then the first index inside it whose running sum passes the target)
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 namespace lc {
 
 constexpr int SP_THREADS = 256;
 constexpr int SP_BLOCKS = 32;
+
+// The workspace of lc_sample_static.  In host code this name is only a stand-in for the
+// symbol: the array's address on a device comes from hipGetSymbolAddress (static_scratch()),
+// and only that pointer is ever given to a kernel.
+static __device__ __align__(256) __attribute__((used)) float scratch[LC_SAMPLE_STATIC_MAX_ROWS * SP_BLOCKS * 3];
+
+constexpr int SP_MAX_DEVICES = 64;
+static float* scratch_ptr[SP_MAX_DEVICES];      // per device: each GPU has its own copy of the array
+static std::mutex scratch_mutex;
+
+// The address of `scratch` on the current device, looked up at the first call there.
+static int static_scratch(float** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    LC_CHECK(e == hipSuccess, "sample_static: hipGetDevice failed: %s", hipGetErrorString(e));
+    LC_CHECK(dev >= 0 && dev < SP_MAX_DEVICES, "sample_static: device %d is beyond the %d this library keeps",
+             dev, SP_MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_ptr[dev]) {
+        float* p = nullptr;
+        e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+        LC_CHECK(e == hipSuccess && p, "sample_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+        scratch_ptr[dev] = p;
+    }
+    *out = scratch_ptr[dev];
+    return 0;
+}
 
 __device__ __forceinline__ void part_range(int V, int part, int& begin, int& end) {
     const int per = (V + SP_BLOCKS - 1) / SP_BLOCKS;
@@ -185,15 +215,8 @@ using namespace lc;
 // Floats of workspace a call needs for R rows.
 LC_API int lc_sample_workspace(int R) { return R * SP_BLOCKS * 3; }
 
-// temperature and uniform may be null (all rows greedy).  workspace: lc_sample_workspace(R)
-// 4-byte words.
-LC_API int lc_sample(const float* logits, const float* temperature, const float* uniform, int* out,
-                     float* workspace, int R, int V, hipStream_t stream) {
-    LC_CHECK(R >= 0 && V > 0, "sample: bad sizes R=%d V=%d", R, V);
-    if (R == 0) return 0;
-    LC_CHECK(logits && out && workspace, "sample: null pointer");
-    LC_CHECK(!temperature || uniform, "sample: temperatures without uniform numbers");
-    LC_CHECK(R <= 65535, "sample: too many rows (%d)", R);
+static int sample_into(const float* logits, const float* temperature, const float* uniform, int* out,
+                       float* workspace, int R, int V, hipStream_t stream) {
     float* ws_max = workspace;
     int* ws_idx = reinterpret_cast<int*>(workspace + (size_t)R * SP_BLOCKS);
     float* ws_sum = workspace + (size_t)2 * R * SP_BLOCKS;
@@ -209,6 +232,36 @@ LC_API int lc_sample(const float* logits, const float* temperature, const float*
     LC_LAUNCH_CHECK("sample_pick");
     return 0;
 }
+
+// temperature and uniform may be null (all rows greedy).  workspace: lc_sample_workspace(R)
+// 4-byte words.
+LC_API int lc_sample(const float* logits, const float* temperature, const float* uniform, int* out,
+                     float* workspace, int R, int V, hipStream_t stream) {
+    LC_CHECK(R >= 0 && V > 0, "sample: bad sizes R=%d V=%d", R, V);
+    if (R == 0) return 0;
+    LC_CHECK(logits && out && workspace, "sample: null pointer");
+    LC_CHECK(!temperature || uniform, "sample: temperatures without uniform numbers");
+    LC_CHECK(R <= 65535, "sample: too many rows (%d)", R);
+    return sample_into(logits, temperature, uniform, out, workspace, R, V, stream);
+}
+
+// lc_sample without a workspace from the caller and without any allocation (no_alloc.h): the
+// workspace is the library's own array on the current device.  Overlapping calls on one GPU
+// race on that array.
+LC_API int lc_sample_static(const float* logits, const float* temperature, const float* uniform,
+                            int* out, int R, int V, hipStream_t stream) {
+    LC_CHECK(R >= 0 && V > 0, "sample_static: bad sizes R=%d V=%d", R, V);
+    LC_CHECK(R <= LC_SAMPLE_STATIC_MAX_ROWS, "sample_static: %d rows are more than the %d the library's "
+             "own workspace holds (use lc_sample with a workspace of the caller's)", R, LC_SAMPLE_STATIC_MAX_ROWS);
+    if (R == 0) return 0;
+    LC_CHECK(logits && out, "sample_static: null pointer");
+    LC_CHECK(!temperature || uniform, "sample_static: temperatures without uniform numbers");
+    float* workspace = nullptr;
+    if (int rc = static_scratch(&workspace)) return rc;
+    return sample_into(logits, temperature, uniform, out, workspace, R, V, stream);
+}
+
+LC_API int lc_sample_static_max_rows(void) { return LC_SAMPLE_STATIC_MAX_ROWS; }
 
 // ids [T] of a batch: where source[i] >= 0 the id is taken from sampled[source[i]] (S rows of an
 // earlier lc_sample on the same stream); other ids stay.
