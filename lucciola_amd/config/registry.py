@@ -71,6 +71,12 @@ FEED_FORWARDS: Registry[type] = Registry("feed-forward")
 NORMS: Registry[type] = Registry("norm")
 POSITION_ENCODINGS: Registry[type] = Registry("position encoding")
 BLOCKS: Registry[type] = Registry("block arrangement")
+EMBEDDINGS: Registry[type] = Registry("embedding")
+HEADS: Registry[type] = Registry("output head")
+
+# the families a block's slots may name
+FAMILIES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS,
+            "position": POSITION_ENCODINGS}
 
 
 def architecture_for(config_dict: Dict[str, Any]) -> Architecture:

@@ -23,18 +23,26 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One decoder layer: an arrangement (block kind) of a mixer, a feed-forward and norms.
+    """One decoder layer: a block arrangement and the parts that fill its slots.
 
-    ``names`` maps each part's logical tensor name (``"mixer.q_proj"``) to the name the
+    The block kind decides which slots there are and of which family each is (its ``slots``:
+    the pre-norm residual block has a mixer, a feed-forward and a norm before each; another
+    arrangement may have one shared norm, or no feed-forward).  ``names`` maps each part's
+    logical tensor name, prefixed with its slot (``"mixer.q_proj"``), to the name the
     checkpoint uses (``"model.layers.3.self_attn.q_proj.weight"``).
     """
 
     block: str
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    parts: Dict[str, PartSpec]
     names: Dict[str, str]
+
+
+def prenorm_layer(mixer: PartSpec, feed_forward: PartSpec, mixer_norm: PartSpec,
+                  feed_forward_norm: PartSpec, names: Dict[str, str]) -> LayerSpec:
+    """A layer in the pre-norm residual arrangement (``prenorm_residual``)."""
+    return LayerSpec("prenorm_residual",
+                     {"mixer": mixer, "feed_forward": feed_forward, "mixer_norm": mixer_norm,
+                      "feed_forward_norm": feed_forward_norm}, names)
 
 
 @dataclass(frozen=True)
@@ -61,6 +69,11 @@ class ModelSpec:
     head_name: Optional[str]  # None: the head uses the embedding table (tied)
     init_std: float = 0.02
     max_positions: int = 0  # 0: no guard
+    # the parts at the model's two ends; None: a plain table look-up and a plain bias-free
+    # product, built from vocab_size and hidden_size
+    embedding: Optional[PartSpec] = None
+    head: Optional[PartSpec] = None
+    head_names: Optional[Dict[str, str]] = None   # a head with tensors beyond "weight" names them here
 
     def validate(self) -> None:
         for i, entry in enumerate(self.run_order):

@@ -29,13 +29,13 @@ void set_error(const char* fmt, ...) {
 // ------------------------------------------------------------------------------- embedding
 template <typename TW>
 __global__ void embedding_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
-                                 float* __restrict__ out, int H, int V) {
+                                 float* __restrict__ out, int H, int V, float scale) {
     const int t = blockIdx.x;
     int id = ids[t];
     if (id < 0 || id >= V) id = 0;  // the host has rejected such ids already
     const TW* row = table + (size_t)id * H;
     float* dst = out + (size_t)t * H;
-    for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = to_f32(row[i]);
+    for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = to_f32(row[i]) * scale;   // scale 1: exact
 }
 
 // ------------------------------------------------------------------------------- RMSNorm
@@ -378,15 +378,15 @@ using namespace lc;
 LC_API const char* lc_last_error() { return g_error; }
 
 LC_API int lc_embedding(const int* ids, const void* table, int table_dt, float* out, int T, int H,
-                        int V, hipStream_t stream) {
+                        int V, float scale, hipStream_t stream) {
     LC_CHECK(T >= 0 && H > 0 && V > 0, "embedding: bad sizes T=%d H=%d V=%d", T, H, V);
     if (T == 0) return 0;
     LC_CHECK(ids && table && out, "embedding: null pointer");
     const int threads = H >= 256 ? 256 : 64;
     if (table_dt == DT_F32)
-        embedding_kernel<float><<<T, threads, 0, stream>>>(ids, (const float*)table, out, H, V);
+        embedding_kernel<float><<<T, threads, 0, stream>>>(ids, (const float*)table, out, H, V, scale);
     else if (table_dt == DT_BF16)
-        embedding_kernel<bf16><<<T, threads, 0, stream>>>(ids, (const bf16*)table, out, H, V);
+        embedding_kernel<bf16><<<T, threads, 0, stream>>>(ids, (const bf16*)table, out, H, V, scale);
     else
         LC_CHECK(false, "embedding: unknown table dtype %d", table_dt);
     LC_LAUNCH_CHECK("embedding");

@@ -9,7 +9,7 @@ sent to the GPU in one copy.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Hashable, List, Optional, Sequence, Tuple
+from typing import Any, Callable, Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -17,8 +17,28 @@ import torch
 from ..cache.manager import CacheManager
 from ..kernels.ops import AttentionBatch
 
-PREFILL_TILE = 64   # query rows of one work item of the prefill attention kernel
 PENDING = -1        # a token that an earlier step has sampled and the host has not seen yet
+
+
+@dataclass
+class HostLayout:
+    """A step's batch as the host knows it, for the parts' planners (``Part.batch_planner``)."""
+
+    num_requests: int
+    num_tokens: int
+    q_start: List[int]          # token offset of each request in the batch, R + 1 entries
+    first_position: List[int]   # cached length of each request before this step
+    block_size: int
+    single: bool                # every request brings one token and wants its logits
+
+
+@dataclass
+class Plan:
+    """What a planner made of a step's batch: its arrays on the device, its numbers."""
+
+    arrays: Dict[str, torch.Tensor]
+    info: Dict[str, Any]
+    made: Dict[Any, Any] = field(default_factory=dict)   # for the parts: what they derive from it
 
 
 @dataclass
@@ -68,6 +88,7 @@ class StepBatch:
     slot_ids: torch.Tensor        # int32 [R]
     feed: torch.Tensor            # int32 [T] row of the carry a token is taken from, or -1
     groups: List[AttentionBatch] = field(default_factory=list)
+    plans: Dict[Any, Plan] = field(default_factory=dict)   # by planner key
     num_wanted: int = 0
     buffer: Optional[torch.Tensor] = None   # the one device buffer all of the above view
 
@@ -121,14 +142,16 @@ class _Packer:
 
 def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
                 pad_blocks: Optional[int] = None, into: Optional[torch.Tensor] = None,
-                refresh_only: bool = False, carry_rows: Optional[dict] = None) -> Optional[StepBatch]:
+                refresh_only: bool = False, carry_rows: Optional[dict] = None,
+                planners: Optional[Dict[Any, Callable]] = None) -> Optional[StepBatch]:
     """Lay the entries out as one flat batch.  Pages for the new tokens must be reserved.
 
     ``pad_blocks``: width of the block tables (at least the longest table), so that batches of
     the same make-up have the same layout; ``into``: the buffer of such an earlier batch;
     ``refresh_only``: only bring that buffer up to date (its views exist already), return None;
     ``carry_rows``: for entries whose one token is PENDING, the row of the carry it comes from
-    (the caller copies it in on the device; the host's copy holds token 0 there)."""
+    (the caller copies it in on the device; the host's copy holds token 0 there);
+    ``planners``: the model's ``batch_planners()``, whose arrays travel in the same copy."""
     bs = cache.block_size
     R = len(entries)
     requests = [e.request for e in entries]
@@ -144,8 +167,6 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
         tok_req = np.arange(R, dtype=np.int32)
         want_rows = tok_req
         ctx_len = positions + 1
-        decode_tokens = tok_req
-        tiles: List[int] = []
     else:
         q_start = [0]
         token_parts, position_parts, req_parts = [], [], []
@@ -166,18 +187,6 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
         positions = np.concatenate(position_parts) if position_parts else np.zeros(0, np.int32)
         tok_req = np.concatenate(req_parts) if req_parts else np.zeros(0, np.int32)
         ctx_len = [first_pos[r] + (q_start[r + 1] - q_start[r]) for r in range(R)]
-        decode_tokens = [q_start[r] for r in range(R) if q_start[r + 1] - q_start[r] == 1]
-        tile_list: List[Tuple[int, int, int, int]] = []
-        for r in range(R):
-            n = q_start[r + 1] - q_start[r]
-            if n == 1:
-                continue
-            for t0 in range(0, n, PREFILL_TILE):
-                tile_list.append((r, q_start[r] + t0, min(PREFILL_TILE, n - t0), first_pos[r] + t0))
-        # the tiles that see the most keys first: the kernel's workgroups start in this order,
-        # and whoever is done takes the longest that is left (the order changes no tile's result)
-        tile_list.sort(key=lambda t: -(t[3] + t[2]))
-        tiles = [v for t in tile_list for v in t]
 
     feed = np.full(T, -1, dtype=np.int32)
     pending = np.nonzero(token_ids == PENDING)[0]
@@ -201,9 +210,12 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
     h_slot = pk.add(slot_list)
     h_qs = pk.add(q_start)
     h_ctx = pk.add(ctx_len)
-    h_dec = pk.add(decode_tokens)
-    h_tiles = pk.add(tiles)
-    num_wanted, num_decode = len(want_rows), len(decode_tokens)
+    num_wanted = len(want_rows)
+    layout = HostLayout(R, T, q_start, first_pos, bs, single)
+    planned = []
+    for key, plan in (planners or {}).items():
+        arrays, info = plan(layout)
+        planned.append((key, {name: (pk.add(a), tuple(np.shape(a))) for name, a in arrays.items()}, info))
 
     group_handles = []
     rows = np.arange(R)
@@ -233,13 +245,13 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
         groups.append(AttentionBatch(
             tok_req=pk.view(h_req), positions=pk.view(h_pos),
             block_table=pk.view(h_bt, (R, mb)), q_start=pk.view(h_qs), ctx_len=pk.view(h_ctx),
-            slots=pk.view(h_sl), num_decode=num_decode,
-            decode_tokens=pk.view(h_dec), prefill_tiles=pk.view(h_tiles, (len(tiles) // 4, 4)),
-            max_ctx=max_ctx, all_decode=num_decode == R))
+            slots=pk.view(h_sl), max_ctx=max_ctx))
+    plans = {key: Plan({name: pk.view(h, shape) for name, (h, shape) in handles.items()}, info)
+             for key, handles, info in planned}
     return StepBatch(
         num_tokens=T, num_requests=R, requests=requests, q_start=q_start,
         first_position=first_pos, slot_list=slot_list,
         max_position=int(positions.max()) if T else 0,
         token_ids=pk.view(h_tok), positions=pk.view(h_pos), tok_req=pk.view(h_req),
         want_rows=pk.view(h_want), slot_ids=pk.view(h_slot), feed=pk.view(h_feed), groups=groups,
-        num_wanted=num_wanted, buffer=buffer)
+        plans=plans, num_wanted=num_wanted, buffer=buffer)

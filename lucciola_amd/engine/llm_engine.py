@@ -47,7 +47,8 @@ class LLMEngine:
         self.runner = ModelRunner(model, engine_config)
         self.scheduler = Scheduler(self.runner.cache, engine_config.max_tokens_per_step,
                                    engine_config.max_seqs,
-                                   max_model_len=model.spec.max_positions)
+                                   max_model_len=model.spec.max_positions,
+                                   portion_multiple=model.portion_multiple())
         self.sampler = Sampler()
         self.sequences: Dict[int, Sequence] = {}
         self._next_id = 1

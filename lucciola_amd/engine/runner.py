@@ -57,6 +57,7 @@ class ModelRunner:
             blocks = self._blocks_from_free_memory(needs)
         self.cache = CacheManager(needs, config.block_size, blocks, config.max_seqs)
         self.cache.allocate_tensors(config.dtype, self.device)
+        self.planners = model.batch_planners()
         self.steps = 0
         self.tokens = 0
         # decode steps replayed from HIP graphs: (requests, block-table width) -> captured step
@@ -153,7 +154,7 @@ class ModelRunner:
                 logits, num_tokens = self._graph_step(entries, carry if fed else None), len(entries)
             else:
                 batch = build_batch(entries, self.cache, self.device,
-                                    carry_rows=carry.rows if fed else None)
+                                    carry_rows=carry.rows if fed else None, planners=self.planners)
                 if fed:
                     ops.feed_tokens(batch.token_ids, batch.feed, carry.ids)
                 logits, num_tokens = self.model.forward(batch, self._sites(batch)), batch.num_tokens
@@ -193,9 +194,10 @@ class ModelRunner:
         pad = max(64, -(-widest // 64) * 64)
         # batches of 5 or more requests are filled up to a multiple of 8 with copies of the
         # first entry (same token, same position, same cache slot: the copies compute and write
-        # what the original does), so that a batch that shrinks by one does not need a new graph
+        # what the original does), so that a batch that shrinks by one does not need a new graph;
+        # not with per-request state, which a copy would update a second time
         real = len(entries)
-        rows = real if real <= 4 else -(-real // 8) * 8
+        rows = real if real <= 4 or self.cache.state_sites else -(-real // 8) * 8
         entries = list(entries) + [entries[0]] * (rows - real)
         epoch = self.model.position_epoch()
         if epoch != self._graph_epoch:      # a position table was made anew: addresses changed
@@ -206,7 +208,7 @@ class ModelRunner:
         next_position = max(self.cache.length(e.request) for e in entries)
         if captured is None or not self.model.positions_ready(next_position):
             batch = build_batch(entries, self.cache, self.device, pad_blocks=pad,
-                                carry_rows=carry.rows if carry else None)
+                                carry_rows=carry.rows if carry else None, planners=self.planners)
             if carry:
                 ops.feed_tokens(batch.token_ids, batch.feed, carry.ids)
             sites = self._sites(batch)
@@ -223,7 +225,7 @@ class ModelRunner:
             self._graphs[key] = _CapturedStep(graph, batch, sites, static_logits)
             return logits[:real]
         build_batch(entries, self.cache, self.device, pad_blocks=pad, into=captured.batch.buffer,
-                    refresh_only=True, carry_rows=carry.rows if carry else None)
+                    refresh_only=True, carry_rows=carry.rows if carry else None, planners=self.planners)
         if carry:       # outside the graph: the carry is at another address every step
             ops.feed_tokens(captured.batch.token_ids, captured.batch.feed, carry.ids)
         captured.graph.replay()

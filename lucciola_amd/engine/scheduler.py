@@ -54,11 +54,14 @@ class ScheduledStep:
 
 class Scheduler:
     def __init__(self, cache: CacheManager, max_tokens_per_step: int = 576,
-                 max_seqs: Optional[int] = None, max_model_len: int = 0):
+                 max_seqs: Optional[int] = None, max_model_len: int = 0, portion_multiple: int = 1):
         self.cache = cache
         self.max_tokens_per_step = int(max_tokens_per_step)
         self.max_seqs = int(max_seqs or cache.max_seqs)
         self.max_model_len = int(max_model_len)
+        # portions of a prompt, but for its last, are multiples of this (what the model's
+        # mixers ask for, ``CausalLM.portion_multiple``)
+        self.portion_multiple = max(1, int(portion_multiple))
         self.waiting: Deque[Sequence] = deque()
         self.running: List[Sequence] = []
         self.num_preemptions = 0
@@ -172,6 +175,8 @@ class Scheduler:
                 room = (-have) % bs + max(free, 0) * bs
                 fit = min(fit, room)
             chunk = fit
+            if chunk < remaining:
+                chunk -= chunk % self.portion_multiple
             if chunk <= 0:
                 break
             if not known:

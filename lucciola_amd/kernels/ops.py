@@ -8,9 +8,10 @@ if the library cannot be built or opened.  Parts call these through the module
 from __future__ import annotations
 
 import ctypes
-from dataclasses import dataclass
+from dataclasses import dataclass, replace
 from typing import Optional
 
+import numpy as np
 import torch
 
 from ..csrc import build as _build
@@ -22,7 +23,7 @@ DT_F32, DT_BF16 = 0, 1
 # argument kinds: p pointer, i int, f float
 _ARG = {"p": ctypes.c_void_p, "i": ctypes.c_int, "f": ctypes.c_float}
 _SIGNATURES = {
-    "lc_embedding": "ppipiiip",
+    "lc_embedding": "ppipiiifp",
     "lc_rmsnorm": "ppppfpiiiipiip",
     "lc_rmsnorm_act": "ppfpiiip",
     "lc_gemm_generic": "pipipiiiip",
@@ -137,14 +138,14 @@ _c_int, _c_float = ctypes.c_int, ctypes.c_float
 
 
 # ------------------------------------------------------------------------------ embedding
-def embedding(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-    """float32 [T, H] rows of ``table`` [V, H] picked by int32 ``ids`` [T]."""
+def embedding(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """float32 [T, H] rows of ``table`` [V, H] picked by int32 ``ids`` [T], times ``scale``."""
     _need(ids, "embedding ids", torch.int32, 1)
     _need(table, "embedding table", None, 2)
     T, (V, H) = ids.shape[0], table.shape
     out = torch.empty((T, H), dtype=torch.float32, device=table.device)
     _call("lc_embedding", _ptr(ids), _ptr(table), _c_int(_dt(table)), _ptr(out), _c_int(T),
-          _c_int(H), _c_int(V), _stream())
+          _c_int(H), _c_int(V), _c_float(scale), _stream())
     return out
 
 
@@ -478,6 +479,51 @@ class AttentionBatch:
     prefill_tiles: Optional[torch.Tensor] = None   # [NT, 4]: request, first token row, rows, first position
     max_ctx: int = 0                               # longest cached length in the batch
     all_decode: bool = False
+
+
+PREFILL_TILE = 64               # query rows of one work item of the prefill attention kernel
+ATTENTION_PLAN = "paged_attention"
+
+
+def plan_attention(layout):
+    """The work lists of the attention kernels for one step's batch (a planner in the sense of
+    ``Part.batch_planner``): the token rows of the portions of length one, which the decode
+    kernel serves, and the tiles of up to PREFILL_TILE query rows that the longer portions are
+    cut into, four numbers each (request, first token row, rows, first position).  The tiles
+    that see the most keys come first: the kernel's workgroups start in this order, and whoever
+    is done takes the longest that is left (the order changes no tile's result)."""
+    R, q_start, first = layout.num_requests, layout.q_start, layout.first_position
+    if layout.single:
+        decode = np.arange(R, dtype=np.int32)
+        tiles = np.zeros((0, 4), dtype=np.int32)
+    else:
+        decode = np.asarray([q_start[r] for r in range(R) if q_start[r + 1] - q_start[r] == 1],
+                            dtype=np.int32)
+        tile_list = []
+        for r in range(R):
+            n = q_start[r + 1] - q_start[r]
+            if n == 1:
+                continue
+            for t0 in range(0, n, PREFILL_TILE):
+                tile_list.append((r, q_start[r] + t0, min(PREFILL_TILE, n - t0), first[r] + t0))
+        tile_list.sort(key=lambda t: -(t[3] + t[2]))
+        tiles = np.asarray(tile_list, dtype=np.int32).reshape(-1, 4)
+    return ({"decode_tokens": decode, "prefill_tiles": tiles},
+            {"num_decode": int(decode.size), "all_decode": int(decode.size) == R})
+
+
+def attention_batch(generic: AttentionBatch, plan) -> AttentionBatch:
+    """``generic`` (a page group's view of the batch) with the work lists of ``plan`` (made by
+    :func:`plan_attention`; None: without, and only the generic kernel can run)."""
+    if plan is None:
+        return generic
+    done = plan.made.get(id(generic))
+    if done is None:
+        done = replace(generic, decode_tokens=plan.arrays["decode_tokens"],
+                       prefill_tiles=plan.arrays["prefill_tiles"],
+                       num_decode=plan.info["num_decode"], all_decode=plan.info["all_decode"])
+        plan.made[id(generic)] = done
+    return done
 
 
 @dataclass

@@ -10,31 +10,50 @@ argmax, src/qwen.cc:875-892).
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional
+import math
+from typing import Callable, Dict, List, Optional
 
 import torch
 
-from ..config.registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
-from ..config.specs import LayerSpec, ModelSpec
+from ..config.registry import BLOCKS, EMBEDDINGS, FAMILIES, HEADS, NORMS
+from ..config.specs import LayerSpec, ModelSpec, PartSpec
 from ..engine.batch import SiteView, StepBatch
-from ..kernels import ops
 from ..parts import BuildContext, ResidualStream, build_part
 from ..weights.loader import ParamDecl, WeightSource, load_declared
 
 
 class _LayerParts:
+    """The parts of one layer, built from its spec, and the block that arranges them."""
+
     def __init__(self, spec: LayerSpec):
         self.spec = spec
-        self.mixer = build_part(MIXERS, spec.mixer)
-        self.feed_forward = build_part(FEED_FORWARDS, spec.feed_forward)
-        self.mixer_norm = build_part(NORMS, spec.mixer_norm)
-        self.feed_forward_norm = build_part(NORMS, spec.feed_forward_norm)
-        self.block = BLOCKS.get(spec.block)(self.mixer, self.feed_forward, self.mixer_norm,
-                                            self.feed_forward_norm)
+        block_cls = BLOCKS.get(spec.block)
+        slots = getattr(block_cls, "slots", None)
+        if not isinstance(slots, dict):
+            raise TypeError(f"block arrangement '{spec.block}' does not say which slots it has")
+        if set(slots) != set(spec.parts):
+            raise ValueError(f"block arrangement '{spec.block}' has the slots {sorted(slots)}, "
+                             f"the layer gives {sorted(spec.parts)}")
+        self.by_slot = {}
+        for slot, family in slots.items():
+            if family not in FAMILIES:
+                raise ValueError(f"block arrangement '{spec.block}': slot '{slot}' names the "
+                                 f"unknown family '{family}'")
+            self.by_slot[slot] = build_part(FAMILIES[family], spec.parts[slot])
+        self.block = block_cls(**self.by_slot)
+        caching = [p for p in self.by_slot.values() if p.cache_need() is not None]
+        if len(caching) > 1:
+            raise ValueError(f"a layer may hold one part with a cache, this one has {len(caching)}")
+        self.cache_part = caching[0] if caching else None
+
+    def __getattr__(self, slot):          # layer.mixer, layer.feed_forward_norm, ...
+        try:
+            return self.__dict__["by_slot"][slot]
+        except KeyError:
+            raise AttributeError(slot) from None
 
     def parts(self):
-        return (("mixer", self.mixer), ("feed_forward", self.feed_forward),
-                ("mixer_norm", self.mixer_norm), ("feed_forward_norm", self.feed_forward_norm))
+        return tuple(self.by_slot.items())
 
     def declared(self) -> Dict[str, ParamDecl]:
         """Checkpoint name -> declaration, through the layer's name map."""
@@ -54,18 +73,36 @@ class _LayerParts:
             part.bind(mine, ctx)
 
 
+def _end_parts(spec: ModelSpec):
+    """The embedding and the head of a spec (built, not bound) and the head's name map."""
+    sizes = {"vocab_size": spec.vocab_size, "hidden_size": spec.hidden_size}
+    embedding = build_part(EMBEDDINGS, spec.embedding or PartSpec("token_embedding", sizes))
+    head_spec = spec.head or PartSpec("linear_head", sizes)
+    head = build_part(HEADS, head_spec.with_params(tied=spec.head_name is None))
+    head_names = dict(spec.head_names or {})
+    if spec.head_name is not None:
+        head_names.setdefault("weight", spec.head_name)
+    return embedding, head, head_names
+
+
 def declared_tensors(spec: ModelSpec) -> Dict[str, ParamDecl]:
     """Every tensor a model of this spec wants, by checkpoint name."""
     spec.validate()
-    out: Dict[str, ParamDecl] = {
-        spec.embedding_name: ParamDecl((spec.vocab_size, spec.hidden_size))}
+    embedding, head, head_names = _end_parts(spec)
+    out: Dict[str, ParamDecl] = {}
+    for logical, decl in embedding.declare().items():
+        if logical != "weight":
+            raise KeyError(f"the embedding's tensor '{logical}' has no checkpoint name")
+        out[spec.embedding_name] = decl
     for layer in spec.layers:
         out.update(_LayerParts(layer).declared())
     norm = build_part(NORMS, spec.final_norm)
     for logical, decl in norm.declare().items():
         out[spec.final_norm_names[logical]] = decl
-    if spec.head_name is not None:
-        out[spec.head_name] = ParamDecl((spec.vocab_size, spec.hidden_size))
+    for logical, decl in head.declare().items():
+        if logical not in head_names:
+            raise KeyError(f"the head's tensor '{logical}' has no checkpoint name")
+        out[head_names[logical]] = decl
     return out
 
 
@@ -77,8 +114,11 @@ class CausalLM:
         self.ctx = BuildContext(dtype=dtype, device=torch.device(device))
         tensors = load_declared(source, declared_tensors(spec), self.ctx.device,
                                 optional=optional_names)
-        self.embedding = tensors[spec.embedding_name]
-        self.head = tensors[spec.head_name] if spec.head_name is not None else self.embedding
+        self.embed, self.head_part, head_names = _end_parts(spec)
+        self.embed.bind({"weight": tensors[spec.embedding_name]}, self.ctx)
+        self.head_part.bind({logical: tensors[head_names[logical]]
+                             for logical in self.head_part.declare()}, self.ctx,
+                            shared=self.embed.table())
         self.layers: List[_LayerParts] = []
         for layer_spec in spec.layers:
             layer = _LayerParts(layer_spec)
@@ -89,26 +129,55 @@ class CausalLM:
                               for logical, name in spec.final_norm_names.items()}, self.ctx)
         self.vocab_size, self.hidden_size = spec.vocab_size, spec.hidden_size
 
+    @property
+    def embedding(self) -> torch.Tensor:
+        return self.embed.table()
+
+    @property
+    def head(self) -> torch.Tensor:
+        return self.head_part.weight
+
+    def _all_parts(self):
+        for layer in self.layers:
+            for _, part in layer.parts():
+                yield part
+
     # ------------------------------------------------------------------ cache needs
     def site_needs(self) -> List[Optional[object]]:
         """For each site of the run order: what it needs of the cache (None when it reads
         another site's cache or needs nothing)."""
         needs = []
         for entry in self.spec.run_order:
-            needs.append(None if entry.cache_of is not None
-                         else self.layers[entry.layer].mixer.cache_need())
+            part = self.layers[entry.layer].cache_part
+            needs.append(None if entry.cache_of is not None or part is None else part.cache_need())
         return needs
 
     def graph_safe(self) -> bool:
-        """Whether every part of every layer may be captured in a HIP graph."""
-        return all(getattr(part, "graph_safe", False)
-                   for layer in self.layers for _, part in layer.parts()) \
-            and getattr(self.final_norm, "graph_safe", False)
+        """Whether every part may be captured in a HIP graph."""
+        return all(getattr(part, "graph_safe", False) for part in self._all_parts()) \
+            and all(getattr(p, "graph_safe", False) for p in (self.final_norm, self.embed, self.head_part))
+
+    def batch_planners(self) -> Dict[object, Callable]:
+        """The work lists that parts want made from every step's batch (``Part.batch_planner``),
+        one per distinct key."""
+        planners: Dict[object, Callable] = {}
+        for part in self._all_parts():
+            planner = part.batch_planner()
+            if planner is not None:
+                planners.setdefault(planner[0], planner[1])
+        return planners
+
+    def portion_multiple(self) -> int:
+        """Portions of a prompt, but for its last, must be multiples of this many tokens."""
+        multiple = 1
+        for part in self._all_parts():
+            multiple = math.lcm(multiple, int(getattr(part, "portion_multiple", 1)))
+        return multiple
 
     # ------------------------------------------------------------------ position tables
     def _position_parts(self):
-        for layer in self.layers:
-            pos = getattr(layer.mixer, "position", None)
+        for part in self._all_parts():
+            pos = getattr(part, "position", None)
             if pos is not None and hasattr(pos, "generation"):
                 yield pos
 
@@ -123,10 +192,10 @@ class CausalLM:
     # ------------------------------------------------------------------ forward
     def forward(self, batch: StepBatch, sites: List[SiteView]) -> torch.Tensor:
         """Run the batch's tokens through every site; float32 logits [wanted, vocab]."""
-        stream = ResidualStream(ops.embedding(batch.token_ids, self.embedding))
+        stream = ResidualStream(self.embed.forward(batch.token_ids))
         for index, entry in enumerate(self.spec.run_order):
             self.layers[entry.layer].block.forward(stream, sites[index])
         if batch.num_wanted == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.ctx.device)
         x = self.final_norm.add_norm_rows(stream, batch.want_rows)
-        return ops.gemm(x, self.head, torch.float32)
+        return self.head_part.forward(x)

@@ -10,7 +10,7 @@ from __future__ import annotations
 
 from ..config.model_config import Qwen3Config
 from ..config.registry import ARCHITECTURES, Architecture
-from ..config.specs import LayerSpec, ModelSpec, PartSpec, RunEntry
+from ..config.specs import ModelSpec, PartSpec, RunEntry, prenorm_layer
 
 
 def qwen3_layer_names(i: int):
@@ -46,9 +46,7 @@ def qwen3_model_spec(cfg: Qwen3Config) -> ModelSpec:
             "num_kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
             "scale": cfg.head_dim ** -0.5, "qk_norm": head_norm, "position": rotary,
             "window": cfg.sliding_window if sliding else None})
-        layers.append(LayerSpec(block="prenorm_residual", mixer=mixer, feed_forward=feed_forward,
-                                mixer_norm=norm, feed_forward_norm=norm,
-                                names=qwen3_layer_names(i)))
+        layers.append(prenorm_layer(mixer, feed_forward, norm, norm, qwen3_layer_names(i)))
     return ModelSpec(
         hidden_size=cfg.hidden_size, vocab_size=cfg.vocab_size,
         embedding_name="model.embed_tokens.weight", layers=layers,

@@ -39,6 +39,7 @@ class Attention(Part):
         self.H, self.nh, self.nkv, self.d = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
         self.scale = float(scale) if scale is not None else self.d ** -0.5
         self.window = int(window) if window else None
+        self.fused_qk_norm = True
         self.q_norm = build_part(NORMS, qk_norm) if qk_norm else None
         self.k_norm = build_part(NORMS, qk_norm) if qk_norm else None
         self.position = build_part(POSITION_ENCODINGS, position) if position else None
@@ -62,19 +63,35 @@ class Attention(Part):
         if self.q_norm is not None:
             self.q_norm.bind({k[7:]: v for k, v in tensors.items() if k.startswith("q_norm.")}, ctx)
             self.k_norm.bind({k[7:]: v for k, v in tensors.items() if k.startswith("k_norm.")}, ctx)
-            if self.q_norm.fused_rms() is None:
-                raise NotImplementedError("attention: the q/k norm must offer fused_rms()")
+            # a norm that the fused kernel cannot apply (no fused_rms()) is applied through its
+            # own ``apply`` on the heads, one kernel more a step
+            fused = getattr(self.q_norm, "fused_rms", None)
+            self.fused_qk_norm = fused is not None and fused() is not None
+            if not self.fused_qk_norm and not hasattr(self.q_norm, "apply"):
+                raise NotImplementedError("attention: the q/k norm must offer fused_rms() or apply()")
         if self.position is not None:
             self.position.bind({}, ctx)
+
+    def _norm_heads(self, qkv: torch.Tensor) -> None:
+        """The q and k heads of ``qkv`` [T, (nh + 2 nkv) d] through the norms' own ``apply``."""
+        T = qkv.shape[0]
+        for norm, first, heads in ((self.q_norm, 0, self.nh), (self.k_norm, self.nh, self.nkv)):
+            cols = slice(first * self.d, (first + heads) * self.d)
+            x = qkv[:, cols].contiguous().view(T * heads, self.d)
+            qkv[:, cols] = norm.apply(x).view(T, heads * self.d)
 
     def cache_need(self):
         return PagedKV(self.nkv, self.d, self.window)
 
+    def batch_planner(self):
+        return ops.ATTENTION_PLAN, ops.plan_attention
+
     def forward(self, x: torch.Tensor, site) -> torch.Tensor:
-        attn = site.attn
+        attn = ops.attention_batch(site.attn, site.batch.plans.get(ops.ATTENTION_PLAN))
         q_w = k_w = None
         eps = 0.0
-        if self.q_norm is not None:
+        own_norm = self.q_norm is not None and not self.fused_qk_norm
+        if self.q_norm is not None and self.fused_qk_norm:
             q_w, eps = self.q_norm.fused_rms()
             k_w, _ = self.k_norm.fused_rms()
         table = None
@@ -83,10 +100,12 @@ class Attention(Part):
         # where the q/k/v product is cut along K and the attention kernel can sum its shares
         # as it reads them, the kernel that would sum them is saved
         rows = x.x.shape[0] if isinstance(x, ops.ScaledRows) else x.shape[0]
-        as_shares = ((table is not None or self.position is None)
+        as_shares = ((table is not None or self.position is None) and not own_norm
                      and ops.attention_takes_shares(attn, rows, self.nh, self.nkv, self.d, site.page_size,
                                                     self.dtype, table.shape[1] if table is not None else 0))
         qkv = ops.gemm(x, self.qkv, self.dtype, shares=as_shares)
+        if own_norm:
+            self._norm_heads(qkv)
         if self.position is not None and table is None:
             self.position.apply(qkv, self.nh, self.nkv, self.d, attn.positions)
         k_cache, v_cache = site.kv

@@ -12,12 +12,15 @@ Interfaces (all tensors on the GPU; "act" is the engine's activation dtype):
                   return ops.ScaledRows; stream.pending may be an ops.PendingProduct
   PositionEncoding  rotary_table(max_position) -> float32 [positions, rot] or None;
                   apply(qkv, nh, nkv, d, positions) in place, when there is no table
-  Mixer           forward(x act [T, H], site: SiteView) -> act [T, H]; cache_need() -> spec
+  Mixer           forward(x act [T, H], site: SiteView) -> act [T, H]; cache_need() -> spec;
+                  batch_planner() -> (key, plan) or None; portion_multiple
   FeedForward     forward(x act [T, H]) -> act [T, H]
                   A mixer or feed-forward with takes_scaled_rows = True may be given
                   ops.ScaledRows as x (ops.gemm and ops.gemm_swiglu take them) and may return
                   ops.gemm(..., defer=True); ops.value(t) turns either into a tensor
-  Block           forward(stream, site) -> None (updates the stream)
+  Block           slots = {slot name: family}; built with the layer's parts by slot name;
+                  forward(stream, site) -> None (updates the stream)
+  Embedding, Head the model's two ends (parts/ends.py)
 """
 from __future__ import annotations
 
@@ -54,8 +57,15 @@ class Part:
 
     # True if ``forward`` only launches kernels on tensors whose addresses and shapes depend
     # on nothing but the batch layout (no host-side reads of batch values, no loops over
-    # requests): such a part may be captured in a HIP graph and replayed.
+    # requests): such a part may be captured in a HIP graph and replayed.  A captured step of
+    # five or more requests is filled up with copies of its first entry (same token, same
+    # position, same pages), so what such a part writes for a request must be the same when
+    # written twice; a model with per-request state slots is never filled up this way.
     graph_safe = False
+
+    # Portions of a prompt, but for its last, are cut at multiples of this many tokens (a
+    # mixer whose kernel works on whole blocks of tokens sets it; the scheduler obeys it).
+    portion_multiple = 1
 
     def __init__(self, **params: Any):
         self.params = dict(params)
@@ -69,6 +79,16 @@ class Part:
 
     def cache_need(self):
         """Mixers: a cache spec (PagedKV, FixedState) or None."""
+        return None
+
+    def batch_planner(self):
+        """Work lists this part's kernels want made from every step's batch, once a step and
+        not once a layer: ``(key, plan)`` or None.  ``plan(layout: engine.batch.HostLayout)``
+        returns ``(arrays, info)``: named int32 arrays (numpy), which reach the GPU in the
+        batch's one copy, and host-side numbers.  Parts with equal keys share one plan; the
+        part finds it as ``site.batch.plans[key]`` (``.arrays`` on the device, ``.info``).
+        For batches of the same make-up the arrays must have the same sizes (captured steps
+        refresh them in place)."""
         return None
 
 

@@ -12,6 +12,11 @@ from .base import ResidualStream
 
 @BLOCKS.register("prenorm_residual")
 class PreNormResidualBlock:
+    # the slots of this arrangement and the family each is built from; the model builds the
+    # parts named in ``LayerSpec.parts`` and hands them over by slot name
+    slots = {"mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "norm",
+             "feed_forward_norm": "norm"}
+
     def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm):
         self.mixer, self.feed_forward = mixer, feed_forward
         self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm

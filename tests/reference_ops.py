@@ -10,8 +10,8 @@ import torch
 F64 = torch.float64
 
 
-def embedding(ids, table):
-    return table[ids.long()].to(torch.float32)
+def embedding(ids, table, scale=1.0):
+    return table[ids.long()].to(torch.float32) * scale
 
 
 def rmsnorm(h, delta, weight, eps, out_dtype, rows=None, scaled=False):   # never hands out scaled rows

@@ -107,10 +107,11 @@ def test_model_spec_is_data():
     arch = architecture_for(configs.TINY_C)
     spec = arch.model_spec(arch.read_config(configs.TINY_C))
     assert [e.layer for e in spec.run_order] == [0, 1, 2, 3]
-    assert [l.mixer.params["window"] for l in spec.layers] == [None, 24, None, 24]
-    assert spec.layers[0].mixer.params["qk_norm"].params == {"size": 48, "eps": 3e-6}
+    assert [l.parts["mixer"].params["window"] for l in spec.layers] == [None, 24, None, 24]
+    assert spec.layers[0].parts["mixer"].params["qk_norm"].params == {"size": 48, "eps": 3e-6}
     assert spec.layers[2].names["mixer.q_proj"] == "model.layers.2.self_attn.q_proj.weight"
     assert spec.head_name == "lm_head.weight"
+    assert sorted(spec.layers[0].parts) == ["feed_forward", "feed_forward_norm", "mixer", "mixer_norm"]
     tied = arch.model_spec(arch.read_config(configs.TINY_A))
     assert tied.head_name is None
     # the run order is checked

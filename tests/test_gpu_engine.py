@@ -537,10 +537,11 @@ def test_position_table_grows_under_captured_steps():
     spec = arch.model_spec(config)
     layers = []
     for layer in spec.layers:
-        position = layer.mixer.params["position"]
+        mixer = layer.parts["mixer"]
+        position = mixer.params["position"]
         assert position.params["max_positions"] >= 2048
-        layers.append(replace(layer, mixer=layer.mixer.with_params(
-            position=position.with_params(max_positions=0, theta=position.params["theta"] + 1))))
+        layers.append(replace(layer, parts=dict(layer.parts, mixer=mixer.with_params(
+            position=position.with_params(max_positions=0, theta=position.params["theta"] + 1)))))
     spec = replace(spec, layers=layers)     # theta + 1: a table of its own, not another test's
     cfg = dict(cfg, rope_theta=cfg["rope_theta"] + 1)
     model = _build(spec, DictSource(weights), "bfloat16", DEV)

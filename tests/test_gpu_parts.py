@@ -14,7 +14,7 @@ from lucciola_amd.cache.manager import CacheManager
 from lucciola_amd.cache.specs import FixedState, PagedKV
 from lucciola_amd.config.engine_config import EngineConfig
 from lucciola_amd.config.registry import ARCHITECTURES, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Architecture
-from lucciola_amd.config.specs import LayerSpec, ModelSpec, PartSpec, RunEntry
+from lucciola_amd.config.specs import LayerSpec, ModelSpec, PartSpec, RunEntry, prenorm_layer
 from lucciola_amd.engine.batch import SiteView, StepEntry, build_batch
 from lucciola_amd.engine.loading import _build
 from lucciola_amd.engine.runner import ModelRunner
@@ -111,7 +111,8 @@ def attention_site(part, T, page, dtype, first=0):
         cache.reserve("r", first)
         cache.commit("r")
     cache.reserve("r", T)
-    batch = build_batch([StepEntry("r", list(range(T)), [])], cache, DEV)
+    batch = build_batch([StepEntry("r", list(range(T)), [])], cache, DEV,
+                        planners=dict([part.batch_planner()]))
     return SiteView(batch=batch, index=0, writes_cache=True, page_size=page, kv=cache.kv[0],
                     attn=batch.groups[0]), cache
 
@@ -249,7 +250,7 @@ def toy_spec(c):
             names.update({f"mixer.{k}_proj": f"l{i}.{k}" for k in "qkvo"})
         else:
             names.update({"mixer.in_proj": f"l{i}.in", "mixer.out_proj": f"l{i}.out"})
-        layers.append(LayerSpec("prenorm_residual", mixer, ff, norm, norm, names))
+        layers.append(prenorm_layer(mixer, ff, norm, norm, names))
     return ModelSpec(hidden_size=c["hidden_size"], vocab_size=c["vocab_size"], embedding_name="emb",
                      layers=layers, run_order=[RunEntry(0), RunEntry(1), RunEntry(2), RunEntry(0)],
                      final_norm=norm, final_norm_names={"weight": "final"}, head_name="head", init_std=0.2)
@@ -417,7 +418,7 @@ def toy2_spec(c):
                  "feed_forward.router": f"l{i}.router"}
         names.update({f"feed_forward.expert{e}": f"l{i}.e{e}" for e in range(c["experts"])})
         names.update({f"mixer.{k}_proj": f"l{i}.{k}" for k in "qkvo"})
-        layers.append(LayerSpec("prenorm_residual", attn, ff, norm, norm, names))
+        layers.append(prenorm_layer(attn, ff, norm, norm, names))
     return ModelSpec(hidden_size=c["hidden_size"], vocab_size=c["vocab_size"], embedding_name="emb",
                      layers=layers, run_order=[RunEntry(0), RunEntry(1)],
                      final_norm=norm, final_norm_names={"weight": "final"}, head_name="head", init_std=0.3)
@@ -471,6 +472,136 @@ def test_toy_routed_feed_forward_and_another_position_encoding():
         FEED_FORWARDS.unregister("toy_routed")
         POSITION_ENCODINGS.unregister("toy_offset")
         ARCHITECTURES.unregister("Toy2ForCausalLM")
+
+
+# ------------------------------------------------------------------ another arrangement, head norm and ends
+class ParallelBlock:
+    """One shared norm, mixer and feed-forward side by side: h += mixer(norm(h)) + ff(norm(h))."""
+
+    slots = {"norm": "norm", "mixer": "mixer", "feed_forward": "feed_forward"}
+
+    def __init__(self, norm, mixer, feed_forward):
+        self.norm, self.mixer, self.feed_forward = norm, mixer, feed_forward
+
+    def forward(self, stream, site):
+        x = self.norm.add_norm(stream)
+        stream.pending = ops.value(self.mixer.forward(x, site)) + ops.value(self.feed_forward.forward(x))
+
+
+class UnitLength(Part):
+    """A head norm that the fused kernel does not know: x / sqrt(sum x^2 + eps) * w."""
+
+    def __init__(self, size, eps):
+        super().__init__(size=size, eps=eps)
+        self.size, self.eps = size, eps
+
+    def declare(self):
+        return {"weight": ParamDecl((self.size,), role="vector", init="ones_plus_normal")}
+
+    def bind(self, tensors, ctx):
+        self.weight = tensors["weight"]
+
+    def apply(self, x):
+        v = x.float()
+        return (v * torch.rsqrt((v * v).sum(-1, keepdim=True) + self.eps) * self.weight).to(x.dtype)
+
+
+class BiasHead(Part):
+    """An output head with a bias."""
+
+    def __init__(self, vocab_size, hidden_size, tied=False):
+        super().__init__(vocab_size=vocab_size, hidden_size=hidden_size, tied=tied)
+        self.V, self.H = vocab_size, hidden_size
+
+    def declare(self):
+        return {"weight": ParamDecl((self.V, self.H)), "bias": ParamDecl((self.V,), role="vector")}
+
+    def bind(self, tensors, ctx, shared=None):
+        self.weight, self.bias = tensors["weight"], tensors["bias"]
+
+    def forward(self, x):
+        return ops.gemm(x, self.weight, torch.float32) + self.bias
+
+
+TOY3 = {"architectures": ["Toy3ForCausalLM"], "hidden_size": 40, "vocab_size": 53, "eps": 1e-6,
+        "heads": 4, "kv_heads": 2, "head_dim": 16, "inner": 56, "scale": 3.0}
+
+
+def toy3_spec(c):
+    H = c["hidden_size"]
+    norm = PartSpec("rms", {"size": H, "eps": c["eps"]})
+    attn = PartSpec("attention", {"hidden_size": H, "num_heads": c["heads"], "num_kv_heads": c["kv_heads"],
+                                  "head_dim": c["head_dim"],
+                                  "qk_norm": PartSpec("unit_length", {"size": c["head_dim"], "eps": c["eps"]}),
+                                  "position": PartSpec("rotary", {"rotary_dim": c["head_dim"], "theta": 500.0})})
+    ff = PartSpec("gated_mlp", {"hidden_size": H, "intermediate_size": c["inner"]})
+    layers = []
+    for i in range(2):
+        names = {"norm.weight": f"l{i}.n", "mixer.q_norm.weight": f"l{i}.qn", "mixer.k_norm.weight": f"l{i}.kn"}
+        names.update({f"mixer.{k}_proj": f"l{i}.{k}" for k in "qkvo"})
+        names.update({f"feed_forward.{k}_proj": f"l{i}.{k}" for k in ("gate", "up", "down")})
+        layers.append(LayerSpec("toy_parallel", {"norm": norm, "mixer": attn, "feed_forward": ff}, names))
+    sizes = {"vocab_size": c["vocab_size"], "hidden_size": H}
+    return ModelSpec(hidden_size=H, vocab_size=c["vocab_size"], embedding_name="emb", layers=layers,
+                     run_order=[RunEntry(0), RunEntry(1)], final_norm=norm,
+                     final_norm_names={"weight": "final"}, head_name="head", init_std=0.3,
+                     embedding=PartSpec("token_embedding", dict(sizes, scale=c["scale"])),
+                     head=PartSpec("bias_head", sizes), head_names={"bias": "head_b"})
+
+
+def toy3_plain(c, w, ids):
+    w = {k: v.double() for k, v in w.items()}
+    T, d, nh, nkv = len(ids), c["head_dim"], c["heads"], c["kv_heads"]
+    unit = lambda x, wt: x / torch.sqrt((x * x).sum(-1, keepdim=True) + c["eps"]) * wt
+    h = w["emb"][torch.tensor(ids)] * c["scale"]
+    for i in range(2):
+        x = plain.rmsnorm(h, w[f"l{i}.n"], c["eps"])
+        q = plain.rope(unit((x @ w[f"l{i}.q"].T).view(T, nh, d), w[f"l{i}.qn"]), range(T), 500.0)
+        k = plain.rope(unit((x @ w[f"l{i}.k"].T).view(T, nkv, d), w[f"l{i}.kn"]), range(T), 500.0)
+        v = (x @ w[f"l{i}.v"].T).view(T, nkv, d)
+        a = plain.attention(q, k, v, list(range(T))).reshape(T, -1) @ w[f"l{i}.o"].T
+        m = plain.swiglu(x @ w[f"l{i}.gate"].T, x @ w[f"l{i}.up"].T) @ w[f"l{i}.down"].T
+        h = h + a + m
+    return plain.rmsnorm(h, w["final"], c["eps"]) @ w["head"].T + w["head_b"]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_block_with_one_norm_and_parallel_branches(dtype):
+    """Registered from this file alone: a block arrangement with other slots than the built-in
+    one (one shared norm, two branches side by side), a q/k norm the fused kernel does not know
+    (applied through its own ``apply``), a scaled embedding and a head with a bias."""
+    from lucciola_amd.config.registry import BLOCKS, HEADS
+    BLOCKS.register("toy_parallel", ParallelBlock, replace=True)
+    NORMS.register("unit_length", UnitLength, replace=True)
+    HEADS.register("bias_head", BiasHead, replace=True)
+    ARCHITECTURES.register("Toy3ForCausalLM", Architecture("Toy3ForCausalLM", read_config=dict,
+                                                           model_spec=toy3_spec), replace=True)
+    try:
+        spec = toy3_spec(TOY3)
+        declared = declared_tensors(spec)
+        assert "head_b" in declared and "l1.qn" in declared and "l0.n" in declared
+        weights = dict(random_tensors(declared, 13, spec.init_std, torch.float32))
+        model = _build(spec, DictSource(weights), dtype, "cuda:0")
+        prompts = prompts_for({"vocab_size": TOY3["vocab_size"]}, [19, 5, 44, 30], 6)
+        refs = {n: toy3_plain(TOY3, weights, ids) for n, ids in prompts.items()}
+        for family in (traces.whole, traces.tail_decode, traces.mixed):
+            steps = family(prompts)
+            runner = ModelRunner(model, EngineConfig(dtype=dtype, block_size=16, max_seqs=4, device="cuda:0",
+                                                     max_blocks=traces.max_live_tokens(steps, 16) // 16))
+            got = replay(runner, steps)
+            compare(got, TOY3, weights, prompts, {torch.float32: 2e-5, torch.bfloat16: 3e-2}[dtype], refs)
+        with pytest.raises(ValueError, match="has the slots"):
+            _build(replace_block(spec, "prenorm_residual"), DictSource(weights), dtype, "cuda:0")
+    finally:
+        BLOCKS.unregister("toy_parallel")
+        NORMS.unregister("unit_length")
+        HEADS.unregister("bias_head")
+        ARCHITECTURES.unregister("Toy3ForCausalLM")
+
+
+def replace_block(spec, block):
+    from dataclasses import replace
+    return replace(spec, layers=[replace(layer, block=block) for layer in spec.layers])
 
 
 def test_block_arrangement_alone():

@@ -181,3 +181,34 @@ def test_random_workloads_finish_and_give_everything_back(seed):
         done += run_step(sched, cache, step, token=rng.randrange(100))
     assert len(done) == 12 and all(s.num_generated == s.params.max_new_tokens for s in done)
     assert cache.groups[0].pool.num_free() == blocks and not cache.requests
+
+
+def test_portions_are_cut_at_the_multiple_a_mixer_asks_for():
+    """A model whose mixer wants portions in multiples of 6: every portion but a prompt's last
+    is one, under the budget and under the pages that are free; an undone step puts the
+    portions back in their order."""
+    cache = CacheManager([PagedKV(1, 16)], 4, 64, 8)
+    sched = Scheduler(cache, 16, 8, portion_multiple=6)
+    a, b = seq(1, 29), seq(2, 8)
+    sched.add_request(a)
+    sched.add_request(b)
+    sizes = []
+    while a.status is not SequenceStatus.RUNNING:
+        step = sched.step()
+        mine = [len(e.tokens) for e, s in zip(step.entries, step.seqs) if s is a]
+        sizes += mine
+        run_step(sched, cache, step)
+    assert sizes == [12, 12, 5]                      # 16 cut down to 12; the last as it comes
+    assert b.status is SequenceStatus.RUNNING        # 8 tokens were its whole prompt: no cut
+    # undo: a step's portions wait again
+    c, d = seq(3, 7), seq(4, 30)
+    sched.add_request(c)
+    sched.add_request(d)
+    step = sched.step()
+    assert [s.seq_id for s in step.seqs] == [1, 2, 3, 4] and step.portions == [0, 0, 7, 6]
+    assert c.status is SequenceStatus.RUNNING and d.prefill_offset == 6
+    sched.undo(step)
+    assert [s.seq_id for s in sched.waiting] == [3, 4] and [s.seq_id for s in sched.running] == [1, 2]
+    assert c.prefill_offset == 0 and d.prefill_offset == 0 and c.status is SequenceStatus.WAITING
+    again = sched.step()
+    assert [len(e.tokens) for e in again.entries] == [1, 1, 7, 6]
