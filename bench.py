@@ -10,7 +10,14 @@ random keys and values instead of running their 8,191-token prompts (a decode st
 does not depend on what the cache holds); the prefill figure is a real 2,048-token prompt in
 one step.  Prints ONE JSON line.
 
-    python bench.py --gpus 1 --steps 20 --warmup 3
+Beside the wall-clock time of a step (``ms_per_step``, the headline) the line carries
+``gpu_ms`` (the same steps between two HIP events on the stream) and ``host_ms`` (what the host
+spends queueing a step, without waiting); ``points`` holds decode at other batch sizes, the
+same batch driven through ``LLMEngine`` and its scheduler after real prompts of the context
+length (``decode_b8_engine``), and the 2,048-token prompt fed in portions of 576, the
+reference's step budget (src/scheduler.cc:48; ``prefill_576``), all in tokens a second.
+
+    python bench.py --gpus 1 --steps 50 --warmup 5
 """
 import argparse
 import json
@@ -33,8 +40,8 @@ SIZES_8B = dict(num_hidden_layers=36, hidden_size=4096, num_attention_heads=32,
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=8192)
     ap.add_argument("--model", default="8b", choices=["8b", "32b", "0.6b"],
@@ -46,6 +53,10 @@ def main() -> int:
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--run-ahead", type=int, default=1, choices=[0, 1],
                     help="1: a step is queued before the host has read the tokens of the one before")
+    ap.add_argument("--portion", type=int, default=576,
+                    help="also feed the prompt in portions of this many tokens (0: skip)")
+    ap.add_argument("--engine-point", type=int, default=1, choices=[0, 1],
+                    help="1: also time the batch through LLMEngine and its scheduler, after real prompts")
     ap.add_argument("--workload", default="decode", choices=["decode", "mixed"],
                     help="decode: the default line; mixed: 64 requests with prompts of 16 to 2,048 "
                          "tokens through the scheduler (Qwen3-0.6B-shaped), chunked prefill beside decode")
@@ -74,7 +85,7 @@ def main() -> int:
     cfg = dict(sizes, architectures=["Qwen3ForCausalLM"], num_hidden_layers=args.layers)
     points = [int(p) for p in args.points.split(",") if p]
     max_batch = max([args.batch] + points)
-    steps_total = args.steps + args.warmup + 8
+    steps_total = max(args.steps, 50) + args.warmup + 8
     per_request = args.context + steps_total
     bs = args.block_size
     blocks = max_batch * (-(-per_request // bs)) + (-(-args.prefill_tokens // bs)) + 8
@@ -111,6 +122,7 @@ def main() -> int:
 
         rows = {n: i for i, n in enumerate(names)}
         under_way = None        # the step whose tokens the host has not read yet
+        wait = [0.0]            # seconds the host waited for tokens inside the current step
 
         def one():
             nonlocal tokens, under_way
@@ -120,26 +132,41 @@ def main() -> int:
                 logits = runner.step([StepEntry(n, [PENDING], [0]) for n in names],
                                      Carry(under_way.ids, rows))
             sampled = sampler.sample_async(logits, params, [0] * batch)
+            t_wait = time.perf_counter()
             if under_way is not None:
                 tokens = under_way.tokens()
             under_way = sampled
             if not args.run_ahead:
                 tokens, under_way = sampled.tokens(), None
+            wait[0] += time.perf_counter() - t_wait
+        host = 0.0
+
+        def timed():
+            nonlocal host
+            t_in = time.perf_counter()
+            one()
+            host += time.perf_counter() - t_in - wait[0]
+            wait[0] = 0.0
         for _ in range(warmup):
             one()
+        wait[0] = 0.0
+        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         t = time.perf_counter()
+        first.record()
         for _ in range(steps):
-            one()
+            timed()
+        last.record()
         if under_way is not None:
             tokens = under_way.tokens()
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t) * 1e3 / steps
+        gpu_ms = first.elapsed_time(last) / steps
         ctx_mid = args.context + warmup + steps / 2.0
         for n in names:
             runner.finish(n)
         bytes_step = weight_bytes + batch * H * esize + batch * ctx_mid * kv_bytes_per_token
-        return ms, batch / (ms / 1e3), bytes_step
+        return ms, batch / (ms / 1e3), bytes_step, gpu_ms, host * 1e3 / steps
 
     def prefill_run(tokens, reps=3):
         gen = torch.Generator().manual_seed(7)
@@ -158,21 +185,80 @@ def main() -> int:
         flops = 2.0 * tokens * L * layer_params + 2.0 * tokens * tokens * nh * d * L + 2.0 * V * H
         return best, flops
 
-    ms, tps, bytes_step = decode_run(args.batch, args.steps, args.warmup)
-    print(f"[bench] decode batch {args.batch}: {ms:.3f} ms/step", file=sys.stderr, flush=True)
+    def prefill_portions(tokens, portion, reps=2):
+        """The same prompt fed in portions of ``portion`` tokens, one a step."""
+        gen = torch.Generator().manual_seed(9)
+        best = None
+        for r in range(reps + 1):
+            ids = torch.randint(0, V, (tokens,), generator=gen).tolist()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            for at in range(0, tokens, portion):
+                part = ids[at:at + portion]
+                final = at + portion >= tokens
+                logits = runner.step([StepEntry(f"q{r}", part, [len(part) - 1] if final else [])])
+            sampler.sample(logits, [SamplingParams()], [0])
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t) * 1e3
+            runner.finish(f"q{r}")
+            if r > 0:
+                best = ms if best is None else min(best, ms)
+        return best
+
+    def engine_run(batch, steps, warmup):
+        """Decode steps of ``batch`` requests driven by LLMEngine and its scheduler: real
+        prompts of the context length are fed first (under a budget of 2,048 tokens a step),
+        then ``steps`` steps of the engine's loop are timed."""
+        from lucciola_amd.engine.llm_engine import LLMEngine
+        # requests that are running already decode while the others' prompts are still fed
+        new = warmup + steps + 8 + batch * (-(-args.context // 2048) + 1)
+        pages = batch * (-(-(args.context + new) // bs)) + 8
+        engine = LLMEngine(model, mcfg, EngineConfig(dtype=dtype, block_size=bs, max_blocks=pages,
+                                                     max_seqs=batch, max_tokens_per_step=2048, device=dev,
+                                                     run_ahead=bool(args.run_ahead)))
+        gen = torch.Generator().manual_seed(100 + batch)
+        for _ in range(batch):
+            engine.add_request(torch.randint(0, V, (args.context - 1,), generator=gen).tolist(),
+                               SamplingParams(max_new_tokens=new, ignore_eos=True))
+        while engine.scheduler.waiting:
+            engine.step()
+        for _ in range(warmup):
+            engine.step()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        got = 0
+        for _ in range(steps):
+            got += len(engine.step())
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t) * 1e3 / steps
+        assert got == steps * batch, f"the engine handed out {got} tokens in {steps} steps of {batch}"
+        del engine
+        return ms, batch / (ms / 1e3)
+
+    ms, tps, bytes_step, gpu_ms, host_ms = decode_run(args.batch, args.steps, args.warmup)
+    print(f"[bench] decode batch {args.batch}: {ms:.3f} ms/step (gpu {gpu_ms:.3f}, host {host_ms:.3f})", file=sys.stderr, flush=True)
     achieved = bytes_step / (ms / 1e3) / 1e9
     pms, pflops = prefill_run(args.prefill_tokens)
     print(f"[bench] prefill {args.prefill_tokens}: {pms:.2f} ms", file=sys.stderr, flush=True)
     point_values = {}
     for b in points:
-        pm, ptps, _ = decode_run(b, max(3, min(args.steps, 10)), 2)
+        pm, ptps, _, pg, ph = decode_run(b, max(args.steps, 50), 3)
         point_values[f"decode_b{b}"] = round(ptps, 2)
-        print(f"[bench] decode batch {b}: {pm:.3f} ms/step", file=sys.stderr, flush=True)
+        print(f"[bench] decode batch {b}: {pm:.3f} ms/step (gpu {pg:.3f}, host {ph:.3f})", file=sys.stderr, flush=True)
+    if args.engine_point:
+        em, etps = engine_run(args.batch, max(args.steps, 50), args.warmup)
+        point_values[f"decode_b{args.batch}_engine"] = round(etps, 2)
+        print(f"[bench] decode batch {args.batch} through the engine's loop: {em:.3f} ms/step", file=sys.stderr, flush=True)
+    if args.portion:
+        qms = prefill_portions(args.prefill_tokens, args.portion)
+        point_values[f"prefill_{args.portion}"] = round(args.prefill_tokens / (qms / 1e3), 1)
+        print(f"[bench] prefill {args.prefill_tokens} in portions of {args.portion}: {qms:.2f} ms", file=sys.stderr, flush=True)
 
     line = {
         "metric": f"decode tok/s (Qwen3-{args.model.upper()}-shaped, batch {args.batch}, context {args.context})",
         "value": round(tps, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "warmup": args.warmup, "ms_per_step": round(ms, 4), "gpu_ms": round(gpu_ms, 4),
+        "host_ms": round(host_ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
         "data": "synthetic: random weights, random token ids, cache of the live requests filled with random keys/values",
         "config": {"model": f"Qwen3-{args.model.upper()}-shaped", "layers": L, "layers_full": layers_full,
