@@ -405,6 +405,50 @@ __global__ __launch_bounds__(128) void attn_prefill_join_kernel(const float* __r
     join_shares<D>(part_o, part_ml, ((size_t)t * nh + h) * splits, splits, out + ((size_t)t * nh + h) * D);
 }
 
+// A lane's part of one raw q row of 128 entries, as the matrix-core operand holds it (entries
+// 32 i + 8 kg + e, i < 4, so an entry and its partner 64 further on sit in the same lane):
+// RMSNorm over the head and the rotary embedding at position p, on the operand registers.  The
+// formulas and the order of their roundings are those of head128_norm_rope; only the sum of
+// squares is added up in another order.
+__device__ __forceinline__ void prepare_q128(bf16x8 (&bq)[4], const DecodePrologue& pro, int p, int kg) {
+    if (!pro.enabled) return;
+    float f[4][8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[i][e] = static_cast<float>(bq[i][e]);
+    if (pro.q_w) {
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss = __fmaf_rn(f[i][e], f[i][e], ss);
+        ss = column_sum(ss);
+        const float inv = rsqrtf(ss / 128.f + pro.eps);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                f[i][e] = __fmul_rn(__fmul_rn(f[i][e], inv), pro.q_w[i * 32 + kg * 8 + e]);
+    }
+    if (pro.rope) {
+        const float* cs = pro.rope + (size_t)p * 128;     // 64 cosines, then 64 sines
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float cosv = cs[i * 32 + kg * 8 + e], sinv = cs[64 + i * 32 + kg * 8 + e];
+                const float a = f[i][e], b = f[i + 2][e];
+                f[i][e] = __fsub_rn(__fmul_rn(a, cosv), __fmul_rn(b, sinv));
+                f[i + 2][e] = __fadd_rn(__fmul_rn(a, sinv), __fmul_rn(b, cosv));
+            }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bq[i][e] = static_cast<bf16>(f[i][e]);
+}
+
 // ------------------------------------------------------------------------------- prefill
 // tiles: [NT, 4] = (request, first token row, rows (<= 64), position of the first row), the
 // tiles that see the most keys first.
@@ -475,50 +519,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
                            (size_t)min(h, nh - 1) * D + kg * 8;
 #pragma unroll
         for (int i = 0; i < D / 32; ++i) bq[c][i] = *reinterpret_cast<const bf16x8*>(qrow + i * 32);
-        if constexpr (D == 128) {
-            // q arrives raw: RMSNorm over the head and the rotary embedding right here, on the
-            // operand registers (the lane holds entries 32 i + 8 kg + e of its row, i < 4, so an
-            // entry and its partner 64 further on sit in the same lane).  The formulas and the
-            // order of their roundings are those of head128_norm_rope; only the sum of squares
-            // is added up in another order.
-            if (pro.enabled) {
-                float f[4][8];
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) f[i][e] = static_cast<float>(bq[c][i][e]);
-                if (pro.q_w) {
-                    float ss = 0.f;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) ss = __fmaf_rn(f[i][e], f[i][e], ss);
-                    ss = column_sum(ss);
-                    const float inv = rsqrtf(ss / 128.f + pro.eps);
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-#pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            f[i][e] = __fmul_rn(__fmul_rn(f[i][e], inv), pro.q_w[i * 32 + kg * 8 + e]);
-                }
-                if (pro.rope) {
-                    const float* cs = pro.rope + (size_t)p * 128;     // 64 cosines, then 64 sines
-#pragma unroll
-                    for (int i = 0; i < 2; ++i)
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) {
-                            const float cosv = cs[i * 32 + kg * 8 + e], sinv = cs[64 + i * 32 + kg * 8 + e];
-                            const float a = f[i][e], b = f[i + 2][e];
-                            f[i][e] = __fsub_rn(__fmul_rn(a, cosv), __fmul_rn(b, sinv));
-                            f[i + 2][e] = __fadd_rn(__fmul_rn(a, sinv), __fmul_rn(b, cosv));
-                        }
-                }
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) bq[c][i][e] = static_cast<bf16>(f[i][e]);
-            }
-        }
+        if constexpr (D == 128) prepare_q128(bq[c], pro, p, kg);
     }
     // pages the workgroup walks, and the part of them this wave needs
     const int t_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
@@ -700,6 +701,269 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     }
 }
 
+// ------------------------------------------------------------------------------- prefill, wide products
+// For heads of 128 in pairs: the tiles and the LDS staging of attn_prefill_kernel<128, 2>, built
+// from v_mfma_f32_32x32x16_bf16.  Two workgroups a CU; a wave does its group's scores, softmax
+// and values one after the other, and the two waves of a SIMD fill each other's gaps.
+// (Measured on this GPU: a product of 16x16x32 holds the vector unit for all of its 16 cycles,
+// so products and softmax take turns even between two waves of a SIMD, 64 products and the
+// softmax of their scores 1,495 ns for two waves; a product of 32x32x16 takes 32 cycles and
+// lets the other wave's vector instructions through meanwhile, 1,065 ns for the same work.)
+//
+// A wave owns 32 query rows of one head.  Per group of 64 keys:
+//   S^T[key, q]  = K[key, :] . Q[q, :]     16 products: A = 32 key rows x 16 dims from LDS,
+//                                          B = Q^T from registers; a lane ends up with 16 keys
+//                                          of one query column per 32-key tile
+//   P^T          = exp2(S^T * scale*log2(e) - reference)       vector unit, float32
+//   O^T[dim, q] += V^T[dim, key] . P^T[key, q]   16 products: A = 32 dims x 16 keys from LDS,
+//                                          B = P^T as the lanes hold it
+// Keys lie in LDS in rows padded by 16 bytes; values per page [dim][16 keys] with a row's four
+// pieces of 4 keys in the order 0, 2, 1, 3, so that the 8 keys a lane supplies to a product (4
+// and the 4 eight further on, as the scores left them in its registers) are one 16-byte read,
+// and with the two halves of a row changing places in every other block of 8 rows, which
+// spreads the 16 rows of a read over all banks (the counters show no bank conflict).  The
+// page numbers come from the block table a group ahead, one page per lane in one vector load:
+// a scalar load per page, each waited for before its page's loads could go out, took a third
+// of the time of a group.
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+// A lane's part of one raw q row of 128 entries in the layout of the 32x32x16 operand (entries
+// 16 i + 8 half + e, i < 8, half = lane / 32: an entry and its partner 64 further on sit in the
+// same lane, the row's other half in lane ^ 32): RMSNorm over the head and the rotary
+// embedding at position p.  Formulas and roundings as in head128_norm_rope; the sum of
+// squares is added up in another order.
+__device__ __forceinline__ void prepare_q128_wide(bf16x8 (&bq)[8], const DecodePrologue& pro, int p, int half) {
+    if (!pro.enabled) return;
+    float f[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[i][e] = static_cast<float>(bq[i][e]);
+    if (pro.q_w) {
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss = __fmaf_rn(f[i][e], f[i][e], ss);
+        float a = ss, b = ss;
+        swap_halves(a, b);
+        ss = a + b;
+        const float inv = rsqrtf(ss / 128.f + pro.eps);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                f[i][e] = __fmul_rn(__fmul_rn(f[i][e], inv), pro.q_w[i * 16 + half * 8 + e]);
+    }
+    if (pro.rope) {
+        const float* cs = pro.rope + (size_t)p * 128;     // 64 cosines, then 64 sines
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float cosv = cs[i * 16 + half * 8 + e], sinv = cs[64 + i * 16 + half * 8 + e];
+                const float a = f[i][e], b = f[i + 4][e];
+                f[i][e] = __fsub_rn(__fmul_rn(a, cosv), __fmul_rn(b, sinv));
+                f[i + 4][e] = __fadd_rn(__fmul_rn(a, sinv), __fmul_rn(b, cosv));
+            }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bq[i][e] = static_cast<bf16>(f[i][e]);
+}
+
+template <int D>
+__global__ __launch_bounds__(256, 2) void attn_prefill_wide_kernel(
+    const bf16* __restrict__ qkv, int q_stride, const bf16* __restrict__ k_cache,
+    const bf16* __restrict__ v_cache, bf16* __restrict__ out, const int* __restrict__ tiles,
+    const int* __restrict__ block_table, int max_blocks, int nh, int nkv, float scale_log2,
+    int window, DecodePrologue pro) {
+    static_assert(D == 128, "heads of 128");
+    constexpr int NP = PF_NP;
+    constexpr int KLD = D + 8;
+    constexpr int KPAGE = PAGE * KLD, VPAGE = D * PAGE;
+    __shared__ __attribute__((aligned(16))) bf16 ks[2][NP * KPAGE];
+    __shared__ __attribute__((aligned(16))) bf16 vs[2][NP * VPAGE];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int q = lane & 31, half = lane >> 5;
+    const int G = nh / nkv;
+    // Workgroups start in the order of their number (x, the head pair, fastest) and two fit on a
+    // CU; the tiles come longest first.  With more workgroups than fit at once, whoever is done
+    // takes the longest tile that is left.  When all fit at once, nobody takes over from a CU
+    // that is done early, and the second workgroup of a CU should be as short as its first is
+    // long: the second half of the numbers takes the tiles from the shortest up.
+    const int total = gridDim.x * gridDim.y, number = blockIdx.y * gridDim.x + blockIdx.x;
+    const int half_of = (total + 1) / 2;
+    const int task = (total <= 2 * 256 && number >= half_of) ? total - 1 - (number - half_of) : number;
+    const int tile_index = task / gridDim.x, heads_index = task - tile_index * gridDim.x;
+    const int h = heads_index * 2 + (wave >> 1);
+    const int wrow = (wave & 1) * 32;
+    const int kvh = (heads_index * 2) / G;
+    {
+        const int* tile = tiles + (size_t)tile_index * 4;
+        const int req = tile[0], row0 = tile[1], rows = tile[2], pos0 = tile[3];
+        const bool active = wrow < rows;
+        const int* table = block_table + (size_t)req * max_blocks;
+
+        const int my = wrow + q;
+        const bool valid = active && my < rows;
+        const int p = pos0 + min(my, rows - 1);
+        const int hi = valid ? p : 0x7fffffff;
+        const int lo = (valid && window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+        bf16x8 bq[D / 16];
+        {
+            const bf16* qrow = qkv + (size_t)(row0 + min(my, rows - 1)) * q_stride + (size_t)h * D + half * 8;
+#pragma unroll
+            for (int i = 0; i < D / 16; ++i) bq[i] = *reinterpret_cast<const bf16x8*>(qrow + i * 16);
+            prepare_q128_wide(bq, pro, p, half);
+        }
+        const int t_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+        const int first = t_lo / PAGE, last = (pos0 + rows - 1) / PAGE;
+        const int groups = (last - first) / NP + 1;
+        const int w_min = pos0 + min(wrow, rows - 1), w_max = pos0 + min(wrow + 31, rows - 1);
+        const int w_lo_max = (window > 0 && w_max - window + 1 > 0) ? w_max - window + 1 : 0;
+
+        float m_ref = -INFINITY, l_sum = 0.f;
+        floatx16 o[D / 32];
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o[t][v] = 0.f;
+
+        bf16x8 kreg[NP], vreg[NP];
+        int ids_ahead;                  // lane n % 4: page n of the group after the one on its way
+        auto lookup = [&](int g) { ids_ahead = table[min(first + g * NP + (lane & 3), last)]; };
+        auto fetch = [&](const int (&ids)[NP]) {
+#pragma unroll
+            for (int n = 0; n < NP; ++n) {
+                const size_t head = (size_t)ids[n] * nkv + kvh;
+                kreg[n] = *reinterpret_cast<const bf16x8*>(k_cache + head * PAGE * D + tid * 8);
+                vreg[n] = *reinterpret_cast<const bf16x8*>(v_cache + head * D * PAGE + tid * 8);
+            }
+        };
+        auto stage = [&](int g) {
+            bf16* kd = ks[g & 1];
+            bf16* vd = vs[g & 1];
+            const int key = tid >> 4, col = (tid & 15) * 8;
+            const int dim = tid >> 1, hsel = tid & 1, flip = (dim >> 3) & 1;
+#pragma unroll
+            for (int n = 0; n < NP; ++n) {
+                *reinterpret_cast<bf16x8*>(&kd[n * KPAGE + key * KLD + col]) = kreg[n];
+                union { bf16x8 full; short4v h[2]; } both;
+                both.full = vreg[n];
+                *reinterpret_cast<short4v*>(&vd[n * VPAGE + dim * 16 + flip * 8 + hsel * 4]) = both.h[0];
+                *reinterpret_cast<short4v*>(&vd[n * VPAGE + dim * 16 + (flip ^ 1) * 8 + hsel * 4]) = both.h[1];
+            }
+        };
+        {
+            int ids[NP];
+#pragma unroll
+            for (int n = 0; n < NP; ++n) ids[n] = table[min(first + n, last)];
+            fetch(ids);
+            lookup(1);
+        }
+        for (int g = 0; g < groups; ++g) {
+            stage(g);
+            {
+                int ids[NP];
+#pragma unroll
+                for (int n = 0; n < NP; ++n) ids[n] = __builtin_amdgcn_readlane(ids_ahead, n);
+                lookup(g + 2);
+                fetch(ids);             // group g + 1 (past the end: the last page again, unused)
+            }
+            __syncthreads();    // also keeps a fast wave from overwriting the stage a slow one reads
+            const int pg0 = first + g * NP;
+            if (!active) continue;
+            const bf16* kd = ks[g & 1];
+            const bf16* vd = vs[g & 1];
+            floatx16 sc[2];
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) sc[kt][v] = 0.f;
+#pragma unroll
+            for (int i = 0; i < D / 16; ++i)
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt) {
+                    const bf16x8 ka = *reinterpret_cast<const bf16x8*>(&kd[(kt * 32 + q) * KLD + i * 16 + half * 8]);
+                    sc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, bq[i], sc[kt], 0, 0, 0);
+                }
+            if ((pg0 + NP) * PAGE - 1 > w_min || pg0 * PAGE < w_lo_max) {     // the group touches a row's own position or the window's edge
+                const int key0 = pg0 * PAGE + half * 4;
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int j = key0 + kt * 32 + (v >> 2) * 8 + (v & 3);
+                        if (j < lo || j > hi) sc[kt][v] = -INFINITY;
+                    }
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sc[kt][v]);
+            {
+                float a = mx, b = mx;
+                swap_halves(a, b);
+                mx = fmaxf(a, b);
+            }
+            const bool move = mx * scale_log2 > m_ref * scale_log2 + 8.f;   // true while m_ref is -inf
+            const float m_new = move ? mx : m_ref;
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = move ? __builtin_amdgcn_exp2f((m_ref - m_use) * scale_log2) : 1.f;
+            const float neg = -m_use * scale_log2;
+            float psum = 0.f;
+            bf16x8 pb[2][2];
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const float pv = __builtin_amdgcn_exp2f(fmaf(sc[kt][v], scale_log2, neg));
+                    psum += pv;
+                    pb[kt][v >> 3][v & 7] = static_cast<bf16>(pv);
+                }
+            l_sum = l_sum * alpha + psum;
+            m_ref = m_new;
+            if (__any(move)) {
+#pragma unroll
+                for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) o[t][v] *= alpha;
+            }
+#pragma unroll
+            for (int page = 0; page < NP; ++page)
+#pragma unroll
+                for (int t = 0; t < D / 32; ++t) {
+                    const int dim = t * 32 + q;
+                    const bf16x8 va = *reinterpret_cast<const bf16x8*>(
+                        &vd[page * VPAGE + dim * 16 + ((half ^ ((dim >> 3) & 1)) * 8)]);
+                    o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[page >> 1][page & 1], o[t], 0, 0, 0);
+                }
+        }
+        {
+            float a = l_sum, b = l_sum;
+            swap_halves(a, b);
+            const float l = a + b;
+            if (valid) {
+                const float inv = 1.f / l;
+                bf16* orow = out + ((size_t)(row0 + my) * nh + h) * D + half * 4;
+#pragma unroll
+                for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+                    for (int blk = 0; blk < 4; ++blk) {
+                        short4v packed;
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) packed[v] = bf16_bits(o[t][blk * 4 + v] * inv);
+                        *reinterpret_cast<short4v*>(orow + t * 32 + blk * 8) = packed;
+                    }
+            }
+        }
+    }
+}
+
 static int g_decode_waves = 0;   // 0: by the launch's shape
 
 template <int D>
@@ -738,11 +1002,23 @@ static bool prefill_head_pairs(int NT, int nh, int nkv, int splits) {
     return (nh / nkv) % 2 == 0 && ((long long)NT * (nh / 2) > 128 || splits > 1);
 }
 
+static int g_prefill_wide = 1;   // 0: never the kernel built from the wide products (tests, tuning)
+
 template <int D>
 static int launch_prefill(const bf16* qkv, int q_stride, const bf16* k, const bf16* v, bf16* out,
                           const int* tiles, const int* table, int max_blocks, int NT, int nh,
                           int nkv, float scale_log2, int window, DecodePrologue pro, int splits,
                           float* part_o, float* part_ml, hipStream_t s) {
+    if constexpr (D == 128) {
+        // heads of 128 in pairs, every tile's keys walked by one workgroup: the kernel built from
+        // the wide products
+        if (g_prefill_wide && (nh / nkv) % 2 == 0 && splits == 1) {
+            attn_prefill_wide_kernel<D><<<dim3(nh / 2, NT), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
+                                                                       max_blocks, nh, nkv, scale_log2, window, pro);
+            LC_LAUNCH_CHECK("attn_prefill_wide");
+            return 0;
+        }
+    }
     if (prefill_head_pairs(NT, nh, nkv, splits))
         attn_prefill_kernel<D, 2><<<dim3(NT * splits, nh / 2), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
                                                                             max_blocks, nh, nkv, scale_log2, window, pro,
@@ -768,6 +1044,13 @@ LC_API int lc_attn_bf16_supported(int nh, int nkv, int d, int page_size) {
     if (page_size != PAGE || nkv <= 0 || nh % nkv != 0) return 0;
     if (nh / nkv > 16 || nh > 65535 || nkv > 65535) return 0;
     return d == 32 || d == 64 || d == 96 || d == 128;
+}
+
+// Whether heads of 128 in pairs go to the prefill kernel built from the wide products (1, the
+// default) or to the general one (0).  For tests and tuning.
+LC_API int lc_attn_prefill_wide(int on) {
+    g_prefill_wide = on ? 1 : 0;
+    return 0;
 }
 
 // Waves of a decode workgroup (4 or 8; 0: chosen by the launch's shape).  For tests and tuning.

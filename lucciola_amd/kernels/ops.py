@@ -50,6 +50,7 @@ _SIGNATURES = {
     "lc_gemm_bf16_sum_shares": "ppiiiip",
     "lc_attn_prefill_bf16": "pippppp" + "iiiiii" + "f" + "i" + "ipfpi" + "ipp" + "p",
     "lc_attn_prefill_splits": "iiii",
+    "lc_attn_prefill_wide": "i",
     "lc_attn_prefill_prepares_q": "ii",
     "lc_swiglu": "ppiiip",
     "lc_sample": "pppppiip",

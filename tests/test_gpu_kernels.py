@@ -390,6 +390,42 @@ def test_attention_bf16_long_contexts(nh, nkv, d, window):
     close(got, want, torch.bfloat16, atol=attention_atol(torch.bfloat16, vc))
 
 
+@pytest.mark.parametrize("nh,nkv,window", [(8, 2, 0), (4, 2, 100), (6, 1, 33), (2, 1, 0)])
+def test_attention_prefill_of_heads_of_128_in_pairs(nh, nkv, window):
+    """Heads of 128 with an even number of heads per kv head go to the prefill kernel built from
+    32x32x16 products: whole prompts, portions after a history, rows that do not fill a tile,
+    a window whose edge cuts through groups of keys, against the plain formulas and against the
+    general kernel."""
+    d = 128
+    lengths = [700, 64, 333, 1, 2049, 95]
+    new = [700, 64, 130, 1, 300, 31]
+    qkv, batch, kc, vc = paged_case(lengths, new, nh, nkv, d, 16, torch.bfloat16, seed=75)
+    want = ref.attention(qkv.cpu(), AttentionBatch(batch.tok_req.cpu(), batch.positions.cpu(),
+                                                   batch.block_table.cpu()),
+                         kc.cpu(), vc.cpu(), nh, nkv, d, 16, d ** -0.5, window)
+    lib = ops.library()
+    try:
+        lib.lc_attn_prefill_wide(1)
+        got = ops.attention(qkv, batch, kc, vc, nh, nkv, d, 16, d ** -0.5, window)
+        lib.lc_attn_prefill_wide(0)
+        general = ops.attention(qkv, batch, kc, vc, nh, nkv, d, 16, d ** -0.5, window)
+    finally:
+        lib.lc_attn_prefill_wide(1)
+    close(got, want, torch.bfloat16, atol=attention_atol(torch.bfloat16, vc))
+    close(general, want, torch.bfloat16, atol=attention_atol(torch.bfloat16, vc))
+    # a far key that stands out, in the first group of keys of a long tile
+    q2, b2, k2, v2 = paged_case([1500], [1500], nh, nkv, d, 16, torch.bfloat16, seed=76)
+    table = b2.block_table[0].tolist()
+    far = 37
+    k2[table[far // 16], :, far % 16, :] = 0
+    k2[table[far // 16], :, far % 16, 5] = 30.0
+    q2.view(1500, nh + 2 * nkv, d)[1400:, :nh, :] = 0
+    q2.view(1500, nh + 2 * nkv, d)[1400:, :nh, 5] = 30.0
+    out = ops.attention(q2, b2, k2, v2, nh, nkv, d, 16, d ** -0.5, 0).view(1500, nh, d)
+    for h in range(nh):
+        close(out[1450, h], v2[table[far // 16], h // (nh // nkv), :, far % 16], torch.bfloat16)
+
+
 @pytest.mark.parametrize("nh,nkv,d,window,rot,normed", [(32, 8, 128, 0, 128, True), (6, 2, 96, 24, 96, True),
                                                         (8, 1, 64, 0, 32, False), (4, 4, 32, 0, 0, True),
                                                         (16, 1, 32, 0, 32, True)])
