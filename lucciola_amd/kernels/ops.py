@@ -137,6 +137,16 @@ def _need(t: torch.Tensor, what: str, dtype=None, dim: Optional[int] = None) -> 
 
 _c_int, _c_float = ctypes.c_int, ctypes.c_float
 
+_said = set()
+
+
+def _say_once(key, message: str) -> None:
+    """A line on stderr the first time a slow path is taken for these sizes."""
+    if key not in _said:
+        _said.add(key)
+        import sys
+        print(f"[lucciola_amd] {message}", file=sys.stderr, flush=True)
+
 
 # ------------------------------------------------------------------------------ embedding
 def embedding(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
@@ -585,6 +595,11 @@ def attention(qkv, batch: AttentionBatch, k_cache: torch.Tensor,
     lib = library()
     fast = (qkv.dtype == torch.bfloat16 and batch.decode_tokens is not None
             and batch.prefill_tiles is not None and lib.lc_attn_bf16_supported(nh, nkv, d, page_size))
+    if qkv.dtype == torch.bfloat16 and not fast:
+        _say_once(("attention", nh, nkv, d, page_size),
+                  f"bfloat16 attention with {nh} heads, {nkv} kv heads of {d} and pages of {page_size} tokens has no "
+                  "matrix-core kernel (heads of 32, 64, 96 or 128, pages of 16, at most 16 heads a kv head): "
+                  "the general kernel runs, correct and many times slower")
     # who prepares q, k, v (norm, rotation, cache write) when they arrive raw: a step of single
     # tokens does it all inside the decode kernel; otherwise a kernel of its own does k and v,
     # and q too unless both attention kernels can prepare their q themselves

@@ -109,7 +109,25 @@ def test_attention_special_cases():
 
 
 def test_attention_window_counts_the_query_itself():
+    """The reference has no sliding window (its kernels mask by position only,
+    src/kernels/attention.cu:90-92), so what a window means here is the engine's own choice and
+    parity is unpinned: a query at p sees the w positions p - w + 1 .. p.  What pins the plain
+    form: a window of one leaves each row its own value, a window as long as the sequence is
+    no window, and a key that every query loves stops counting exactly w positions later."""
     T, d, w = 12, 8, 4
+    q1, k1, v1 = rnd(T, 2, d), rnd(T, 1, d, seed=1), rnd(T, 1, d, seed=2)
+    torch.testing.assert_close(plain.attention(q1, k1, v1, list(range(T)), window=1),
+                               v1.expand(T, 2, d).contiguous())
+    loved = 3
+    q2, k2, v2 = torch.zeros(T, 1, d, dtype=torch.float64), torch.zeros(T, 1, d, dtype=torch.float64), rnd(T, 1, d, seed=5)
+    q2[:, 0, 0] = 50.0
+    k2[loved, 0, 0] = 50.0
+    seen = plain.attention(q2, k2, v2, list(range(T)), window=w)
+    for t in range(loved, T):
+        if t - loved < w:       # still inside the window: the loved key takes all the weight
+            torch.testing.assert_close(seen[t, 0], v2[loved, 0])
+        else:                   # w positions later it is gone: the mean of the window's values
+            torch.testing.assert_close(seen[t, 0], v2[t - w + 1:t + 1, 0].mean(0))
     q, k, v = rnd(T, 1, d), rnd(T, 1, d, seed=1), rnd(T, 1, d, seed=2)
     got = plain.attention(q, k, v, list(range(T)), window=w)
     for t in range(T):
