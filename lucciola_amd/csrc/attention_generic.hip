@@ -43,13 +43,41 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
     const int g = tid / d_pow2, di = tid % d_pow2;
     const bool pv_active = di < d;
 
+    // Whole 16-byte (8-byte) pieces where the sizes allow it: four lanes share a key's row for
+    // the scores (a wave then reads 16 rows as one contiguous stretch), and a lane takes four
+    // neighbouring keys of its dim at a time for the values (they lie side by side in a page).
+    const bool vec = (d & 15) == 0 && (page_size & 3) == 0;
     float m = -INFINITY, l = 0.f, acc = 0.f;
     for (int c0 = j_lo; c0 <= p; c0 += AG_THREADS) {
         const int j = c0 + tid;
         const bool valid = j <= p;
         float s = -INFINITY;
         long long off = 0;
-        if (valid) {
+        if (vec) {
+            const int part = tid & 3, quarter = d >> 2;
+#pragma unroll 1
+            for (int pass = 0; pass < 4; ++pass) {
+                const int kc = pass * (AG_THREADS / 4) + (tid >> 2), jk = c0 + kc;
+                float dot = 0.f;
+                if (jk <= p) {
+                    const long long head = (long long)table[jk / page_size] * nkv + kvh;
+                    const T* krow = k_cache + (head * page_size + (jk % page_size)) * d + part * quarter;
+                    const float* qp = qs + part * quarter;
+                    for (int i = 0; i < quarter; i += 4) {
+                        float k4[4];
+                        load4(k4, krow + i);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) dot = fmaf(qp[i + e], k4[e], dot);
+                    }
+                }
+                dot += __shfl_xor(dot, 1, kWave);      // the row's four quarters, in a fixed order
+                dot += __shfl_xor(dot, 2, kWave);
+                if (part == 0) ps[kc] = dot;
+            }
+            __syncthreads();
+            if (valid) s = ps[tid];
+            __syncthreads();                            // ps is written again below
+        } else if (valid) {
             const int page = table[j / page_size];
             const long long head = (long long)page * nkv + kvh;
             off = head * d * page_size + (j % page_size);          // of the value column
@@ -70,8 +98,25 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
         acc *= alpha;
         if (pv_active) {
             const int count = min(AG_THREADS, p - c0 + 1);
-            for (int jj = g; jj < count; jj += groups)
-                acc = fmaf(ps[jj], to_f32(v_cache[voff[jj] + (long long)di * page_size]), acc);
+            if (vec) {
+                // runs of four keys that start at a multiple of four lie in one page; a run may
+                // reach over the chunk's ends, where the keys count nothing
+                const int first_run = c0 >> 2, last_run = (c0 + count - 1) >> 2;
+                for (int run = first_run + g; run <= last_run; run += groups) {
+                    const int j4 = run * 4;
+                    const long long head = (long long)table[j4 / page_size] * nkv + kvh;
+                    float v4[4];
+                    load4(v4, v_cache + head * d * page_size + (long long)di * page_size + (j4 % page_size));
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int jj = j4 + e - c0;
+                        if (jj >= 0 && jj < count) acc = fmaf(ps[jj], v4[e], acc);
+                    }
+                }
+            } else {
+                for (int jj = g; jj < count; jj += groups)
+                    acc = fmaf(ps[jj], to_f32(v_cache[voff[jj] + (long long)di * page_size]), acc);
+            }
         }
         __syncthreads();  // ps/voff are rewritten by the next chunk
     }

@@ -36,6 +36,18 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// four consecutive elements as floats, in one load
+__device__ __forceinline__ void load4(float (&dst)[4], const float* p) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+}
+__device__ __forceinline__ void load4(float (&dst)[4], const bf16* p) {
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+    const bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dst[j] = static_cast<float>(v[j]);
+}
+
 // Sum over a workgroup of up to 1024 threads; `scratch` holds one float per wave (16 floats).
 // Every thread gets the total.  The order of the additions is fixed by the thread layout.
 __device__ __forceinline__ float block_sum(float v, float* scratch) {

@@ -4,56 +4,110 @@
 // in_features] row-major, applied as y = x . W^T without bias (reference:
 // src/kernels/linear.cu:24-27, one thread per output element; here LDS-tiled 64x64x16 with a
 // 4x4 register tile per thread).
+//
+// The order of the additions is a function of the output element alone: K is cut into chunks of
+// 256; within a chunk the products are added one after the other from 0, and the chunks' sums
+// are added one after the other from 0.  With few tiles (a decode step: up to 64 rows and a
+// narrow N) the chunks are shared out over workgroups, which leave their sums in a workspace,
+// and a second kernel adds them in the same order: a row's result has the same bits whether it
+// is computed alone or among thousands.
 #include "common.h"
 
 namespace lc {
 
 constexpr int GB_M = 64, GB_N = 64, GB_K = 16;
+constexpr int GB_CHUNK = 256;   // k elements whose products are added up before they join the total
 
+// part == nullptr: out = x . w^T.  Else blockIdx.z owns the chunks [z * per, (z + 1) * per) and
+// writes each chunk's sums to part[chunk][M][N].
 template <typename TX, typename TW, typename TO>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const TX* __restrict__ x,
                                                            const TW* __restrict__ w,
                                                            TO* __restrict__ out, int M, int N,
-                                                           int K) {
+                                                           int K, float* __restrict__ part, int per) {
     __shared__ float xs[GB_K][GB_M + 4];
     __shared__ float ws[GB_K][GB_N + 4];
     const int tid = threadIdx.x;
     const int m0 = blockIdx.y * GB_M, n0 = blockIdx.x * GB_N;
     const int tm = (tid / 16) * 4, tn = (tid % 16) * 4;
-    float acc[4][4] = {};
+    const int chunks = (K + GB_CHUNK - 1) / GB_CHUNK;
+    const int c_begin = part ? blockIdx.z * per : 0;
+    const int c_end = part ? min(c_begin + per, chunks) : chunks;
+    float total[4][4] = {};
 
-    // loader mapping: 64 rows x 16 k; thread loads 4 consecutive k of one row
+    // loader mapping: 64 rows x 16 k; a thread loads 4 consecutive k of one row of x and of w,
+    // a step ahead of the products that use them (the loads of step k0 + 16 are in flight while
+    // step k0 is multiplied)
     const int lrow = tid / 4, lk = (tid % 4) * 4;
-    for (int k0 = 0; k0 < K; k0 += GB_K) {
-        {
-            const int m = m0 + lrow;
+    const bool x_row = m0 + lrow < M, w_row = n0 + lrow < N;
+    const TX* xp = x + (size_t)min(m0 + lrow, M - 1) * K + lk;
+    const TW* wp = w + (size_t)min(n0 + lrow, N - 1) * K + lk;
+    // whole 16-byte (8-byte) pieces where the row length allows it
+    const bool vec = (K & 3) == 0 && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
+    float xr[4], wr[4];
+    auto fetch = [&](int k0) {
+        if (vec && k0 + lk + 3 < K) {
+            load4(xr, xp + k0);
+            load4(wr, wp + k0);
+        } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int k = k0 + lk + j;
-                xs[lk + j][lrow] = (m < M && k < K) ? to_f32(x[(size_t)m * K + k]) : 0.f;
-            }
-            const int n = n0 + lrow;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int k = k0 + lk + j;
-                ws[lk + j][lrow] = (n < N && k < K) ? to_f32(w[(size_t)n * K + k]) : 0.f;
+                xr[j] = k < K ? to_f32(xp[k0 + j]) : 0.f;
+                wr[j] = k < K ? to_f32(wp[k0 + j]) : 0.f;
             }
         }
-        __syncthreads();
+        if (!x_row) { xr[0] = xr[1] = xr[2] = xr[3] = 0.f; }
+        if (!w_row) { wr[0] = wr[1] = wr[2] = wr[3] = 0.f; }
+    };
+    if (c_begin < c_end) fetch(c_begin * GB_CHUNK);
+    for (int c = c_begin; c < c_end; ++c) {
+        float acc[4][4] = {};
+        const int k_end = min(K, (c + 1) * GB_CHUNK);
+        for (int k0 = c * GB_CHUNK; k0 < k_end; k0 += GB_K) {
 #pragma unroll
-        for (int kk = 0; kk < GB_K; ++kk) {
-            float a[4], b[4];
+            for (int j = 0; j < 4; ++j) {
+                xs[lk + j][lrow] = xr[j];
+                ws[lk + j][lrow] = wr[j];
+            }
+            __syncthreads();
+            {   // the step after this one, which may be the first of the next chunk
+                const int next = k0 + GB_K;
+                if (next < k_end || c + 1 < c_end) fetch(next < k_end ? next : (c + 1) * GB_CHUNK);
+            }
 #pragma unroll
-            for (int i = 0; i < 4; ++i) a[i] = xs[kk][tm + i];
+            for (int kk = 0; kk < GB_K; ++kk) {
+                float a[4], b[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) b[j] = ws[kk][tn + j];
+                for (int i = 0; i < 4; ++i) a[i] = xs[kk][tm + i];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) b[j] = ws[kk][tn + j];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+            }
+            __syncthreads();
+        }
+        if (part) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int m = m0 + tm + i;
+                if (m >= M) continue;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int n = n0 + tn + j;
+                    if (n < N) part[((size_t)c * M + m) * N + n] = acc[i][j];
+                }
+            }
+        } else {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+                for (int j = 0; j < 4; ++j) total[i][j] = __fadd_rn(total[i][j], acc[i][j]);
         }
-        __syncthreads();
     }
+    if (part) return;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int m = m0 + tm + i;
@@ -61,17 +115,56 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TX* __restrict_
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int n = n0 + tn + j;
-            if (n < N) out[(size_t)m * N + n] = from_f32<TO>(acc[i][j]);
+            if (n < N) out[(size_t)m * N + n] = from_f32<TO>(total[i][j]);
         }
     }
 }
 
+// out = the chunks' sums part[c][M][N] added one after the other from 0, as the kernel above
+// adds them when it keeps them to itself
+template <typename TO>
+__global__ void gemm_generic_sum_kernel(const float* __restrict__ part, TO* __restrict__ out, size_t MN,
+                                        int chunks) {
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < MN;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        float total = 0.f;
+        for (int c = 0; c < chunks; ++c) total = __fadd_rn(total, part[(size_t)c * MN + idx]);
+        out[idx] = from_f32<TO>(total);
+    }
+}
+
+// Chunks a workgroup takes when they are shared out (0: they are not): with fewer than 1024
+// tiles, as many workgroups as it takes to have about 2048.
+static int chunks_per_workgroup(int M, int N, int K) {
+    const long long tiles = (long long)((N + GB_N - 1) / GB_N) * ((M + GB_M - 1) / GB_M);
+    const int chunks = (K + GB_CHUNK - 1) / GB_CHUNK;
+    if (tiles >= 1024 || chunks < 2) return 0;
+    long long shares = (2048 + tiles - 1) / tiles;
+    if (shares > chunks) shares = chunks;
+    if (shares < 2) return 0;
+    return (int)((chunks + shares - 1) / shares);
+}
+
 template <typename TX, typename TW, typename TO>
-static int launch_generic(const void* x, const void* w, void* out, int M, int N, int K,
+static int launch_generic(const void* x, const void* w, void* out, int M, int N, int K, float* workspace,
                           hipStream_t stream) {
+    const int per = chunks_per_workgroup(M, N, K);
+    const int chunks = (K + GB_CHUNK - 1) / GB_CHUNK;
+    if (per > 0) {
+        LC_CHECK(workspace, "gemm: M=%d N=%d K=%d needs a workspace", M, N, K);
+        dim3 grid((N + GB_N - 1) / GB_N, (M + GB_M - 1) / GB_M, (chunks + per - 1) / per);
+        gemm_generic_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>((const TX*)x, (const TW*)w, (TO*)out, M, N, K,
+                                                                  workspace, per);
+        LC_LAUNCH_CHECK("gemm_generic");
+        const size_t MN = (size_t)M * N;
+        gemm_generic_sum_kernel<TO><<<(int)((MN + 255) / 256 < 4096 ? (MN + 255) / 256 : 4096), 256, 0, stream>>>(
+            workspace, (TO*)out, MN, chunks);
+        LC_LAUNCH_CHECK("gemm_generic_sum");
+        return 0;
+    }
     dim3 grid((N + GB_N - 1) / GB_N, (M + GB_M - 1) / GB_M);
     gemm_generic_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>((const TX*)x, (const TW*)w,
-                                                              (TO*)out, M, N, K);
+                                                              (TO*)out, M, N, K, nullptr, 0);
     LC_LAUNCH_CHECK("gemm_generic");
     return 0;
 }
@@ -80,20 +173,26 @@ static int launch_generic(const void* x, const void* w, void* out, int M, int N,
 
 using namespace lc;
 
+// float32 words of workspace that lc_gemm_generic needs for these sizes (0: none)
+LC_API long long lc_gemm_generic_workspace(int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    return chunks_per_workgroup(M, N, K) > 0 ? (long long)((K + GB_CHUNK - 1) / GB_CHUNK) * M * N : 0;
+}
+
 LC_API int lc_gemm_generic(const void* x, int x_dt, const void* w, int w_dt, void* out, int out_dt,
-                           int M, int N, int K, hipStream_t stream) {
+                           int M, int N, int K, float* workspace, hipStream_t stream) {
     LC_CHECK(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     if (M == 0) return 0;
     LC_CHECK(x && w && out, "gemm: null pointer");
     LC_CHECK((size_t)((M + GB_M - 1) / GB_M) <= 65535, "gemm: M=%d is too large", M);
     const int key = x_dt * 4 + w_dt * 2 + out_dt;
     switch (key) {
-        case 0: return launch_generic<float, float, float>(x, w, out, M, N, K, stream);
-        case 2: return launch_generic<float, bf16, float>(x, w, out, M, N, K, stream);
-        case 4: return launch_generic<bf16, float, float>(x, w, out, M, N, K, stream);
-        case 5: return launch_generic<bf16, float, bf16>(x, w, out, M, N, K, stream);
-        case 6: return launch_generic<bf16, bf16, float>(x, w, out, M, N, K, stream);
-        case 7: return launch_generic<bf16, bf16, bf16>(x, w, out, M, N, K, stream);
+        case 0: return launch_generic<float, float, float>(x, w, out, M, N, K, workspace, stream);
+        case 2: return launch_generic<float, bf16, float>(x, w, out, M, N, K, workspace, stream);
+        case 4: return launch_generic<bf16, float, float>(x, w, out, M, N, K, workspace, stream);
+        case 5: return launch_generic<bf16, float, bf16>(x, w, out, M, N, K, workspace, stream);
+        case 6: return launch_generic<bf16, bf16, float>(x, w, out, M, N, K, workspace, stream);
+        case 7: return launch_generic<bf16, bf16, bf16>(x, w, out, M, N, K, workspace, stream);
         default:
             LC_CHECK(false, "gemm: unsupported dtypes x=%d w=%d out=%d", x_dt, w_dt, out_dt);
     }

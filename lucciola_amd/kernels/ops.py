@@ -26,7 +26,7 @@ _SIGNATURES = {
     "lc_embedding": "ppipiiifp",
     "lc_rmsnorm": "ppppfpiiiipiip",
     "lc_rmsnorm_act": "ppfpiiip",
-    "lc_gemm_generic": "pipipiiiip",
+    "lc_gemm_generic": "pipipiiiipp",
     "lc_gemm_bf16": "pppiiiiipp",
     "lc_gemm_bf16_supported": "iii",
     "lc_gemm_bf16_force_tile": "i",
@@ -83,6 +83,8 @@ def library():
         lib.lc_last_error.restype = ctypes.c_char_p
         lib.lc_gemm_bf16_workspace.restype = ctypes.c_longlong
         lib.lc_gemm_bf16_workspace.argtypes = [ctypes.c_int] * 3
+        lib.lc_gemm_generic_workspace.restype = ctypes.c_longlong
+        lib.lc_gemm_generic_workspace.argtypes = [ctypes.c_int] * 3
         for name, sig in _SIGNATURES.items():
             fn = getattr(lib, name, None)
             if fn is None:
@@ -346,8 +348,10 @@ def gemm(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None, defer: boo
         _call("lc_gemm_bf16", _ptr(x), _ptr(w), _ptr(out), _c_int(_dt(out)), _c_int(M), _c_int(N),
               _c_int(K), 0, _ptr(_gemm_workspace(M, N, K, x.device)), _stream())
     else:
+        words = library().lc_gemm_generic_workspace(M, N, K)
+        workspace = torch.empty((words,), dtype=torch.float32, device=x.device) if words else None
         _call("lc_gemm_generic", _ptr(x), _c_int(_dt(x)), _ptr(w), _c_int(_dt(w)), _ptr(out),
-              _c_int(_dt(out)), _c_int(M), _c_int(N), _c_int(K), _stream())
+              _c_int(_dt(out)), _c_int(M), _c_int(N), _c_int(K), _ptr(workspace), _stream())
     return out
 
 
