@@ -3,7 +3,7 @@
 // is a true 32-bit product).  The weight layout is the checkpoint's: [out_features,
 // in_features] row-major, applied as y = x . W^T without bias (reference:
 // src/kernels/linear.cu:24-27, one thread per output element; here LDS-tiled 64x64x16 with a
-// 4x4 register tile per thread).
+// 4x4 register tile per thread; up to 16 rows: 16x64x16 with four rows of a column per thread).
 //
 // The order of the additions is a function of the output element alone: K is cut into chunks of
 // 256; within a chunk the products are added one after the other from 0, and the chunks' sums
@@ -120,6 +120,93 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TX* __restrict_
     }
 }
 
+// The same product for up to 16 rows of x (a decode step): tiles of 16 x 64, a thread owns four
+// rows of one column and reads four k of both operands at a time.  Every output element sees
+// the same operations in the same order as in the kernel above.
+constexpr int GF_M = 16;
+
+template <typename TX, typename TW, typename TO>
+__global__ __launch_bounds__(256) void gemm_generic_few_kernel(const TX* __restrict__ x,
+                                                               const TW* __restrict__ w,
+                                                               TO* __restrict__ out, int M, int N,
+                                                               int K, float* __restrict__ part, int per) {
+    __shared__ __align__(16) float xs[GF_M][GB_K];
+    __shared__ __align__(16) float ws[GB_N][GB_K + 4];
+    const int tid = threadIdx.x;
+    const int m0 = blockIdx.y * GF_M, n0 = blockIdx.x * GB_N;
+    const int tn = tid % GB_N, tm = (tid / GB_N) * 4;
+    const int chunks = (K + GB_CHUNK - 1) / GB_CHUNK;
+    const int c_begin = part ? blockIdx.z * per : 0;
+    const int c_end = part ? min(c_begin + per, chunks) : chunks;
+    float total[4] = {};
+
+    const int lrow = tid / 4, lk = (tid % 4) * 4;
+    const bool x_loader = lrow < GF_M, x_row = x_loader && m0 + lrow < M, w_row = n0 + lrow < N;
+    const TX* xp = x + (size_t)min(m0 + lrow, M - 1) * K + lk;
+    const TW* wp = w + (size_t)min(n0 + lrow, N - 1) * K + lk;
+    const bool vec = (K & 3) == 0 && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
+    float xr[4] = {}, wr[4];
+    auto fetch = [&](int k0) {
+        if (vec && k0 + lk + 3 < K) {
+            if (x_row) load4(xr, xp + k0);
+            load4(wr, wp + k0);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int k = k0 + lk + j;
+                xr[j] = (x_row && k < K) ? to_f32(xp[k0 + j]) : 0.f;
+                wr[j] = k < K ? to_f32(wp[k0 + j]) : 0.f;
+            }
+        }
+        if (!x_row) { xr[0] = xr[1] = xr[2] = xr[3] = 0.f; }
+        if (!w_row) { wr[0] = wr[1] = wr[2] = wr[3] = 0.f; }
+    };
+    if (c_begin < c_end) fetch(c_begin * GB_CHUNK);
+    for (int c = c_begin; c < c_end; ++c) {
+        float acc[4] = {};
+        const int k_end = min(K, (c + 1) * GB_CHUNK);
+        for (int k0 = c * GB_CHUNK; k0 < k_end; k0 += GB_K) {
+            if (x_loader) *reinterpret_cast<float4*>(&xs[lrow][lk]) = make_float4(xr[0], xr[1], xr[2], xr[3]);
+            *reinterpret_cast<float4*>(&ws[lrow][lk]) = make_float4(wr[0], wr[1], wr[2], wr[3]);
+            __syncthreads();
+            {
+                const int next = k0 + GB_K;
+                if (next < k_end || c + 1 < c_end) fetch(next < k_end ? next : (c + 1) * GB_CHUNK);
+            }
+#pragma unroll
+            for (int kk = 0; kk < GB_K; kk += 4) {
+                const float4 b = *reinterpret_cast<const float4*>(&ws[tn][kk]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float4 a = *reinterpret_cast<const float4*>(&xs[tm + i][kk]);
+                    acc[i] = fmaf(a.x, b.x, acc[i]);
+                    acc[i] = fmaf(a.y, b.y, acc[i]);
+                    acc[i] = fmaf(a.z, b.z, acc[i]);
+                    acc[i] = fmaf(a.w, b.w, acc[i]);
+                }
+            }
+            __syncthreads();
+        }
+        const int n = n0 + tn;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int m = m0 + tm + i;
+            if (part) {
+                if (m < M && n < N) part[((size_t)c * M + m) * N + n] = acc[i];
+            } else {
+                total[i] = __fadd_rn(total[i], acc[i]);
+            }
+        }
+    }
+    if (part) return;
+    const int n = n0 + tn;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + tm + i;
+        if (m < M && n < N) out[(size_t)m * N + n] = from_f32<TO>(total[i]);
+    }
+}
+
 // out = the chunks' sums part[c][M][N] added one after the other from 0, as the kernel above
 // adds them when it keeps them to itself
 template <typename TO>
@@ -150,11 +237,16 @@ static int launch_generic(const void* x, const void* w, void* out, int M, int N,
                           hipStream_t stream) {
     const int per = chunks_per_workgroup(M, N, K);
     const int chunks = (K + GB_CHUNK - 1) / GB_CHUNK;
+    const bool few = M <= GF_M;
     if (per > 0) {
         LC_CHECK(workspace, "gemm: M=%d N=%d K=%d needs a workspace", M, N, K);
-        dim3 grid((N + GB_N - 1) / GB_N, (M + GB_M - 1) / GB_M, (chunks + per - 1) / per);
-        gemm_generic_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>((const TX*)x, (const TW*)w, (TO*)out, M, N, K,
-                                                                  workspace, per);
+        dim3 grid((N + GB_N - 1) / GB_N, few ? 1 : (M + GB_M - 1) / GB_M, (chunks + per - 1) / per);
+        if (few)
+            gemm_generic_few_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>((const TX*)x, (const TW*)w, (TO*)out, M,
+                                                                          N, K, workspace, per);
+        else
+            gemm_generic_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>((const TX*)x, (const TW*)w, (TO*)out, M, N,
+                                                                      K, workspace, per);
         LC_LAUNCH_CHECK("gemm_generic");
         const size_t MN = (size_t)M * N;
         gemm_generic_sum_kernel<TO><<<(int)((MN + 255) / 256 < 4096 ? (MN + 255) / 256 : 4096), 256, 0, stream>>>(
@@ -162,9 +254,13 @@ static int launch_generic(const void* x, const void* w, void* out, int M, int N,
         LC_LAUNCH_CHECK("gemm_generic_sum");
         return 0;
     }
-    dim3 grid((N + GB_N - 1) / GB_N, (M + GB_M - 1) / GB_M);
-    gemm_generic_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>((const TX*)x, (const TW*)w,
-                                                              (TO*)out, M, N, K, nullptr, 0);
+    dim3 grid((N + GB_N - 1) / GB_N, few ? 1 : (M + GB_M - 1) / GB_M);
+    if (few)
+        gemm_generic_few_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>((const TX*)x, (const TW*)w, (TO*)out, M, N,
+                                                                      K, nullptr, 0);
+    else
+        gemm_generic_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>((const TX*)x, (const TW*)w, (TO*)out, M, N, K,
+                                                                  nullptr, 0);
     LC_LAUNCH_CHECK("gemm_generic");
     return 0;
 }

@@ -41,7 +41,7 @@ _SIGNATURES = {
     "lc_gemm_bf16_scaled_rows": "pppiiiipifp",
     "lc_gemm_bf16_scaled_rows_supported": "iii",
     "lc_qk_norm_rope_write": "piiiiippfppipppiip",
-    "lc_attention_generic": "pipppipppiiiiiifip",
+    "lc_attention_generic": "pipppipppiiiiiifipp",
     "lc_attn_bf16_supported": "iiii",
     "lc_attn_decode_splits": "iii",
     "lc_attn_decode_waves": "i",
@@ -85,6 +85,8 @@ def library():
         lib.lc_gemm_bf16_workspace.argtypes = [ctypes.c_int] * 3
         lib.lc_gemm_generic_workspace.restype = ctypes.c_longlong
         lib.lc_gemm_generic_workspace.argtypes = [ctypes.c_int] * 3
+        lib.lc_attention_generic_workspace.restype = ctypes.c_longlong
+        lib.lc_attention_generic_workspace.argtypes = [ctypes.c_int] * 5
         for name, sig in _SIGNATURES.items():
             fn = getattr(lib, name, None)
             if fn is None:
@@ -655,10 +657,13 @@ def attention(qkv, batch: AttentionBatch, k_cache: torch.Tensor,
                   _c_float(prologue.eps if own_q else 0.0), _ptr(rope if own_q else None),
                   rot if own_q else 0, pf_splits, _ptr(pf_o), _ptr(pf_ml), _stream())
         return out
+    words = lib.lc_attention_generic_workspace(T, nh, nkv, batch.block_table.shape[1], page_size)
+    workspace = torch.empty((words,), dtype=torch.float32, device=qkv.device) if words else None
     _call("lc_attention_generic", _ptr(qkv), _c_int(qkv.shape[1]), _ptr(k_cache), _ptr(v_cache),
           _ptr(out), _c_int(_dt(qkv)), _ptr(batch.tok_req), _ptr(batch.positions),
           _ptr(batch.block_table), _c_int(batch.block_table.shape[1]), _c_int(T), _c_int(nh),
-          _c_int(nkv), _c_int(d), _c_int(page_size), _c_float(scale), _c_int(window), _stream())
+          _c_int(nkv), _c_int(d), _c_int(page_size), _c_float(scale), _c_int(window),
+          _ptr(workspace), _stream())
     return out
 
 

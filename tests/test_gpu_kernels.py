@@ -82,13 +82,27 @@ def test_rmsnorm_eps_matters():
     (torch.float32, torch.float32, torch.float32), (torch.float32, torch.bfloat16, torch.float32),
     (torch.bfloat16, torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.bfloat16, torch.float32),
     (torch.bfloat16, torch.float32, torch.bfloat16)])
-@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (3, 331, 72), (65, 130, 200), (64, 64, 16), (17, 1000, 257)])
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (3, 331, 72), (65, 130, 200), (64, 64, 16), (17, 1000, 257),
+                                   (16, 200, 1030), (9, 70, 515)])
 def test_gemm_generic(dt_x, dt_w, dt_o, M, N, K):
     x = rnd(M, K, dtype=dt_x, seed=7)
     w = rnd(N, K, dtype=dt_w, seed=8)
     got = ops.gemm(x, w, dt_o)
     want = ref.gemm(x, w, dt_o)
     close(got, want, dt_o, scale=K ** 0.5)
+
+
+@pytest.mark.parametrize("K", [600, 601, 256, 77])
+def test_gemm_generic_same_bits_for_any_number_of_rows(K):
+    """A row's float32 product has the same bits alone (tiles of 16 rows, K shared out over
+    workgroups), among a few dozen rows and among a thousand (tiles of 64 rows, K not shared)."""
+    x = rnd(1100, K, seed=11)
+    w = rnd(3700, K, seed=12)
+    whole = ops.gemm(x, w, torch.float32)
+    close(whole, ref.gemm(x, w, torch.float32), torch.float32, scale=K ** 0.5)
+    for first, count in ((0, 7), (500, 1), (1084, 16), (30, 40)):
+        rows = ops.gemm(x[first:first + count].contiguous(), w, torch.float32)
+        assert torch.equal(rows, whole[first:first + count]), (first, count)
 
 
 def make_rope_table(positions, rot, theta):
@@ -173,6 +187,28 @@ def test_attention_mixed_batch(dtype, nh, nkv, d, page, window):
                                                    batch.block_table.cpu()),
                          kc.cpu(), vc.cpu(), nh, nkv, d, page, d ** -0.5, window)
     close(got, want, dtype, atol=attention_atol(dtype, vc))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,page,window", [(6, 2, 48, 16, 0), (6, 2, 48, 16, 700), (10, 2, 20, 8, 0),
+                                                   (4, 4, 128, 16, 1100)])
+def test_attention_general_kernel_same_bits_alone_and_in_a_prompt(dtype, nh, nkv, d, page, window):
+    """The last tokens of a long prompt, once as rows of the whole prompt (one workgroup works
+    through all their keys) and once alone (the keys are shared out over workgroups and joined
+    by a second kernel): the same bits, and both near the plain result."""
+    if dtype == torch.bfloat16 and ops.library().lc_attn_bf16_supported(nh, nkv, d, page):
+        pytest.skip("these sizes have a matrix-core kernel in bfloat16")
+    length, whole, alone = 1500, 700, 5
+    qkv, batch, kc, vc = paged_case([length], [whole], nh, nkv, d, page, dtype, seed=26)
+    got = ops.attention(qkv, batch, kc, vc, nh, nkv, d, page, d ** -0.5, window)
+    want = ref.attention(qkv.cpu(), AttentionBatch(batch.tok_req.cpu(), batch.positions.cpu(),
+                                                   batch.block_table.cpu()),
+                         kc.cpu(), vc.cpu(), nh, nkv, d, page, d ** -0.5, window)
+    close(got, want, dtype, atol=attention_atol(dtype, vc))
+    _, few, kc2, vc2 = paged_case([length], [alone], nh, nkv, d, page, dtype, seed=26)
+    assert torch.equal(kc2, kc) and torch.equal(few.block_table, batch.block_table)
+    tail = ops.attention(qkv[-alone:].contiguous(), few, kc, vc, nh, nkv, d, page, d ** -0.5, window)
+    assert torch.equal(tail, got[-alone:])
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
