@@ -52,6 +52,16 @@ __device__ __forceinline__ float swiglu_f(float g, float u) {
     return g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u;
 }
 
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef __attribute__((address_space(1))) const void* glb_ptr_t;
+
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));   // other counters untouched
+}
+template <int N> __device__ __forceinline__ void wait_lgkmcnt() {
+    __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));
+}
+
 // ------------------------------------------------------------------------------- skinny
 constexpr int SK_KBLOCK = 128; // k elements per wave iteration
 
@@ -319,6 +329,250 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
     }
 }
 
+// ------------------------------------------------------------------------------- skinny, rows in runs
+// The same product (up to 16 rows of x, tiles of up to 16 rows of w, the same epilogues), with
+// w read as memory likes it.  The matrix-core operand of the kernel above makes every load
+// instruction fetch 64 bytes of each of 16 rows of w, which are K elements apart: measured,
+// such loads move 4.2 to 4.4 TB/s where loads of 1 KB runs move 5.4 to 6.0.  Here a wave's load
+// instruction takes 1 KB of ONE row (512 k) straight into LDS (global_load_lds_dwordx4), the 16
+// waves of a workgroup fill one stage (16 rows x 512 k) of a ring of eight, and the operands
+// are read from LDS: wave q multiplies the k-step q of every stage (32 k, one product), so a
+// wave needs of x only its own K / 16 columns, which it keeps in registers.  Within a row the
+// 16-byte chunk c lies at place c ^ row: the 16 lanes that LDS serves together (16 rows, one
+// chunk) then use all banks.  The ring runs on across the workgroup's tiles; a stage is
+// reused one barrier after its last reader.  Counted waits and raw barriers: the compiler
+// would wait for all loads in flight at every LDS access and barrier.
+constexpr int SR_K = 512;             // k elements of a run
+constexpr int SR_RING = 8;
+constexpr int SR_STAGE = 16 * SR_K;   // bf16 elements of a stage
+
+__device__ __forceinline__ void lds_put(unsigned addr, float v) {
+    asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(v) : "memory");
+}
+__device__ __forceinline__ float lds_get(unsigned addr) {
+    float v;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+}
+
+// at most min(n, MAXN) of the youngest loads may still be in flight
+template <int MAXN> __device__ __forceinline__ void wait_vmcnt_upto(int n) {
+    static_assert(MAXN == 6 || MAXN == 12, "the cases below");
+    if (n >= MAXN) { wait_vmcnt<MAXN>(); return; }
+    if (MAXN == 12) n >>= 1;      // even numbers only: two loads a stage
+    switch (n) {
+    case 0: wait_vmcnt<0>(); break;
+    case 1: wait_vmcnt<MAXN / 6>(); break;
+    case 2: wait_vmcnt<2 * (MAXN / 6)>(); break;
+    case 3: wait_vmcnt<3 * (MAXN / 6)>(); break;
+    case 4: wait_vmcnt<4 * (MAXN / 6)>(); break;
+    default: wait_vmcnt<5 * (MAXN / 6)>(); break;
+    }
+}
+// a barrier for LDS written by ordinary stores (it does not wait for global loads in flight)
+__device__ __forceinline__ void raw_barrier() {
+    wait_lgkmcnt<0>();
+    asm volatile("s_barrier" : : : "memory");
+}
+
+// XS > 0 (K <= XS * 512): a wave keeps its columns of x in registers for all of its workgroup's
+// tiles.  XS = 0 (any K): a wave's 16 bytes of x for a stage travel with the stage's run of w,
+// seven stages ahead, into a ring of registers.
+template <int EPI, bool SCALE, int XS, typename TO>
+__global__ __launch_bounds__(1024) void gemm_runs_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
+                                                         TO* __restrict__ out, int M, int N, int K, int rows,
+                                                         SkinnyFuse fuse) {
+    constexpr int RS = 256 + 4;        // a wave's 256 sums, padded
+    constexpr int PER = XS > 0 ? 1 : 2;   // loads a wave issues per stage
+    __shared__ __attribute__((aligned(1024))) bf16 ring[SR_RING * SR_STAGE];
+    __shared__ float red[16 * RS];
+    __shared__ float part_sq[16][16];
+    __shared__ float factors[16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, g = lane >> 4;
+    const int tiles = (N + rows - 1) / rows;
+    if ((int)blockIdx.x >= tiles) return;
+    const int spt = K / SR_K;                                        // stages per tile
+    const int my_tiles = (tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    const int total_stages = my_tiles * spt;
+    const unsigned ring0 = (unsigned)(uintptr_t)(lds_ptr_t)ring;
+    const unsigned red0 = (unsigned)(uintptr_t)(lds_ptr_t)red;
+
+    // this wave's columns of x: of every stage the k-step `wave`
+    const bf16* xp = x + (size_t)min(r, M - 1) * K + wave * 32 + g * 8;
+    bf16x8 xr[XS > 0 ? XS : SR_RING];
+    if (XS > 0) {
+#pragma unroll
+        for (int s = 0; s < XS; ++s) xr[s] = *reinterpret_cast<const bf16x8*>(xp + min(s, spt - 1) * SR_K);
+    }
+    float piece[SK_MAX_PIECES / 64];
+    if (SCALE) {
+#pragma unroll
+        for (int i = 0; i < SK_MAX_PIECES / 64; ++i) {   // thread t: row t % stride of pieces t / stride + ...
+            const int at = threadIdx.x + 1024 * i;
+            piece[i] = at < fuse.scale_count * fuse.stride ? fuse.scale_partials[at] : 0.f;
+        }
+    }
+
+    // the loads of the ring, in the order of the stages: wave q fetches row q of the stage's tile
+    int issue_tile = blockIdx.x, issue_s = 0, issued = 0;
+    auto issue = [&](bf16x8& x_to) {
+        const int n0 = issue_tile * rows, n_end = min(N, n0 + rows);
+        const int row = min(n0 + wave, n_end - 1);
+        const bf16* src = w + (size_t)row * K + issue_s * SR_K + ((lane ^ wave) * 8);
+        __builtin_amdgcn_global_load_lds((glb_ptr_t)src,
+            (lds_ptr_t)(ring + (issued & (SR_RING - 1)) * SR_STAGE + wave * SR_K), 16, 0, 0);
+        if (XS == 0) asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(x_to) : "v"(xp + issue_s * SR_K) : "memory");
+        ++issued;
+        if (++issue_s == spt) { issue_s = 0; issue_tile += gridDim.x; }
+    };
+#pragma unroll
+    for (int i = 0; i < SR_RING - 1; ++i)
+        if (issued < total_stages) issue(xr[XS > 0 ? 0 : i]);
+
+    float factor = 1.f;                  // of the row that this thread's results belong to (m = thread / 16)
+    if (SCALE) {
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < SK_MAX_PIECES / 64; ++i) sum += piece[i];
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1)
+            if (off >= fuse.stride) sum += __shfl_xor(sum, off, 64);
+        if (lane < fuse.stride) part_sq[wave][lane] = sum;
+        raw_barrier();
+        if (threadIdx.x < 16) {
+            float ss = 0.f;
+            if ((int)threadIdx.x < fuse.stride)
+#pragma unroll
+                for (int wv = 0; wv < 16; ++wv) ss += part_sq[wv][threadIdx.x];
+            factors[threadIdx.x] = rsqrtf(ss / (float)K + fuse.scale_eps);
+        }
+        raw_barrier();
+        factor = factors[(threadIdx.x >> 4) & 15];
+    }
+
+    // the operand of this lane in a stage: row r, chunk 4 wave + g, at place chunk ^ r
+    const unsigned a_at = ring0 + (r * SR_K + (((wave * 4 + g) ^ r) * 8)) * 2;
+    // a thread of the first four waves owns the result (row e_m of x, row e_j of the tile)
+    const int e_m = (threadIdx.x >> 4) & 15, e_j = threadIdx.x & 15;
+    int stage_at = 0;
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    float e_resid = 0.f, e_w = 0.f;
+    auto begin_tile = [&](int tile) {
+        const int n0 = tile * rows, n_end = min(N, n0 + rows);
+        acc = floatx4{0.f, 0.f, 0.f, 0.f};
+        if (EPI == 2 && threadIdx.x < 256 && e_m < M && n0 + e_j < n_end) {
+            e_resid = fuse.resid[(size_t)e_m * N + n0 + e_j];
+            e_w = fuse.next_w[n0 + e_j];
+        }
+    };
+    // one stage: x_use holds this wave's x of the stage; the load of the stage seven on brings its x to x_fill
+    auto stage = [&](const bf16x8& x_use, bf16x8& x_fill) {
+        wait_vmcnt_upto<PER * (SR_RING - 2)>(PER * (issued - stage_at - 1));   // this wave's loads of the stage have landed
+        __builtin_amdgcn_s_barrier();         // everybody's have; nobody reads the stage before any more
+        __builtin_amdgcn_sched_barrier(0);
+        bf16x8 b = x_use;
+        if (XS == 0) asm volatile("" : "+v"(b));
+        if (issued < total_stages) issue(x_fill);   // into the stage before
+        bf16x8 a;
+        asm volatile("ds_read_b128 %0, %1" : "=v"(a) : "v"(a_at + (stage_at & (SR_RING - 1)) * (SR_STAGE * 2)));
+        wait_lgkmcnt<0>();
+        asm volatile("" : "+v"(a));
+        __builtin_amdgcn_sched_barrier(0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+        ++stage_at;
+    };
+    auto end_tile = [&](int tile) {
+        const int n0 = tile * rows, n_end = min(N, n0 + rows);
+        // acc[v] = this wave's part of out[m = lane % 16][n = n0 + 4 (lane / 16) + v]; kept at red[wave][16 m + n - n0].
+        // The stores are inline assembly, where the compiler does not see that they read what the last product
+        // writes: the wait states between a matrix-core write and an LDS read of the same registers (up to 19).
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_nop 15\n\ts_nop 3");
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) lds_put(red0 + (wave * RS + r * 16 + g * 4 + v) * 4, acc[v]);
+        wait_lgkmcnt<0>();
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        if (threadIdx.x < 256) {
+            // the sum over the waves of this thread's element, and for SwiGLU of the up row eight further on
+            auto sum_of = [&](int e) {
+                float t = 0.f;
+#pragma unroll
+                for (int w0 = 0; w0 < 16; w0 += 4) {
+                    float got[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) got[k] = lds_get(red0 + ((w0 + k) * RS + e) * 4);
+                    wait_lgkmcnt<0>();
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        asm volatile("" : "+v"(got[k]));
+                        t += got[k];
+                    }
+                }
+                return t;
+            };
+            const float t = sum_of(threadIdx.x);
+            float t_up = 0.f;
+            if (EPI == 1) t_up = sum_of(threadIdx.x | 8);
+            const int n = n0 + e_j;
+            const bool mine = e_m < M && n < n_end;
+            if (EPI == 0) {
+                if (mine) store_out<TO>(out + (size_t)e_m * N + n, t * factor);
+            } else if (EPI == 1) {
+                // rows of w come in blocks of 16: 8 gate rows, then their 8 up rows; out has N / 2 columns
+                if (mine && e_j < 8)
+                    store_out<TO>(out + (size_t)e_m * (N / 2) + (n >> 4) * 8 + (n & 7), swiglu_f(t * factor, t_up * factor));
+            } else {
+                float sq = 0.f;
+                if (mine) {
+                    const float v = e_resid + t;
+                    fuse.resid[(size_t)e_m * N + n] = v;
+                    fuse.next_x[(size_t)e_m * N + n] = static_cast<bf16>(v * e_w);
+                    sq = v * v;
+                }
+                // a row's squares over the tile's columns: the 16 neighbouring lanes of a row of lanes
+                sq += lane_swap<0xB1>(sq);                                   // lane ^ 1
+                sq += lane_swap<0x4E>(sq);                                   // lane ^ 2
+                sq += __shfl_xor(sq, 4, 64);
+                sq += __shfl_xor(sq, 8, 64);
+                if (e_j == 0 && e_m < fuse.stride) fuse.next_partials[(size_t)tile * fuse.stride + e_m] = sq;
+            }
+        }
+        // red is written again after the next tile's stages, each of which has a barrier of its own
+    };
+
+    if constexpr (XS > 0) {
+        for (int ti = 0; ti < my_tiles; ++ti) {
+            const int tile = blockIdx.x + ti * gridDim.x;
+            begin_tile(tile);
+#pragma unroll
+            for (int s = 0; s < XS; ++s)
+                if (s < spt) stage(xr[s], xr[s]);
+            end_tile(tile);
+        }
+    } else {
+        // the ring of x is indexed by the stage's number among all of the workgroup's: eight at a time
+        int tile = blockIdx.x, s_in = 0;
+        begin_tile(tile);
+        for (int st0 = 0; st0 < total_stages; st0 += SR_RING) {
+#pragma unroll
+            for (int k = 0; k < SR_RING; ++k) {
+                if (st0 + k < total_stages) {
+                    stage(xr[k], xr[(k + SR_RING - 1) % SR_RING]);
+                    if (++s_in == spt) {
+                        end_tile(tile);
+                        s_in = 0;
+                        tile += gridDim.x;
+                        if (st0 + k + 1 < total_stages) begin_tile(tile);
+                    }
+                }
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------- tiled
 // Workgroup tile BM x BN x 64, four waves in a 2 x 2 grid, each owning (BM/64) x (BN/64) tiles
 // of 32 x 32.
@@ -339,15 +593,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 // have finished reading the stage that the next loads overwrite) and reads the next block's
 // first operands while the rest of its products run.  sched_barrier pins that order.
 constexpr int TL_K = 64;
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-typedef __attribute__((address_space(1))) const void* glb_ptr_t;
-
-template <int N> __device__ __forceinline__ void wait_vmcnt() {
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));   // other counters untouched
-}
-template <int N> __device__ __forceinline__ void wait_lgkmcnt() {
-    __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));
-}
 
 // The grid's workgroups take the tiles [tile_base, tile_base + tile_count) of the tiles_m x
 // tiles_n tiles of the product.
@@ -839,10 +1084,29 @@ static int skinny_shape(int M, int N, int K) {
 // keeps them).
 struct SkinnyPlan {
     int shape, rows, items, groups;
+    bool runs;      // the kernel that reads w in runs of 1 KB
 };
 static int g_even_rows = 1;
+static int g_runs = 1;
 static SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
     SkinnyPlan p;
+    p.runs = false;
+    // (measured at 8 rows: 201 MB of w 41.8 -> 38.7 us, 100 MB 24.8 -> 22.3, 1.2 GB 221 -> 213; 50 MB 12.4 -> 13.5 and
+    // 34 MB 9.8 -> 10.1: the ring's start and the barrier of every stage cost the small ones more than the runs gain)
+    if (g_runs && g_force_skinny < 0 && K % SR_K == 0 && (g_runs > 1 || (long long)N * K >= (1ll << 25))) {
+        // tiles of 16 rows, or of as many as give every CU the same number (the SwiGLU epilogue keeps whole blocks of 16)
+        p.runs = true;
+        p.shape = SKINNY_PLAIN;
+        p.rows = 16;
+        p.items = (N + 15) / 16;
+        const int per_cu = (p.items + kCUs - 1) / kCUs;
+        if (g_even_rows && epilogue != 1 && p.items > kCUs && p.items % kCUs != 0 && per_cu <= 4) {
+            p.rows = (N + kCUs * per_cu - 1) / (kCUs * per_cu);
+            p.items = (N + p.rows - 1) / p.rows;
+        }
+        p.groups = p.items < kCUs ? p.items : kCUs;
+        return p;
+    }
     p.shape = skinny_shape(M, N, K);
     p.rows = p.shape == SKINNY_WIDE ? 32 : 16;
     p.items = (N + p.rows - 1) / p.rows;
@@ -868,6 +1132,13 @@ template <int EPI, bool SCALE, typename TO>
 static void launch_skinny_any(const bf16* x, const bf16* w, TO* out, int M, int N, int K, SkinnyFuse fuse,
                               hipStream_t s) {
     const SkinnyPlan p = skinny_plan(M, N, K, EPI);
+    if (p.runs) {
+        const int spt = K / SR_K;
+        // x stays in registers where a workgroup has several tiles to use it for
+        if (spt <= 8 && p.items > p.groups) gemm_runs_kernel<EPI, SCALE, 8, TO><<<p.groups, 1024, 0, s>>>(x, w, out, M, N, K, p.rows, fuse);
+        else gemm_runs_kernel<EPI, SCALE, 0, TO><<<p.groups, 1024, 0, s>>>(x, w, out, M, N, K, p.rows, fuse);
+        return;
+    }
     const int per_wave = (K / SK_KBLOCK + 15) / 16;
     switch (p.shape) {
     case SKINNY_DEEP: launch_skinny<1, 1, 16, 4, EPI, SCALE, 0, TO>(x, w, out, M, N, K, p.rows, fuse, p.groups, s); break;
@@ -1009,6 +1280,14 @@ LC_API int lc_gemm_bf16(const void* x, const void* w, void* out, int out_dt, int
 
 // 0: work items of 16 or 32 rows whatever N is; 1 (the default): N cut into equal items where
 // that gives every CU the same number of rows.  For tests and tuning.
+// Whether products of up to 16 rows read w in runs of 1 KB through LDS: where K allows it and w
+// is large enough to gain (1, the default), wherever K allows it (2), never (0).  For tests
+// and tuning.
+LC_API int lc_gemm_bf16_runs(int on) {
+    g_runs = on;
+    return 0;
+}
+
 LC_API int lc_gemm_bf16_even_rows(int on) {
     g_even_rows = on ? 1 : 0;
     return 0;

@@ -32,6 +32,7 @@ _SIGNATURES = {
     "lc_gemm_bf16_force_tile": "i",
     "lc_gemm_bf16_force_skinny": "i",
     "lc_gemm_bf16_even_rows": "i",
+    "lc_gemm_bf16_runs": "i",
     "lc_gemm_bf16_small_partials": "i",
     "lc_gemm_bf16_residual_pieces": "iii",
     "lc_gemm_bf16_piece_stride": "i",
@@ -407,6 +408,13 @@ def gemm_even_rows(on: bool) -> None:
     """Whether the bfloat16 product of up to 16 rows may cut N into work items of fewer than 16
     rows so that every CU gets the same number (on by default).  For tests and tuning."""
     _call("lc_gemm_bf16_even_rows", _c_int(1 if on else 0))
+
+
+def gemm_runs(mode) -> None:
+    """Whether the bfloat16 product of up to 16 rows reads w in runs of 1 KB through LDS: where K
+    is a multiple of 512 and w is large enough to gain (1 or True, the default), wherever K is
+    a multiple of 512 (2), never (0 or False).  For tests and tuning."""
+    _call("lc_gemm_bf16_runs", _c_int(int(mode)))
 
 
 def force_gemm_skinny(shape: int) -> None:

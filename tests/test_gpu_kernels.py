@@ -334,12 +334,24 @@ def test_gemm_bf16_last_round_cut_along_k(tile, M, N, K):
 
 @pytest.mark.parametrize("M,H,K,N2", [(1, 5120, 128, 6160), (8, 5120, 256, 10250), (16, 6272, 384, 5130),
                                       (1, 128, 128, 48), (2, 384, 256, 1000), (5, 256, 640, 272), (8, 4096, 512, 2064),
-                                      (11, 640, 128, 16), (12, 16384, 6272, 16416), (12, 8192, 128, 48), (16, 1152, 384, 130)])
-def test_norm_folded_into_the_products_around_it(M, H, K, N2):
+                                      (11, 640, 128, 16), (12, 16384, 6272, 16416), (12, 8192, 128, 48), (16, 1152, 384, 130),
+                                      (8, 4096, 12288, 6144), (3, 1024, 1536, 2064), (16, 4096, 4096, 4112), (2, 512, 9216, 528)])
+@pytest.mark.parametrize("runs", [2, 0])
+def test_norm_folded_into_the_products_around_it(M, H, K, N2, runs):
     """Up to 16 rows: the product before a norm adds its result to the stream and leaves
     bf16(h * weight) and the pieces of the rows' sums of squares; the product after it applies
     the rows' factors to its sums.  Each piece is checked against the plain formulas, and the
     chain against norm-then-product; the first norm of a model has no product before it."""
+    if not runs and K % 512 and H % 512:
+        pytest.skip("neither product would read w in runs")
+    ops.gemm_runs(runs)
+    try:
+        norm_folded_case(M, H, K, N2)
+    finally:
+        ops.gemm_runs(True)
+
+
+def norm_folded_case(M, H, K, N2):
     eps = 3e-6
     h = rnd(M, H, seed=70, scale=2.0)
     x = rnd(M, K, dtype=torch.bfloat16, seed=71)
@@ -649,6 +661,20 @@ def test_gemm_bf16_few_rows_cut_evenly(M, N, K, even):
         few_rows_case(M, N, K)
     finally:
         ops.gemm_even_rows(True)
+
+
+@pytest.mark.parametrize("runs", [2, 1, 0])
+@pytest.mark.parametrize("M,N,K", [(8, 6144, 4096), (1, 4096, 512), (16, 24576, 1024), (5, 4112, 12288), (13, 1000, 2560),
+                                   (8, 151936, 1024), (2, 300, 16384)])
+def test_gemm_bf16_few_rows_in_runs(M, N, K, runs):
+    """Up to 16 rows and K a multiple of 512: w is read in runs of 1 KB through LDS (one tile a
+    workgroup with x streamed beside w, or several with x kept in registers) at every size (2),
+    where w is large (1), or, switched off (0), as the matrix-core operand lies.  Every epilogue."""
+    ops.gemm_runs(runs)
+    try:
+        few_rows_case(M, N, K)
+    finally:
+        ops.gemm_runs(True)
 
 
 def few_rows_case(M, N, K):
