@@ -158,11 +158,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
         return rsqrtf(ss / (float)K + fuse.scale_eps);
     };
     float factor = 1.f;
-    if (SCALE && XR > 0) {   // a workgroup of many tiles waits for them once, and needs the registers
-        leave_pieces();
-        __syncthreads();
-        factor = row_factor();
-    }
     const bf16* xp[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) xp[mt] = x + (size_t)min(mt * 16 + r, M - 1) * K + g * 8;
@@ -317,6 +312,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
         int tile = blockIdx.x;
         if (tile < tiles)
             load_w_blocks<XR, WAVES>(a_now, w + (size_t)min(tile * rows + r, min(N, (tile + 1) * rows) - 1) * K + g * 8, wave, kblocks);
+        if (SCALE) {   // a workgroup of many tiles waits for the pieces once, while x and the first tile's rows of w are on their way
+            leave_pieces();
+            __syncthreads();
+            factor = row_factor();
+        }
         while (tile < tiles) {
             one_tile(tile, a_now, a_next);
             tile += gridDim.x;
@@ -325,6 +325,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
             tile += gridDim.x;
         }
     } else {
+        if (SCALE && XR > 0) {
+            leave_pieces();
+            __syncthreads();
+            factor = row_factor();
+        }
         for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x) one_tile(tile, a_now, a_now);
     }
 }
@@ -1093,7 +1098,8 @@ static SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
     p.runs = false;
     // (measured at 8 rows: 201 MB of w 41.8 -> 38.7 us, 100 MB 24.8 -> 22.3, 1.2 GB 221 -> 213; 50 MB 12.4 -> 13.5 and
     // 34 MB 9.8 -> 10.1: the ring's start and the barrier of every stage cost the small ones more than the runs gain)
-    if (g_runs && g_force_skinny < 0 && K % SR_K == 0 && (g_runs > 1 || (long long)N * K >= (1ll << 25))) {
+    // With one or two rows of x the kernel above, one tile a workgroup, is the faster one (1.2 GB of w: 196 against 206 us).
+    if (g_runs && g_force_skinny < 0 && K % SR_K == 0 && (g_runs > 1 || (M >= 4 && (long long)N * K >= (1ll << 25)))) {
         // tiles of 16 rows, or of as many as give every CU the same number (the SwiGLU epilogue keeps whole blocks of 16)
         p.runs = true;
         p.shape = SKINNY_PLAIN;
