@@ -362,6 +362,13 @@ __device__ __forceinline__ void join_shares(const float* __restrict__ part_o,
     __shared__ float f[64];
     __shared__ float inv_l;
     const int tid = threadIdx.x;
+    // up to eight shares: their sums are asked for before the factors are, one trip to memory instead of two
+    float early[8];
+    const bool ahead = splits <= 8 && tid < D;
+    if (ahead) {
+#pragma unroll
+        for (int s = 0; s < 8; ++s) early[s] = s < splits ? part_o[(base + s) * D + tid] : 0.f;
+    }
     if (tid < 64) {
         const float ms = tid < splits ? part_ml[(base + tid) * 2] : -INFINITY;
         const float ls = tid < splits ? part_ml[(base + tid) * 2 + 1] : 0.f;
@@ -372,6 +379,14 @@ __device__ __forceinline__ void join_shares(const float* __restrict__ part_o,
         if (tid == 0) inv_l = 1.f / l;
     }
     __syncthreads();
+    if (ahead) {
+        float o = 0.f;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) o += f[s] * early[s];     // f is 0 beyond the shares
+        out_row[tid] = static_cast<bf16>(o * inv_l);
+        return;
+    }
+    if (splits <= 8) return;
     for (int dim = tid; dim < D; dim += 128) {
         float o = 0.f;
 #pragma unroll 8
