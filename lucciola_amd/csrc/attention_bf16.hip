@@ -351,23 +351,18 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
     }
 }
 
-// Joins the shares of a row's keys: out = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m), the
-// shares of (row, head) lying at part_o[base + s][D] and part_ml[base + s][2].  The factors are
-// worked out once (one thread per share) and left in LDS, so that the sum over the shares is a
-// run of independent loads.  128 threads; at most 64 shares.
-template <int D>
-__device__ __forceinline__ void join_shares(const float* __restrict__ part_o,
-                                            const float* __restrict__ part_ml, size_t base,
-                                            int splits, bf16* __restrict__ out_row) {
+template <int D, int MOST>
+__device__ __forceinline__ void join_shares_of(const float* __restrict__ part_o,
+                                               const float* __restrict__ part_ml, size_t base,
+                                               int splits, bf16* __restrict__ out_row) {
     __shared__ float f[64];
     __shared__ float inv_l;
     const int tid = threadIdx.x;
-    // up to eight shares: their sums are asked for before the factors are, one trip to memory instead of two
-    float early[8];
-    const bool ahead = splits <= 8 && tid < D;
-    if (ahead) {
+    // the shares' sums are asked for before their factors are: one trip to memory instead of two
+    float early[MOST];
+    if (tid < D) {
 #pragma unroll
-        for (int s = 0; s < 8; ++s) early[s] = s < splits ? part_o[(base + s) * D + tid] : 0.f;
+        for (int s = 0; s < MOST; ++s) early[s] = s < splits ? part_o[(base + s) * D + tid] : 0.f;
     }
     if (tid < 64) {
         const float ms = tid < splits ? part_ml[(base + tid) * 2] : -INFINITY;
@@ -379,20 +374,24 @@ __device__ __forceinline__ void join_shares(const float* __restrict__ part_o,
         if (tid == 0) inv_l = 1.f / l;
     }
     __syncthreads();
-    if (ahead) {
+    if (tid < D) {
         float o = 0.f;
 #pragma unroll
-        for (int s = 0; s < 8; ++s) o += f[s] * early[s];     // f is 0 beyond the shares
+        for (int s = 0; s < MOST; ++s) o += f[s] * early[s];     // f is 0 beyond the shares
         out_row[tid] = static_cast<bf16>(o * inv_l);
-        return;
     }
-    if (splits <= 8) return;
-    for (int dim = tid; dim < D; dim += 128) {
-        float o = 0.f;
-#pragma unroll 8
-        for (int s = 0; s < splits; ++s) o += f[s] * part_o[(base + s) * D + dim];
-        out_row[dim] = static_cast<bf16>(o * inv_l);
-    }
+}
+
+// Joins the shares of a row's keys: out = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m), the
+// shares of (row, head) lying at part_o[base + s][D] and part_ml[base + s][2].  The factors are
+// worked out once (one thread per share) and left in LDS.  128 threads (D <= 128); at most 64 shares.
+template <int D>
+__device__ __forceinline__ void join_shares(const float* __restrict__ part_o,
+                                            const float* __restrict__ part_ml, size_t base,
+                                            int splits, bf16* __restrict__ out_row) {
+    if (splits <= 8) join_shares_of<D, 8>(part_o, part_ml, base, splits, out_row);
+    else if (splits <= 32) join_shares_of<D, 32>(part_o, part_ml, base, splits, out_row);
+    else join_shares_of<D, 64>(part_o, part_ml, base, splits, out_row);
 }
 
 template <int D>

@@ -376,8 +376,8 @@ template <int MAXN> __device__ __forceinline__ void wait_vmcnt_upto(int n) {
 }
 // a barrier for LDS written by ordinary stores (it does not wait for global loads in flight)
 __device__ __forceinline__ void raw_barrier() {
-    wait_lgkmcnt<0>();
-    asm volatile("s_barrier" : : : "memory");
+    // one statement: the compiler keeps ordinary stores before it, and the wait cannot part from the barrier
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory");
 }
 
 // XS > 0 (K <= XS * 512): a wave keeps its columns of x in registers for all of its workgroup's
