@@ -152,11 +152,13 @@ __device__ __forceinline__ void attend_range(AttnState<D, QT>& st, const bf16x8 
                                              const bf16* __restrict__ v_cache,
                                              const int* __restrict__ table, int begin, int end,
                                              int step, int nkv, int kvh, const int (&lo)[QT],
-                                             const int (&hi)[QT], float scale_log2, int lane) {
+                                             const int (&hi)[QT], float scale_log2, int lane,
+                                             const int (&first_pages)[2]) {
+    // first_pages: table[begin] and table[begin + step], where they exist
     if (begin >= end) return;
     PageRegs<D> cur, nxt;
-    load_page<D>(cur, k_cache, v_cache, table[begin], nkv, kvh, lane);
-    int next_page = (begin + step < end) ? table[begin + step] : 0;
+    load_page<D>(cur, k_cache, v_cache, first_pages[0], nkv, kvh, lane);
+    int next_page = first_pages[1];
     for (int pg = begin; pg < end; pg += step) {
         const bool more = pg + step < end;
         if (more) {
@@ -219,6 +221,9 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
     const int begin = first_page + split * per;
     const int end = min(begin + per, last_page + 1);
     const int* table = block_table + (size_t)req * max_blocks;
+    // the numbers of the wave's first two pages: asked for now, they are back before the q/k preparation below is done
+    const int pg0 = begin + wave;
+    const int first_pages[2] = {pg0 < end ? table[pg0] : 0, pg0 + NW < end ? table[pg0 + NW] : 0};
 
     bf16x8 bq[1][D / 32];
     if (pro.enabled) {
@@ -314,7 +319,7 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
     init_state<D, 1>(st);
     const int lo[1] = {j_lo}, hi[1] = {p};
     attend_range<D, 1>(st, bq, k_cache, v_cache, table, begin + wave, end, NW, nkv, kvh, lo, hi,
-                       scale_log2, lane);
+                       scale_log2, lane, first_pages);
 
     // the waves' results meet in LDS
     float l = st.l[0];
