@@ -47,9 +47,10 @@ class RequestState:
 
 class CacheManager:
     def __init__(self, site_specs: Sequence[Optional[object]], block_size: int, num_blocks: int,
-                 max_seqs: int):
+                 max_seqs: int, scatter_pages: bool = True):
         """``site_specs[i]``: what site i of the run order needs (PagedKV, FixedState or None).
-        A site that reads another site's cache is passed as None here."""
+        A site that reads another site's cache is passed as None here.  ``scatter_pages``: see
+        :class:`PagePool`."""
         if block_size <= 0 or num_blocks <= 0:
             raise ValueError("block_size and num_blocks must be positive")
         self.block_size = block_size
@@ -69,7 +70,7 @@ class CacheManager:
                         self.site_group[i] = gi
                         break
                 else:
-                    self.groups.append(PageGroup(spec, [i], PagePool(num_blocks)))
+                    self.groups.append(PageGroup(spec, [i], PagePool(num_blocks, scatter_pages)))
                     self.site_group[i] = len(self.groups) - 1
             elif isinstance(spec, FixedState):
                 self.state_sites.append(i)

@@ -14,7 +14,7 @@ WINDOW = PagedKV(2, 16, window=10)
 
 def test_pool_is_first_in_first_out():
     # src/block_manager.cc:26-40: allocate pops the front, free pushes to the back
-    pool = PagePool(4)
+    pool = PagePool(4, scatter=False)
     assert [pool.allocate() for _ in range(4)] == [0, 1, 2, 3]
     with pytest.raises(OutOfPages):
         pool.allocate()
@@ -26,6 +26,21 @@ def test_pool_is_first_in_first_out():
     pool.free(1)
     with pytest.raises(ValueError, match="freed twice"):
         pool.free(1)
+    pool.check()
+
+
+def test_pool_scatters_its_first_round():
+    """By default the first round of pages comes in a fixed shuffled order (a function of the
+    pool's size), every page once; after that the pool is first in, first out as above."""
+    first = [PagePool(64).allocate() for _ in range(1)]
+    pool = PagePool(64)
+    order = [pool.allocate() for _ in range(64)]
+    assert sorted(order) == list(range(64)) and order != list(range(64)) and order[:1] == first
+    again = PagePool(64)
+    assert [again.allocate() for _ in range(64)] == order
+    for page in (order[5], order[2], order[40]):
+        pool.free(page)
+    assert [pool.allocate() for _ in range(3)] == [order[5], order[2], order[40]]
     pool.check()
 
 
@@ -50,7 +65,7 @@ def test_groups_are_formed_by_equal_needs():
 
 
 def test_pages_follow_the_length():
-    cm = CacheManager([FULL], 4, 10, 2)
+    cm = CacheManager([FULL], 4, 10, 2, scatter_pages=False)
     cm.admit("a")
     cm.reserve("a", 5)
     assert cm.block_table(0, "a") == [0, 1] and cm.length("a") == 0
