@@ -382,7 +382,12 @@ __device__ __forceinline__ void raw_barrier() {
 
 // XS > 0 (K <= XS * 512): a wave keeps its columns of x in registers for all of its workgroup's
 // tiles.  XS = 0 (any K): a wave's 16 bytes of x for a stage travel with the stage's run of w,
-// seven stages ahead, into a ring of registers.
+// seven stages ahead, into a ring of registers.  Those loads are inline assembly (the compiler
+// would wait for them, and with them for every load of the ring issued before them, at their
+// first use); a register of the ring is written by the hardware long after the statement that
+// names it, which is safe only because every such register is read again after the counted wait
+// and before anything else may be put into it: a load whose value nobody reads would leave its
+// registers to the compiler's next use while the value is still on its way.
 template <int EPI, bool SCALE, int XS, typename TO>
 __global__ __launch_bounds__(1024) void gemm_runs_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                                                          TO* __restrict__ out, int M, int N, int K, int rows,
