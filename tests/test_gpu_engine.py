@@ -464,6 +464,29 @@ def test_layers_of_the_8b_size(dtype):
         del runner
 
 
+def test_8b_size_requests_that_decode_side_by_side():
+    """Six requests at the 8B-shaped sizes whose last tokens are decoded together, six rows a
+    step, and twelve: the products of four to sixteen rows, which read large weights in runs
+    through LDS, chained through the folded norms as the engine chains them, and the decode
+    attention over six and twelve requests at once; against the plain implementation."""
+    weights, prompts, refs = case_8b()
+    for copies in (3, 6):
+        many = {f"{name}{c}": ids for c in range(copies) for name, ids in prompts.items()}
+        many_refs = {f"{name}{c}": refs[name] for c in range(copies) for name in prompts}
+        tail = 5
+        steps = [([(name, list(ids[:-tail]), [len(ids) - tail - 1]) for name, ids in many.items()], [])]
+        for i in range(tail, 0, -1):
+            steps.append(([(name, [ids[-i]], [0]) for name, ids in many.items()],
+                          list(many) if i == 1 else []))
+        runner = make_runner(_8B, weights, 16, traces.max_live_tokens(steps, 16) // 16, "bfloat16", DEV,
+                             max_seqs=2 * copies)
+        got = replay(runner, steps)
+        assert len(got) == 2 * copies * (tail + 1)
+        worst = compare(got, _8B, weights, many, TOL["bfloat16"], many_refs)
+        print(f"8B-size layers, {2 * copies} requests side by side: worst relative error {worst:.3e}")
+        del runner
+
+
 def test_float32_logits_do_not_depend_on_the_cut():
     """In float32 the logits at a position are the same bits however the tokens are cut into
     steps, whatever else is in the batch, whichever pages are used and whatever the page size
