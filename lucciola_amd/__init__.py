@@ -10,7 +10,9 @@ include/scheduler.h, include/sequence.h):
 
 and, stepped by the caller: ``LLMEngine`` (``add_request`` / ``step`` / ``generate``),
 ``Scheduler`` (``add_request`` / ``step`` / ``has_unfinished_requests`` / ``free_sequence``),
-``Sequence``, ``SamplingParams``, ``EngineConfig``.  Requests carry token ids.
+``Sequence``, ``SamplingParams``, ``EngineConfig``.  Requests carry token ids; where the model
+folder holds a ``vocab.json``, ``generate_async`` also takes a string as the reference does
+(``VocabTokenizer``, ``ChatFormat``) and calls back with text.
 """
 __version__ = "0.1.0"
 
@@ -27,6 +29,8 @@ _LAZY = {
     "Qwen3Config": ("lucciola_amd.config.model_config", "Qwen3Config"),
     "load_model": ("lucciola_amd.engine.loading", "load_model"),
     "random_model": ("lucciola_amd.engine.loading", "random_model"),
+    "VocabTokenizer": ("lucciola_amd.text.vocab_tokenizer", "VocabTokenizer"),
+    "ChatFormat": ("lucciola_amd.text.vocab_tokenizer", "ChatFormat"),
     "write_model_folder": ("lucciola_amd.weights.random_init", "write_model_folder"),
 }
 

@@ -3,13 +3,18 @@
 of ``block_size`` tokens, read a request per input line until ``exit``, run the scheduler loop
 and stream what is generated, at most 100 tokens a request).
 
-Requests are token ids here (there is no tokenizer): a line of ids separated by blanks or
-commas.  Options carry the reference's names where it has them: ``--max-blocks`` and
-``--block-size`` are the arguments of ``AsyncEngine(model_path, max_blocks, block_size)``
-(include/async_engine.h:24-25), ``--max-new-tokens`` that of ``generate_async``.
+Requests are token ids: a line of ids separated by blanks or commas.  Where the model folder
+holds a ``vocab.json``, ``--prompt`` and ``--text`` take text as the reference does: encoded by
+longest match against the vocabulary (src/tokenizer.cc:87-132) inside the reference's chat
+format (examples/qwen_dynamic.cc:48-66), and what is generated is printed as text.  Options
+carry the reference's names where it has them: ``--max-blocks`` and ``--block-size`` are the
+arguments of ``AsyncEngine(model_path, max_blocks, block_size)`` (include/async_engine.h:24-25),
+``--max-new-tokens`` that of ``generate_async``.
 
     python -m lucciola_amd --model DIR                       # ids from standard input
     python -m lucciola_amd --model DIR --prompt-ids 1,2,3 --prompt-ids 4,5
+    python -m lucciola_amd --model DIR --text                # a line of text per request
+    python -m lucciola_amd --model DIR --prompt "Why is the sky blue?"
     python -m lucciola_amd --random-config config.json --seed 0 --write-model DIR
 """
 from __future__ import annotations
@@ -46,6 +51,15 @@ def main(argv=None) -> int:
     ap.add_argument("--ignore-eos", action="store_true")
     ap.add_argument("--prompt-ids", action="append", default=[],
                     help="a request as comma-separated token ids (may be given several times)")
+    ap.add_argument("--prompt", action="append", default=[],
+                    help="a request as text (needs vocab.json in the model folder; may be given several times)")
+    ap.add_argument("--text", action="store_true",
+                    help="lines of standard input are text, not token ids (needs vocab.json)")
+    ap.add_argument("--no-chat-format", action="store_true",
+                    help="encode text as it is, without the reference's chat format around it")
+    ap.add_argument("--chat-ids", default="",
+                    help="three token ids for the chat format: start, end, line break "
+                         "(default: the reference's 151644,151645,1699)")
     ap.add_argument("--prompt-ids-file", help="a file with one request of token ids per line")
     ap.add_argument("--random-prompts", help="comma-separated lengths: one request of random ids for each")
     ap.add_argument("--random-config", help="a config.json to make random weights for")
@@ -84,7 +98,25 @@ def main(argv=None) -> int:
         return SamplingParams(max_new_tokens=args.max_new_tokens, temperature=args.temperature,
                               seed=args.seed + i, ignore_eos=args.ignore_eos)
 
+    tokenizer = None
+    if args.prompt or args.text:
+        from .text.vocab_tokenizer import ChatFormat, find_vocab
+        tokenizer = find_vocab(args.model)
+        if tokenizer is None:
+            ap.error(f"--prompt and --text need a vocab.json in {args.model}")
+        chat = None
+        if not args.no_chat_format:
+            marks = _ids(args.chat_ids)
+            if len(marks) not in (0, 3):
+                ap.error("--chat-ids takes three ids: start, end, line break")
+            chat = ChatFormat(*marks)
+
+    def from_text(text: str) -> List[int]:
+        return chat.prompt(tokenizer, text) if chat else tokenizer.encode(text)
+
     prompts = [_ids(p) for p in args.prompt_ids]
+    as_text = [False] * len(prompts) + [True] * len(args.prompt)
+    prompts += [from_text(p) for p in args.prompt]
     if args.prompt_ids_file:
         with open(args.prompt_ids_file, "r", encoding="utf-8") as fh:
             prompts += [_ids(line) for line in fh if line.strip()]
@@ -94,9 +126,10 @@ def main(argv=None) -> int:
         prompts += [[rng.randrange(engine.model.vocab_size) for _ in range(n)]
                     for n in _ids(args.random_prompts)]
     if prompts:
+        as_text += [False] * (len(prompts) - len(as_text))
         outputs = engine.generate(prompts, [params(i) for i in range(len(prompts))])
-        for out in outputs:
-            print(" ".join(str(t) for t in out), flush=True)
+        for out, text in zip(outputs, as_text):
+            print(tokenizer.decode(out) if text else " ".join(str(t) for t in out), flush=True)
         return 0
 
     # interactive: a request per line, generated ids streamed as they come
@@ -108,6 +141,13 @@ def main(argv=None) -> int:
         if not line:
             continue
         try:
+            if args.text:
+                stream = tokenizer.stream()
+                engine.generate([from_text(line)], [params(count)],
+                                on_token=lambda _id, tok, done: print(
+                                    stream.feed(tok, done), end="\n" if done else "", flush=True))
+                count += 1
+                continue
             prompt = _ids(line)
             engine.generate([prompt], [params(count)],
                             on_token=lambda _id, tok, done: print(tok, end="\n" if done else " ", flush=True))

@@ -395,7 +395,27 @@ def test_command_line_and_async_engine(tmp_path):
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert [int(t) for t in proc.stdout.split()] == want[0]
 
+    # text: a vocab.json beside the weights (every byte a token), the chat format with ids of this vocabulary
+    import json
+    from lucciola_amd.text.vocab_tokenizer import ChatFormat, VocabTokenizer, byte_alphabet
+    vocab = {c: b for b, c in enumerate(byte_alphabet())}
+    with open(os.path.join(folder, "vocab.json"), "w", encoding="utf-8") as fh:
+        json.dump(vocab, fh)
+    tok, fmt = VocabTokenizer(vocab), ChatFormat(380, 381, 382)
+    text_prompt = fmt.prompt(tok, "hi there")
+    text_want = tok.decode(plain_qwen3.greedy(cfg, weights, text_prompt, 6))
+    text_cmd = cmd[:cmd.index("--prompt-ids")] + ["--chat-ids", "380,381,382"]
+    utf8 = dict(os.environ, PYTHONUTF8="1")          # bytes, not text: random tokens hold line ends of every kind
+    proc = subprocess.run(text_cmd + ["--prompt", "hi there"], cwd=ROOT, capture_output=True, timeout=600, env=utf8)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout == (text_want + "\n").encode("utf-8")
+    proc = subprocess.run(text_cmd + ["--text"], cwd=ROOT, capture_output=True, timeout=600, env=utf8,
+                          input=b"hi there\nexit\n")
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout == (text_want + "\n").encode("utf-8")
+
     engine = AsyncEngine(folder, max_blocks=32, block_size=page, dtype="float32")
+    assert engine.tokenizer is not None and len(engine.tokenizer) == 256
     got = {0: [], 1: []}
     done = [threading.Event(), threading.Event()]
 
