@@ -45,6 +45,9 @@ class RequestState:
     started: bool = False     # False until the first commit: state slots are zeroed then
 
 
+KERNEL_PAGE = 16       # tokens of a page as the kernels see it, where the page size is a multiple of it
+
+
 class CacheManager:
     def __init__(self, site_specs: Sequence[Optional[object]], block_size: int, num_blocks: int,
                  max_seqs: int, scatter_pages: bool = True):
@@ -54,6 +57,14 @@ class CacheManager:
         if block_size <= 0 or num_blocks <= 0:
             raise ValueError("block_size and num_blocks must be positive")
         self.block_size = block_size
+        # What the kernels see: a page of 32, 48, 64, ... tokens lies in memory as that many
+        # pages of 16 in a row, each in the layout of a page of 16, and the block tables that
+        # go to the device name those (page p becomes p * pieces ... p * pieces + pieces - 1).
+        # A slot id, page * block_size + offset, is the same number either way.  So the
+        # matrix-core kernels, which are built for pages of 16, serve every such size.
+        self.kernel_block = KERNEL_PAGE if block_size > KERNEL_PAGE and block_size % KERNEL_PAGE == 0 \
+            else block_size
+        self.pieces = block_size // self.kernel_block
         self.num_blocks = num_blocks
         self.max_seqs = max_seqs
         self.site_specs = list(site_specs)
@@ -102,12 +113,13 @@ class CacheManager:
         return total
 
     def allocate_tensors(self, dtype: torch.dtype, device) -> None:
-        """Per paged site: keys [num_blocks, kv_heads, block_size, head_dim] and values
-        [num_blocks, kv_heads, head_dim, block_size] (transposed inside a page);
-        state per state site: [max_seqs, *shape]."""
+        """Per paged site: keys [num_blocks * pieces, kv_heads, kernel_block, head_dim] and
+        values [num_blocks * pieces, kv_heads, head_dim, kernel_block] (transposed inside a
+        page); state per state site: [max_seqs, *shape]."""
         for g in self.groups:
-            k_shape = (self.num_blocks, g.spec.num_kv_heads, self.block_size, g.spec.head_dim)
-            v_shape = (self.num_blocks, g.spec.num_kv_heads, g.spec.head_dim, self.block_size)
+            pages = self.num_blocks * self.pieces
+            k_shape = (pages, g.spec.num_kv_heads, self.kernel_block, g.spec.head_dim)
+            v_shape = (pages, g.spec.num_kv_heads, g.spec.head_dim, self.kernel_block)
             for site in g.sites:
                 self.kv[site] = (torch.zeros(k_shape, dtype=dtype, device=device),
                                  torch.zeros(v_shape, dtype=dtype, device=device))

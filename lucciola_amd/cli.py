@@ -37,7 +37,7 @@ def main(argv=None) -> int:
     ap.add_argument("--max-blocks", "--num-pages", dest="max_blocks", type=int, default=0,
                     help="pages of the cache; 0 sizes it from free memory (the reference's default)")
     ap.add_argument("--block-size", "--page-size", dest="block_size", type=int, default=16,
-                    help="tokens in a page")
+                    help="tokens in a page (multiples of 16 are served by the matrix-core attention kernels)")
     ap.add_argument("--mem-fraction", type=float, default=0.90,
                     help="with --max-blocks 0: share of the free memory the cache may take "
                          "(the reference's 0.90, src/async_engine.cc:13)")

@@ -66,8 +66,8 @@ class SiteView:
     batch: "StepBatch"
     index: int
     writes_cache: bool
-    page_size: int
-    kv: Optional[Tuple[torch.Tensor, torch.Tensor]] = None   # keys, values [pages, kvh, page, d]
+    page_size: int              # tokens of a page of kv and of a block-table entry, as the kernels see them
+    kv: Optional[Tuple[torch.Tensor, torch.Tensor]] = None   # keys [pages, kvh, page, d], values [pages, kvh, d, page]
     attn: Optional[AttentionBatch] = None                    # of this site's page group
     state: Optional[torch.Tensor] = None                     # [max_seqs, *shape]
 
@@ -232,6 +232,12 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
                 flat[r, :len(t)] = np.frombuffer(t, dtype=np.int32)
         pages = flat[tok_req, positions // bs] if T else np.zeros(0, np.int32)
         slots = np.where(pages >= 0, pages * bs + positions % bs, -1).astype(np.int32)
+        if cache.pieces > 1:        # the kernels' pages: every page as its pieces in a row
+            pieces = cache.pieces
+            flat = np.where(flat[:, :, None] >= 0,
+                            flat[:, :, None] * pieces + np.arange(pieces, dtype=np.int32), -1)
+            flat = flat.reshape(R, mb * pieces).astype(np.int32)
+            mb *= pieces
         group_handles.append((pk.add(flat), mb, pk.add(slots)))
 
     buffer = pk.upload(device, into)

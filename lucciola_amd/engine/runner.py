@@ -238,7 +238,7 @@ class ModelRunner:
         for index, entry in enumerate(self.model.spec.run_order):
             owner = index if entry.cache_of is None else entry.cache_of
             view = SiteView(batch=batch, index=index, writes_cache=entry.cache_of is None,
-                            page_size=cache.block_size)
+                            page_size=cache.kernel_block)
             if owner in cache.kv:
                 view.kv = cache.kv[owner]
                 view.attn = batch.groups[cache.site_group[owner]]

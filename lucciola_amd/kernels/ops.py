@@ -612,7 +612,7 @@ def attention(qkv, batch: AttentionBatch, k_cache: torch.Tensor,
     if qkv.dtype == torch.bfloat16 and not fast:
         _say_once(("attention", nh, nkv, d, page_size),
                   f"bfloat16 attention with {nh} heads, {nkv} kv heads of {d} and pages of {page_size} tokens has no "
-                  "matrix-core kernel (heads of 32, 64, 96 or 128, pages of 16, at most 16 heads a kv head): "
+                  "matrix-core kernel (heads of 32, 64, 96 or 128, pages of a multiple of 16 tokens, at most 16 heads a kv head): "
                   "the general kernel runs, correct and many times slower")
     # who prepares q, k, v (norm, rotation, cache write) when they arrive raw: a step of single
     # tokens does it all inside the decode kernel; otherwise a kernel of its own does k and v,

@@ -43,6 +43,25 @@ def test_step_function_matches_plain(monkeypatch, key, family):
         assert g.pool.num_free() == blocks
 
 
+@pytest.mark.parametrize("key,page", [("C", 32), ("A", 48), ("D", 64)])
+@pytest.mark.parametrize("family", ["chunked", "mixed"])
+def test_pages_of_several_kernel_pages(monkeypatch, key, page, family):
+    """A page of 32, 48 or 64 tokens goes to the kernels as two, three or four pages of 16 in a
+    row: the cache counts in its own pages, the block tables on the device name the pieces."""
+    reference_ops.install(monkeypatch)
+    cfg, _, seed = configs.ALL[key]
+    prompts = prompts_for(cfg, [70, 33, 50, 3, 131], seed)
+    steps = {"chunked": traces.chunked, "mixed": traces.mixed}[family](prompts)
+    blocks = traces.max_live_tokens(steps, page) // page
+    runner, weights = make(cfg, seed, page, blocks)
+    assert runner.cache.kernel_block == 16 and runner.cache.pieces == page // 16
+    assert runner.cache.kv[0][0].shape[0] == blocks * (page // 16) and runner.cache.kv[0][0].shape[2] == 16
+    got = replay(runner, steps)
+    compare(got, cfg, weights, prompts, 2e-5)
+    for g in runner.cache.groups:
+        assert g.pool.num_free() == blocks
+
+
 def host_engine(cfg, weights, page, blocks, **kw):
     from lucciola_amd.engine.llm_engine import LLMEngine
     from lucciola_amd.engine.loading import _build

@@ -61,6 +61,28 @@ def test_replay_families(dtype, key, family):
         assert g.pool.num_free() == blocks
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key,page", [("C", 32), ("A", 48), ("D", 64), ("D", 32)])
+def test_pages_of_several_kernel_pages(dtype, key, page):
+    """Pages of 32, 48 and 64 tokens, which the kernels see as runs of pages of 16: mixed with
+    so few pages that they are used again, and with a decoded tail.  (D's heads of 64 go
+    through the matrix-core kernels in bfloat16.)"""
+    cfg, _, seed = configs.ALL[key]
+    weights = random_weights(cfg, seed)
+    prompts = prompts_for(cfg, [70, 33, 150, 3, 131], seed + 5)
+    refs = {n: plain_qwen3.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    for family in (traces.mixed, traces.tail_decode):
+        steps = family(prompts)
+        blocks = traces.max_live_tokens(steps, page) // page
+        runner = make_runner(cfg, weights, page, blocks, dtype, DEV)
+        assert runner.cache.pieces == page // 16
+        got = replay(runner, steps)
+        assert len(got) == sum(len(p) for p in prompts.values())
+        compare(got, cfg, weights, prompts, TOL[dtype], refs)
+        for g in runner.cache.groups:
+            assert g.pool.num_free() == blocks
+
+
 def random_configuration(seed):
     """A configuration drawn at random from what config.json allows: any number of heads and
     groups, head sizes in steps of 16, widths, feed-forward sizes and vocabularies that are odd
@@ -560,7 +582,7 @@ def test_cache_sized_from_free_memory():
         cap = 4 * (cfg["max_position_embeddings"] // page)
         assert engine.runner.cache.num_blocks == min(by_memory, cap)
         assert (by_memory < cap) == (fraction < 0.1) and by_memory > 20
-        assert engine.runner.cache.kv[0][0].shape[0] == engine.runner.cache.num_blocks
+        assert engine.runner.cache.kv[0][0].shape[0] == engine.runner.cache.num_blocks * engine.runner.cache.pieces
         prompts = list(prompts_for(cfg, [5, 11, 17], seed + 30).values())
         got = engine.generate(prompts, SamplingParams(max_new_tokens=8))
         assert got == [plain_qwen3.greedy(cfg, weights, p, 8) for p in prompts]

@@ -113,7 +113,7 @@ def attention_site(part, T, page, dtype, first=0):
     cache.reserve("r", T)
     batch = build_batch([StepEntry("r", list(range(T)), [])], cache, DEV,
                         planners=dict([part.batch_planner()]))
-    return SiteView(batch=batch, index=0, writes_cache=True, page_size=page, kv=cache.kv[0],
+    return SiteView(batch=batch, index=0, writes_cache=True, page_size=cache.kernel_block, kv=cache.kv[0],
                     attn=batch.groups[0]), cache
 
 
