@@ -1235,6 +1235,9 @@ LC_API int lc_gemm_bf16_supported(int M, int N, int K) {
     return 1;
 }
 
+// What K must be a multiple of for the matrix-core kernels.
+LC_API int lc_gemm_bf16_kblock() { return SK_KBLOCK; }
+
 // Forces the shape of the skinny kernel for every later product of up to 16 rows (0: deep
 // unroll, 1: plain, 2: two row tiles of w a workgroup, 3: several tiles a workgroup with x kept
 // in registers, where K allows it; -1: choose by size again).  For tests and tuning.

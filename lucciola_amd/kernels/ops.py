@@ -29,6 +29,7 @@ _SIGNATURES = {
     "lc_gemm_generic": "pipipiiiipp",
     "lc_gemm_bf16": "pppiiiiipp",
     "lc_gemm_bf16_supported": "iii",
+    "lc_gemm_bf16_kblock": "",
     "lc_gemm_bf16_force_tile": "i",
     "lc_gemm_bf16_force_skinny": "i",
     "lc_gemm_bf16_even_rows": "i",
@@ -351,6 +352,10 @@ def gemm(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None, defer: boo
         _call("lc_gemm_bf16", _ptr(x), _ptr(w), _ptr(out), _c_int(_dt(out)), _c_int(M), _c_int(N),
               _c_int(K), 0, _ptr(_gemm_workspace(M, N, K, x.device)), _stream())
     else:
+        if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and N * K >= 1 << 22:
+            _say_once(("gemm", N, K),
+                      f"a bfloat16 product with w [{N}, {K}] has no matrix-core kernel (K must be a multiple "
+                      f"of {library().lc_gemm_bf16_kblock()}): the general kernel runs, correct and many times slower")
         words = library().lc_gemm_generic_workspace(M, N, K)
         workspace = torch.empty((words,), dtype=torch.float32, device=x.device) if words else None
         _call("lc_gemm_generic", _ptr(x), _c_int(_dt(x)), _ptr(w), _c_int(_dt(w)), _ptr(out),

@@ -438,6 +438,26 @@ def test_attention_bf16_long_contexts(nh, nkv, d, window):
     close(got, want, torch.bfloat16, atol=attention_atol(torch.bfloat16, vc))
 
 
+def test_slow_paths_say_so_once(capfd):
+    """A large bfloat16 product whose K the matrix-core kernels do not take, and bfloat16
+    attention with pages that are no multiple of 16, run through the general kernels, right,
+    and say so on stderr the first time."""
+    ops._said.clear()
+    x = torch.randn(5, 2056, device=DEV).bfloat16()
+    w = torch.randn(2048, 2056, device=DEV).bfloat16()
+    for _ in range(2):
+        got = ops.gemm(x, w)
+    close(got, ref.gemm(x.cpu(), w.cpu()), torch.bfloat16)
+    qkv, batch, kc, vc = paged_case([40], [40], 4, 2, 64, 8, torch.bfloat16, seed=3)
+    for _ in range(2):
+        ops.attention(qkv, batch, kc, vc, 4, 2, 64, 8, 64 ** -0.5, 0)
+    err = capfd.readouterr().err
+    assert err.count("product with w [2048, 2056] has no matrix-core kernel") == 1
+    assert err.count("pages of 8 tokens has no matrix-core kernel") == 1
+    ops.gemm(torch.randn(5, 2048, device=DEV).bfloat16(), torch.randn(2048, 2048, device=DEV).bfloat16())
+    assert "no matrix-core" not in capfd.readouterr().err
+
+
 @pytest.mark.parametrize("nh,nkv,window", [(8, 2, 0), (4, 2, 100), (6, 1, 33), (2, 1, 0)])
 def test_attention_prefill_of_heads_of_128_in_pairs(nh, nkv, window):
     """Heads of 128 with an even number of heads per kv head go to the prefill kernel built from
