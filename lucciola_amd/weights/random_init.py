@@ -112,9 +112,14 @@ def random_tensors(declared: Mapping[str, ParamDecl], seed: int, std: float,
 
 
 def write_model_folder(folder: str, config_dict: Dict[str, Any], seed: int,
-                       dtype: torch.dtype = torch.bfloat16, std: float = None) -> str:
+                       dtype: torch.dtype = torch.bfloat16, std: float = None,
+                       device: str = None) -> str:
     """Make ``folder`` a model folder: config.json and model.safetensors with random weights
-    for the architecture that ``config_dict`` names."""
+    for the architecture that ``config_dict`` names.  ``device``: where the values are worked
+    out (they are the same everywhere; a GPU makes a model of 8B size in seconds, a CPU in
+    minutes); None: the GPU if there is one."""
+    if device is None:
+        device = "cuda:0" if torch.cuda.is_available() else "cpu"
     from ..config.registry import architecture_for
     from ..models.causal_lm import declared_tensors
 
@@ -126,5 +131,6 @@ def write_model_folder(folder: str, config_dict: Dict[str, Any], seed: int,
     with open(os.path.join(folder, "config.json"), "w", encoding="utf-8") as fh:
         json.dump(config_dict, fh, indent=2)
     write_safetensors(os.path.join(folder, "model.safetensors"),
-                      random_tensors(declared, seed, spec.init_std if std is None else std, dtype))
+                      random_tensors(declared, seed, spec.init_std if std is None else std, dtype,
+                                     device=device))
     return folder

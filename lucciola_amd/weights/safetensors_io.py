@@ -133,6 +133,5 @@ def write_safetensors(path: str, tensors: Iterable[Tuple[str, torch.Tensor]]) ->
         fh.write(blob)
         for _, t in items:
             if t.numel():
-                fh.write(t.view(torch.uint8).numpy().tobytes() if t.dim() else
-                         t.reshape(1).view(torch.uint8).numpy().tobytes())
+                fh.write(memoryview(t.reshape(-1).view(torch.uint8).numpy()))
     os.replace(tmp, path)
