@@ -473,6 +473,67 @@ def test_command_line_and_async_engine(tmp_path):
     assert not engine.engine.runner.cache.requests
 
 
+@pytest.mark.parametrize("dtype,blocks", [("bfloat16", 12), ("float32", 9)])
+def test_async_engine_under_threads_aborts_and_preemption(dtype, blocks):
+    """Several threads submit requests to one AsyncEngine, end some of them early and wait for
+    others, with so few pages that running requests are preempted: every request's callback
+    sees exactly one end, nothing is left in the cache, no page is lost."""
+    import random
+    import threading
+    import time
+    from lucciola_amd.engine.async_engine import AsyncEngine
+    cfg, page, seed = configs.ALL["D"]
+    weights = random_weights(cfg, seed, std=0.3)
+    engine = engine_for(cfg, weights, page, blocks, dtype, max_tokens_per_step=32, max_seqs=8)
+    front = AsyncEngine("", engine=engine)
+    problems, ends = [], []
+
+    def worker(wid):
+        rng = random.Random(wid)
+        waiting = []
+        for k in range(12):
+            prompt = [rng.randrange(cfg["vocab_size"]) for _ in range(rng.randint(1, 60))]
+            done, state = threading.Event(), {"tokens": 0, "ends": 0}
+
+            def on_token(tok, finished, state=state, done=done):
+                state["tokens"] += 1
+                if finished:
+                    state["ends"] += 1
+                    done.set()
+            rid = front.generate_async(prompt, rng.randint(1, 40), on_token,
+                                       temperature=rng.choice([0.0, 0.9]), seed=k)
+            if rng.random() < 0.3:
+                time.sleep(rng.random() * 0.01)
+                front.abort(rid)
+            waiting.append((done, state))
+            if rng.random() < 0.6:
+                for d, st in waiting:
+                    if not d.wait(120):
+                        problems.append(("no end", wid, k))
+                ends.extend(st["ends"] for _, st in waiting)
+                waiting = []
+        for d, st in waiting:
+            if not d.wait(120):
+                problems.append(("no end", wid))
+            ends.append(st["ends"])
+
+    threads = [threading.Thread(target=worker, args=(w,)) for w in range(6)]
+    try:
+        for th in threads:
+            th.start()
+        for th in threads:
+            th.join()
+    finally:
+        front.stop()
+    assert not problems
+    assert len(ends) == 6 * 12 and all(e == 1 for e in ends)
+    assert engine.scheduler.num_preemptions > 0
+    engine.runner.cache.check()
+    assert not engine.runner.cache.requests
+    for g in engine.runner.cache.groups:
+        assert g.pool.num_free() == blocks
+
+
 _8B = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 4096,
        "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
        "intermediate_size": 12288, "vocab_size": 151936, "rope_theta": 1000000.0,
