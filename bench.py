@@ -98,7 +98,7 @@ def main() -> int:
     model, mcfg = random_model(cfg, seed=0, dtype=dtype, device=dev)
     runner = ModelRunner(model, EngineConfig(dtype=dtype, block_size=bs, max_blocks=blocks,
                                              max_seqs=max_batch + 2, device=dev))
-    for k, v in runner.cache.kv.values():
+    for ((k, v),) in runner.cache.storage.values():
         k.normal_(0, 0.5)
         v.normal_(0, 0.5)
     sampler = Sampler()

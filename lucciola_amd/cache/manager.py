@@ -1,7 +1,8 @@
 """The cache manager: pages of keys and values with a block table per request, and slots for
 per-request state of fixed size.
 
-Every site of a model's run order states what it needs (:mod:`lucciola_amd.cache.specs`).
+Every site of a model's run order states what it needs (:mod:`lucciola_amd.cache.specs`); a
+need counts its own bytes and makes its own memory, the manager keeps the books.
 Sites with equal paged needs form a *group*: one pool of page ids and one block table per
 request serve the whole group, and each site of the group has key and value tensors of its
 own that are indexed by those page ids.  Groups differ in what they keep: all keys, or a
@@ -10,18 +11,18 @@ window of them, in which case the pages the window has passed are given back aft
 The reference has one group (every layer alike, src/qwen.cc:507-516), takes a page when
 ``ceil(len / block_size)`` exceeds the table (src/scheduler.cc:55-58,89-97) and gives all of
 a request's pages back when it ends (src/scheduler.cc:20-31).  The bookkeeping here is host
-code only; the tensors are made by :meth:`CacheManager.allocate_tensors`.
+code only; the device memory is made by the needs in :meth:`CacheManager.allocate_tensors`.
 """
 from __future__ import annotations
 
 from array import array
 from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+from typing import Any, Dict, Hashable, List, Optional, Sequence, Tuple
 
 import torch
 
 from .page_pool import OutOfPages, PagePool, SlotPool
-from .specs import FixedState, PagedKV
+from .specs import CacheLayout, CacheNeed
 
 
 def _ceil_div(a: int, b: int) -> int:
@@ -30,9 +31,11 @@ def _ceil_div(a: int, b: int) -> int:
 
 @dataclass
 class PageGroup:
-    spec: PagedKV
+    spec: CacheNeed
     sites: List[int]
     pool: PagePool
+    kernel_page: int          # tokens of a page as the group's kernels index it
+    pieces: int               # kernel pages in one of the manager's pages
     # a request's page ids in order, as a typed array (numpy views it without a copy); -1: given back
     tables: Dict[Hashable, array] = field(default_factory=dict)
 
@@ -45,88 +48,84 @@ class RequestState:
     started: bool = False     # False until the first commit: state slots are zeroed then
 
 
-KERNEL_PAGE = 16       # tokens of a page as the kernels see it, where the page size is a multiple of it
-
-
 class CacheManager:
     def __init__(self, site_specs: Sequence[Optional[object]], block_size: int, num_blocks: int,
                  max_seqs: int, scatter_pages: bool = True):
-        """``site_specs[i]``: what site i of the run order needs (PagedKV, FixedState or None).
-        A site that reads another site's cache is passed as None here.  ``scatter_pages``: see
-        :class:`PagePool`."""
+        """``site_specs[i]``: what site i of the run order needs: a :class:`CacheNeed`, a
+        tuple of them (a layer with several caching parts, in the order of its slots) or
+        None.  A site that reads another site's cache is passed as None here.
+        ``scatter_pages``: see :class:`PagePool`."""
         if block_size <= 0 or num_blocks <= 0:
             raise ValueError("block_size and num_blocks must be positive")
         self.block_size = block_size
-        # What the kernels see: a page of 32, 48, 64, ... tokens lies in memory as that many
-        # pages of 16 in a row, each in the layout of a page of 16, and the block tables that
-        # go to the device name those (page p becomes p * pieces ... p * pieces + pieces - 1).
-        # A slot id, page * block_size + offset, is the same number either way.  So the
-        # matrix-core kernels, which are built for pages of 16, serve every such size.
-        self.kernel_block = KERNEL_PAGE if block_size > KERNEL_PAGE and block_size % KERNEL_PAGE == 0 \
-            else block_size
-        self.pieces = block_size // self.kernel_block
         self.num_blocks = num_blocks
         self.max_seqs = max_seqs
-        self.site_specs = list(site_specs)
+        self.site_needs: List[Tuple[CacheNeed, ...]] = []
+        for i, spec in enumerate(site_specs):
+            needs = () if spec is None else tuple(spec) if isinstance(spec, (tuple, list)) else (spec,)
+            for need in needs:
+                if not isinstance(need, CacheNeed):
+                    raise TypeError(f"site {i}: {need!r} is not a cache need")
+            self.site_needs.append(needs)
+        # What a group's kernels see: where a need's kernels are built for a smaller page than
+        # the manager's (a page of 32, 48, 64, ... tokens for kernels made for 16), a page lies
+        # in memory as that many kernel pages in a row, and the block tables that go to the
+        # device name those (page p becomes p * pieces ... p * pieces + pieces - 1).  A slot id,
+        # page * block_size + offset, is the same number either way.
         self.groups: List[PageGroup] = []
-        self.site_group: Dict[int, int] = {}
-        self.state_sites: List[int] = []
-        for i, spec in enumerate(self.site_specs):
-            if spec is None:
-                continue
-            if isinstance(spec, PagedKV):
+        self.need_group: Dict[Tuple[int, int], int] = {}     # (site, which of its needs) -> group
+        for i, needs in enumerate(self.site_needs):
+            for k, need in enumerate(needs):
+                if not need.paged:
+                    continue
                 for gi, g in enumerate(self.groups):
-                    if g.spec == spec:
+                    if g.spec == need:
                         g.sites.append(i)
-                        self.site_group[i] = gi
+                        self.need_group[(i, k)] = gi
                         break
                 else:
-                    self.groups.append(PageGroup(spec, [i], PagePool(num_blocks, scatter_pages)))
-                    self.site_group[i] = len(self.groups) - 1
-            elif isinstance(spec, FixedState):
-                self.state_sites.append(i)
-            else:
-                raise TypeError(f"site {i}: unknown cache need {spec!r}")
+                    page = int(need.kernel_page(block_size))
+                    if page <= 0 or block_size % page:
+                        raise ValueError(f"site {i}: a kernel page of {page} tokens does not divide "
+                                         f"the page size {block_size}")
+                    self.groups.append(PageGroup(need, [i], PagePool(num_blocks, scatter_pages),
+                                                 page, block_size // page))
+                    self.need_group[(i, k)] = len(self.groups) - 1
+        self.has_fixed_state = any(not need.paged for needs in self.site_needs for need in needs)
         self.slots = SlotPool(max_seqs)
         self.requests: Dict[Hashable, RequestState] = {}
-        # device tensors (made by allocate_tensors)
-        self.kv: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
-        self.state: Dict[int, torch.Tensor] = {}
+        # device memory (made by allocate_tensors): per site, what each of its needs allocated
+        self.storage: Dict[int, Tuple[Any, ...]] = {}
 
     # ------------------------------------------------------------------ tensors
     def bytes_per_block(self, dtype: torch.dtype) -> int:
-        size = torch.empty((), dtype=dtype).element_size()
-        total = 0
-        for g in self.groups:
-            total += len(g.sites) * 2 * g.spec.num_kv_heads * self.block_size * g.spec.head_dim * size
-        return total
+        """Bytes that one page costs over all paged sites."""
+        return sum(len(g.sites) * g.spec.bytes_per_page(self.block_size, dtype) for g in self.groups)
 
-    def state_bytes(self) -> int:
-        """Bytes of the per-request state tensors of all state sites."""
-        total = 0
-        for site in self.state_sites:
-            spec = self.site_specs[site]
-            count = self.max_seqs
-            for n in spec.shape:
-                count *= int(n)
-            total += count * torch.empty((), dtype=spec.dtype).element_size()
-        return total
+    def state_bytes(self, dtype: torch.dtype = torch.float32) -> int:
+        """Bytes of the per-request pieces of all fixed needs."""
+        return sum(self.max_seqs * need.bytes_per_request(dtype)
+                   for needs in self.site_needs for need in needs if not need.paged)
+
+    def layout_of(self, site: int, which: int) -> CacheLayout:
+        gi = self.need_group.get((site, which))
+        page = self.groups[gi].kernel_page if gi is not None else self.block_size
+        return CacheLayout(self.num_blocks, self.block_size, page, self.max_seqs)
 
     def allocate_tensors(self, dtype: torch.dtype, device) -> None:
-        """Per paged site: keys [num_blocks * pieces, kv_heads, kernel_block, head_dim] and
-        values [num_blocks * pieces, kv_heads, head_dim, kernel_block] (transposed inside a
-        page); state per state site: [max_seqs, *shape]."""
-        for g in self.groups:
-            pages = self.num_blocks * self.pieces
-            k_shape = (pages, g.spec.num_kv_heads, self.kernel_block, g.spec.head_dim)
-            v_shape = (pages, g.spec.num_kv_heads, g.spec.head_dim, self.kernel_block)
-            for site in g.sites:
-                self.kv[site] = (torch.zeros(k_shape, dtype=dtype, device=device),
-                                 torch.zeros(v_shape, dtype=dtype, device=device))
-        for site in self.state_sites:
-            spec = self.site_specs[site]
-            self.state[site] = torch.zeros((self.max_seqs,) + tuple(spec.shape), dtype=spec.dtype,
-                                           device=device)
+        """Every need makes its own memory (``CacheNeed.allocate``); the manager keeps it by site
+        and hands it to the site's view of a step."""
+        for i, needs in enumerate(self.site_needs):
+            if needs:
+                self.storage[i] = tuple(need.allocate(self.layout_of(i, k), dtype, device)
+                                        for k, need in enumerate(needs))
+
+    def start_slots(self, slots: Sequence[int]) -> None:
+        """Requests begin in these slots: every need brings its memory there to its initial state."""
+        for i, stored in self.storage.items():
+            for need, storage in zip(self.site_needs[i], stored):
+                for slot in slots:
+                    need.start(storage, slot)
 
     # ------------------------------------------------------------------ requests
     def has(self, request: Hashable) -> bool:

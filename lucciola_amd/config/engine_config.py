@@ -42,6 +42,7 @@ class EngineConfig:
     graph_max_batch: int = 256      # largest decode batch that is captured
     graph_cache_size: int = 16      # captured steps kept
     run_ahead: bool = True          # queue a step before the host has the tokens of the one before
+    time_steps: bool = False        # bracket every step with two events: LLMEngine.stats() gives its GPU time
 
     def __post_init__(self) -> None:
         self.dtype = parse_dtype(self.dtype)

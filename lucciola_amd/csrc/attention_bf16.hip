@@ -490,7 +490,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     const bf16* __restrict__ v_cache, bf16* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ block_table, int max_blocks, int nh, int nkv, float scale_log2,
     int window, DecodePrologue pro, int splits, float* __restrict__ part_o,
-    float* __restrict__ part_ml) {
+    float* __restrict__ part_ml, int resident) {
     constexpr int QT = HPW, NP = PF_NP;
     constexpr int KLD = D + 8;
     constexpr int KPAGE = PAGE * KLD, VPAGE = D * PAGE;   // elements of a page in LDS
@@ -508,7 +508,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     // tasks from the shortest up.
     const int total = gridDim.x * gridDim.y, number = blockIdx.y * gridDim.x + blockIdx.x;
     const int half = (total + 1) / 2;
-    const int task = (total <= 2 * 256 && number >= half) ? total - 1 - (number - half) : number;
+    const int task = (total <= resident && number >= half) ? total - 1 - (number - half) : number;
     // with few tiles and many keys, a tile's pages are cut into `splits` shares (x counts tile
     // and share), each a workgroup of its own whose sums a second kernel joins
     const int tile_share = task / gridDim.y, heads_index = task - tile_share * gridDim.y;
@@ -797,7 +797,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_wide_kernel(
     const bf16* __restrict__ qkv, int q_stride, const bf16* __restrict__ k_cache,
     const bf16* __restrict__ v_cache, bf16* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ block_table, int max_blocks, int nh, int nkv, float scale_log2,
-    int window, DecodePrologue pro) {
+    int window, DecodePrologue pro, int resident) {
     static_assert(D == 128, "heads of 128");
     constexpr int NP = PF_NP;
     constexpr int KLD = D + 8;
@@ -815,7 +815,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_wide_kernel(
     // long: the second half of the numbers takes the tiles from the shortest up.
     const int total = gridDim.x * gridDim.y, number = blockIdx.y * gridDim.x + blockIdx.x;
     const int half_of = (total + 1) / 2;
-    const int task = (total <= 2 * 256 && number >= half_of) ? total - 1 - (number - half_of) : number;
+    const int task = (total <= resident && number >= half_of) ? total - 1 - (number - half_of) : number;
     const int tile_index = task / gridDim.x, heads_index = task - tile_index * gridDim.x;
     const int h = heads_index * 2 + (wave >> 1);
     const int wrow = (wave & 1) * 32;
@@ -983,7 +983,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_wide_kernel(
     }
 }
 
-static int g_decode_waves = 0;   // 0: by the launch's shape
+static thread_local int g_decode_waves = 0;   // 0: by the launch's shape
 
 template <int D>
 static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* out,
@@ -1018,22 +1018,23 @@ static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* 
 // would get nothing to do, single heads and twice the workgroups are faster (measured)
 // (where the keys are shared out, the shares fill the CUs, and pairs stay)
 static bool prefill_head_pairs(int NT, int nh, int nkv, int splits) {
-    return (nh / nkv) % 2 == 0 && ((long long)NT * (nh / 2) > 128 || splits > 1);
+    return (nh / nkv) % 2 == 0 && ((long long)NT * (nh / 2) > device_cus() / 2 || splits > 1);
 }
 
-static int g_prefill_wide = 1;   // 0: never the kernel built from the wide products (tests, tuning)
+static thread_local int g_prefill_wide = 1;   // 0: never the kernel built from the wide products (tests, tuning)
 
 template <int D>
 static int launch_prefill(const bf16* qkv, int q_stride, const bf16* k, const bf16* v, bf16* out,
                           const int* tiles, const int* table, int max_blocks, int NT, int nh,
                           int nkv, float scale_log2, int window, DecodePrologue pro, int splits,
                           float* part_o, float* part_ml, hipStream_t s) {
+    const int resident = 2 * device_cus();     // workgroups of these kernels that run at once: two a CU
     if constexpr (D == 128) {
         // heads of 128 in pairs, every tile's keys walked by one workgroup: the kernel built from
         // the wide products
         if (g_prefill_wide && (nh / nkv) % 2 == 0 && splits == 1) {
             attn_prefill_wide_kernel<D><<<dim3(nh / 2, NT), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
-                                                                       max_blocks, nh, nkv, scale_log2, window, pro);
+                                                                       max_blocks, nh, nkv, scale_log2, window, pro, resident);
             LC_LAUNCH_CHECK("attn_prefill_wide");
             return 0;
         }
@@ -1041,11 +1042,11 @@ static int launch_prefill(const bf16* qkv, int q_stride, const bf16* k, const bf
     if (prefill_head_pairs(NT, nh, nkv, splits))
         attn_prefill_kernel<D, 2><<<dim3(NT * splits, nh / 2), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
                                                                             max_blocks, nh, nkv, scale_log2, window, pro,
-                                                                            splits, part_o, part_ml);
+                                                                            splits, part_o, part_ml, resident);
     else
         attn_prefill_kernel<D, 1><<<dim3(NT * splits, nh), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
                                                                         max_blocks, nh, nkv, scale_log2, window, pro,
-                                                                        splits, part_o, part_ml);
+                                                                        splits, part_o, part_ml, resident);
     LC_LAUNCH_CHECK("attn_prefill");
     if (splits > 1) {
         attn_prefill_join_kernel<D><<<dim3(NT * 64, nh), 128, 0, s>>>(part_o, part_ml, tiles, out, nh, splits);
@@ -1064,6 +1065,10 @@ LC_API int lc_attn_bf16_supported(int nh, int nkv, int d, int page_size) {
     if (nh / nkv > 16 || nh > 65535 || nkv > 65535) return 0;
     return d == 32 || d == 64 || d == 96 || d == 128;
 }
+
+// Tokens of a cache page as these kernels index it; a page of a multiple of it is served as so
+// many pages of this size in a row.
+LC_API int lc_attn_page_granule() { return PAGE; }
 
 // Whether heads of 128 in pairs go to the prefill kernel built from the wide products (1, the
 // default) or to the general one (0).  For tests and tuning.
@@ -1090,7 +1095,8 @@ LC_API int lc_attn_decode_splits(int num_decode, int nkv, int max_ctx) {
     if (num_decode <= 0) return 1;
     const int pages = (max_ctx + PAGE - 1) / PAGE;
     const long long base = (long long)num_decode * nkv;
-    long long splits = base >= 448 ? 1 : base >= 384 ? 2 : base > 256 ? 3 : 512 / base;
+    const int cus = device_cus();       // the thresholds were measured with 256 of them
+    long long splits = base >= cus * 7 / 4 ? 1 : base >= cus * 3 / 2 ? 2 : base > cus ? 3 : 2 * cus / base;
     const int most = (pages + 7) / 8;
     if (splits > most) splits = most;
     if (splits > 32) splits = 32;
@@ -1157,8 +1163,8 @@ LC_API int lc_attn_decode_bf16(const void* qkv, int q_stride, void* k_cache, voi
 LC_API int lc_attn_prefill_splits(int num_tiles, int nh, int nkv, int max_ctx) {
     if (num_tiles <= 0 || nkv <= 0) return 1;
     const long long groups = (long long)num_tiles * ((nh / nkv) % 2 == 0 ? nh / 2 : nh);
-    if (groups >= 256) return 1;
-    long long splits = 512 / groups;                      // no more workgroups than run at once
+    if (groups >= device_cus()) return 1;
+    long long splits = 2 * device_cus() / groups;         // no more workgroups than run at once
     const int most = (max_ctx + PAGE - 1) / PAGE / 64;
     if (splits > most) splits = most;
     if (splits > 16) splits = 16;

@@ -135,6 +135,10 @@ __device__ __forceinline__ head_chunk head128_norm_rope(head_chunk x, int j, con
     return out;
 }
 
+// Compute units of the GPU.  They only steer how work is laid over the device (tile plans, the
+// number of shares); no result depends on them.
+int device_cus();
+
 // Error text of the last failed call on this thread; entry points return 0 on success.
 void set_error(const char* fmt, ...);
 

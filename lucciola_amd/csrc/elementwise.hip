@@ -26,6 +26,20 @@ void set_error(const char* fmt, ...) {
     va_end(ap);
 }
 
+// Asked once per process, of the device that is current then (the library serves one GPU).
+int device_cus() {
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            return 256;     // no device to ask (a build check on a machine without one)
+        }
+        return n;
+    }();
+    return cus;
+}
+
 // ------------------------------------------------------------------------------- embedding
 template <typename TW>
 __global__ void embedding_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
@@ -414,10 +428,7 @@ LC_API int lc_rmsnorm(float* h, const void* delta, const int* rows, const float*
     // kernel, and with it the grouping of a row's sum of squares, follows from n alone
     const bool few = dt == DT_BF16 && R <= 128 && n > 2048 && n <= 8192;
     if (dt == DT_F32) {
-        if (vec && few)
-            rmsnorm_vec_kernel<float, 1024, 1><<<R, 1024, 0, stream>>>(h, (const float*)delta, rows, w, eps,
-                                                                       (float*)out, n, write_h, sumsq, shares, share_stride);
-        else if (vec)
+        if (vec)
             rmsnorm_vec_kernel<float, RN_THREADS, RN_CHUNKS><<<R, RN_THREADS, 0, stream>>>(h, (const float*)delta, rows, w, eps,
                                                                     (float*)out, n, write_h, sumsq, shares, share_stride);
         else

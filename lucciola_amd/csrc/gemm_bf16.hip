@@ -938,8 +938,9 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restric
 // lc_gemm_bf16_force_tile (tests and tuning).
 enum : int { TILE_AUTO = -1, TILE_64x128 = 0, TILE_128x128 = 1, TILE_256x128 = 2, TILE_256x192 = 3, TILE_256x256 = 4,
               TILE_192x128 = 5, TILE_192x256 = 6, TILE_64x64 = 7, TILE_COUNT = 8 };
-static int g_force_tile = TILE_AUTO;
-constexpr int kCUs = 256;
+static thread_local int g_force_tile = TILE_AUTO;   // the switches are per thread: a test that flips one
+                                                    // never changes what an engine's thread launches
+#define kCUs (::lc::device_cus())   // the GPU's compute units: they steer the tile plans only
 
 static int tile_bm(int t) {
     return (t == TILE_64x128 || t == TILE_64x64) ? 64 : t == TILE_128x128 ? 128 : (t == TILE_192x128 || t == TILE_192x256) ? 192 : 256;
@@ -979,7 +980,7 @@ static TailPlan tail_plan(int t, int M, int N, int K) {
 // workgroups (64 x 4096 x 4096 and the norm that sums its shares: 17.8 instead of 23.5 us;
 // 64 x 6144 x 4096 and the sum of its shares: 16.4 instead of 19.6); whole, it saves the kernel
 // that sums (see pick_tile).
-static int g_small_partials = 1;   // 0: shares that are handed on come from 64 x 128 tiles (tests, tuning)
+static thread_local int g_small_partials = 1;   // 0: shares that are handed on come from 64 x 128 tiles (tests, tuning)
 static bool whole_k_64x64(int M, int N, int K) {
     const long long tiles64 = tile_count(TILE_64x64, M, N);
     return (tiles64 >= kCUs && tiles64 <= 3 * kCUs) || (K <= 2048 && tiles64 >= 48);
@@ -1074,7 +1075,7 @@ static void launch_skinny(const bf16* x, const bf16* w, TO* out, int M, int N, i
 // (only where that still leaves every CU two workgroups).
 enum : int { SKINNY_DEEP = 0, SKINNY_PLAIN = 1, SKINNY_WIDE = 2, SKINNY_KEEP_X = 3 };
 constexpr int SK_KEEP_MAX = 3;   // k blocks of x per wave that fit in registers beside w's
-static int g_force_skinny = -1;
+static thread_local int g_force_skinny = -1;
 static int skinny_shape(int M, int N, int K) {
     if (g_force_skinny >= 0 && (g_force_skinny != SKINNY_KEEP_X || K <= SK_KEEP_MAX * 16 * SK_KBLOCK))
         return g_force_skinny;
@@ -1096,8 +1097,41 @@ struct SkinnyPlan {
     int shape, rows, items, groups;
     bool runs;      // the kernel that reads w in runs of 1 KB
 };
-static int g_even_rows = 1;
-static int g_runs = 1;
+static thread_local int g_even_rows = 1;
+static thread_local int g_runs = 1;
+
+// Whether gemm_runs_kernel keeps its x in registers for all of a workgroup's tiles (XS = 8) or
+// fetches it stage by stage into a ring of registers (XS = 0).
+static bool runs_keeps_x(const SkinnyPlan& p, int K) { return K / SR_K <= 8 && p.items > p.groups; }
+
+// The XS = 0 form loads x by inline assembly into registers that it reads only after a counted
+// wait; in between, the compiler takes those registers to hold values already.  That is sound
+// as long as the ring stays in registers: were one of them spilled to scratch memory, the spill
+// would store whatever the register held before the load landed.  So the compiled kernels are
+// asked, once: if any XS = 0 instantiation uses scratch memory (or cannot be asked), that form
+// is not run and the plain skinny kernel takes its sizes.
+static int runs_ring_state() {       // 1: in registers, 0: spilled, -1: could not ask
+    static const int state = [] {
+        const void* kernels[] = {
+            (const void*)gemm_runs_kernel<0, false, 0, bf16>, (const void*)gemm_runs_kernel<0, false, 0, float>,
+            (const void*)gemm_runs_kernel<1, false, 0, bf16>, (const void*)gemm_runs_kernel<1, false, 0, float>,
+            (const void*)gemm_runs_kernel<2, false, 0, float>,
+            (const void*)gemm_runs_kernel<0, true, 0, bf16>, (const void*)gemm_runs_kernel<1, true, 0, bf16>,
+        };
+        for (const void* kernel : kernels) {
+            hipFuncAttributes attr;
+            if (hipFuncGetAttributes(&attr, kernel) != hipSuccess) {
+                (void)hipGetLastError();
+                return -1;
+            }
+            if (attr.localSizeBytes != 0) return 0;
+        }
+        return 1;
+    }();
+    return state;
+}
+static bool runs_ring_in_registers() { return runs_ring_state() == 1; }
+
 static SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
     SkinnyPlan p;
     p.runs = false;
@@ -1116,7 +1150,10 @@ static SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
             p.items = (N + p.rows - 1) / p.rows;
         }
         p.groups = p.items < kCUs ? p.items : kCUs;
-        return p;
+        // the form of the kernel that keeps x in a ring of registers filled by hand-counted loads
+        // runs only when the compiler has put that ring into registers (see runs_ring_in_registers)
+        if (runs_keeps_x(p, K) || runs_ring_in_registers()) return p;
+        p.runs = false;
     }
     p.shape = skinny_shape(M, N, K);
     p.rows = p.shape == SKINNY_WIDE ? 32 : 16;
@@ -1144,9 +1181,8 @@ static void launch_skinny_any(const bf16* x, const bf16* w, TO* out, int M, int 
                               hipStream_t s) {
     const SkinnyPlan p = skinny_plan(M, N, K, EPI);
     if (p.runs) {
-        const int spt = K / SR_K;
         // x stays in registers where a workgroup has several tiles to use it for
-        if (spt <= 8 && p.items > p.groups) gemm_runs_kernel<EPI, SCALE, 8, TO><<<p.groups, 1024, 0, s>>>(x, w, out, M, N, K, p.rows, fuse);
+        if (runs_keeps_x(p, K)) gemm_runs_kernel<EPI, SCALE, 8, TO><<<p.groups, 1024, 0, s>>>(x, w, out, M, N, K, p.rows, fuse);
         else gemm_runs_kernel<EPI, SCALE, 0, TO><<<p.groups, 1024, 0, s>>>(x, w, out, M, N, K, p.rows, fuse);
         return;
     }
@@ -1247,8 +1283,8 @@ LC_API int lc_gemm_bf16_force_skinny(int shape) {
     return 0;
 }
 
-// Forces the tile shape of the tiled kernel for every later product of any M (-1: choose by
-// size again).  For tests and tuning; not for use while other threads launch products.
+// Forces the tile shape of the tiled kernel for every later product of any M that the calling
+// thread launches (-1: choose by size again).  For tests and tuning.
 LC_API int lc_gemm_bf16_force_tile(int tile) {
     LC_CHECK(tile >= TILE_AUTO && tile < TILE_COUNT, "gemm_bf16: no tile shape %d", tile);
     g_force_tile = tile;
@@ -1301,6 +1337,11 @@ LC_API int lc_gemm_bf16_runs(int on) {
     g_runs = on;
     return 0;
 }
+
+// 1: the form of the runs kernel that keeps x in a ring of registers filled by hand-counted loads
+// is compiled without scratch memory and may run; 0: it spills and is not run; -1: the kernels
+// could not be asked (no device) and it is not run.
+LC_API int lc_gemm_bf16_runs_ring_ok() { return runs_ring_state(); }
 
 LC_API int lc_gemm_bf16_even_rows(int on) {
     g_even_rows = on ? 1 : 0;

@@ -221,11 +221,14 @@ __global__ void gemm_generic_sum_kernel(const float* __restrict__ part, TO* __re
 }
 
 // Chunks a workgroup takes when they are shared out (0: they are not): with fewer than 1024
-// tiles, as many workgroups as it takes to have about 2048.
+// tiles, as many workgroups as it takes to have about 2048, if the workspace stays modest.
 static int chunks_per_workgroup(int M, int N, int K) {
     const long long tiles = (long long)((N + GB_N - 1) / GB_N) * ((M + GB_M - 1) / GB_M);
     const int chunks = (K + GB_CHUNK - 1) / GB_CHUNK;
     if (tiles >= 1024 || chunks < 2) return 0;
+    // the workspace holds every chunk's sums for all of M x N: no more than 64 M floats (256 MiB),
+    // beyond which the chunks stay with their tile (the same additions in the same order)
+    if ((long long)chunks * M * N > (64ll << 20)) return 0;
     long long shares = (2048 + tiles - 1) / tiles;
     if (shares > chunks) shares = chunks;
     if (shares < 2) return 0;

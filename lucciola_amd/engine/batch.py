@@ -15,7 +15,6 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
-from ..kernels.ops import AttentionBatch
 
 PENDING = -1        # a token that an earlier step has sampled and the host has not seen yet
 
@@ -60,16 +59,46 @@ class Carry:
 
 
 @dataclass
+class PagesView:
+    """What a step looks like to one group of cache pages: the pages every request of the batch
+    holds and the place where each token's own entry is written.  All tensors are int32 on the
+    device.  Parts that keep paged memory read it through this; what a part's kernels want
+    beyond it (work lists, records of their own) the part derives itself and may keep in
+    ``made``, which lives as long as the batch (through every replay of a captured step)."""
+
+    block_table: torch.Tensor   # [R, width] page of position // page_size, in kernel pages; -1: given back
+    slots: torch.Tensor         # [T] page * page_size + offset of each token of the batch; -1: none
+    page_size: int              # tokens of a page as the group's kernels index it
+    made: Dict[Any, Any] = field(default_factory=dict)
+
+
+@dataclass
 class SiteView:
-    """What one site of the run order sees of the step: the batch and its own cache."""
+    """What one site of the run order sees of the step: the batch and its own cache.
+
+    ``caches[k]`` is what the k-th need of the site's layer allocated (``CacheNeed.allocate``:
+    a tensor, a tuple of tensors, ...), ``page_views[k]`` the view of that need's page group
+    (None for a need without pages).  A layer with one caching part, the usual case, reads
+    ``site.cache`` and ``site.pages``; an arrangement with several hands ``site.part(k)`` to
+    the k-th of them."""
 
     batch: "StepBatch"
     index: int
     writes_cache: bool
-    page_size: int              # tokens of a page of kv and of a block-table entry, as the kernels see them
-    kv: Optional[Tuple[torch.Tensor, torch.Tensor]] = None   # keys [pages, kvh, page, d], values [pages, kvh, d, page]
-    attn: Optional[AttentionBatch] = None                    # of this site's page group
-    state: Optional[torch.Tensor] = None                     # [max_seqs, *shape]
+    caches: Tuple[Any, ...] = ()
+    page_views: Tuple[Optional[PagesView], ...] = ()
+
+    @property
+    def cache(self) -> Any:
+        return self.caches[0] if self.caches else None
+
+    @property
+    def pages(self) -> Optional[PagesView]:
+        return self.page_views[0] if self.page_views else None
+
+    def part(self, k: int) -> "SiteView":
+        return SiteView(self.batch, self.index, self.writes_cache, self.caches[k:k + 1],
+                        self.page_views[k:k + 1])
 
 
 @dataclass
@@ -87,7 +116,10 @@ class StepBatch:
     want_rows: torch.Tensor       # int32 [W] rows of the batch whose logits are wanted
     slot_ids: torch.Tensor        # int32 [R]
     feed: torch.Tensor            # int32 [T] row of the carry a token is taken from, or -1
-    groups: List[AttentionBatch] = field(default_factory=list)
+    q_offsets: Optional[torch.Tensor] = None   # int32 [R + 1]: q_start on the device
+    ctx_len: Optional[torch.Tensor] = None     # int32 [R]: cached length of each request after this step
+    max_ctx: int = 0              # the longest of them (of a captured step: what its layout allows)
+    groups: List[PagesView] = field(default_factory=list)   # by page group of the cache manager
     plans: Dict[Any, Plan] = field(default_factory=dict)   # by planner key
     num_wanted: int = 0
     buffer: Optional[torch.Tensor] = None   # the one device buffer all of the above view
@@ -218,7 +250,6 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
         planned.append((key, {name: (pk.add(a), tuple(np.shape(a))) for name, a in arrays.items()}, info))
 
     group_handles = []
-    rows = np.arange(R)
     for gi, g in enumerate(cache.groups):
         tables = [g.tables[req] for req in requests]
         mb = max((len(t) for t in tables), default=1) or 1
@@ -232,13 +263,13 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
                 flat[r, :len(t)] = np.frombuffer(t, dtype=np.int32)
         pages = flat[tok_req, positions // bs] if T else np.zeros(0, np.int32)
         slots = np.where(pages >= 0, pages * bs + positions % bs, -1).astype(np.int32)
-        if cache.pieces > 1:        # the kernels' pages: every page as its pieces in a row
-            pieces = cache.pieces
+        if g.pieces > 1:        # the kernels' pages: every page as its pieces in a row
+            pieces = g.pieces
             flat = np.where(flat[:, :, None] >= 0,
                             flat[:, :, None] * pieces + np.arange(pieces, dtype=np.int32), -1)
             flat = flat.reshape(R, mb * pieces).astype(np.int32)
             mb *= pieces
-        group_handles.append((pk.add(flat), mb, pk.add(slots)))
+        group_handles.append((pk.add(flat), mb, pk.add(slots), g.kernel_page))
 
     buffer = pk.upload(device, into)
     if refresh_only:
@@ -246,12 +277,8 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
     max_ctx = int(max(ctx_len)) if R else 0
     if pad_blocks is not None:
         max_ctx = pad_blocks * bs      # what the layout allows, not what this batch holds
-    groups = []
-    for (h_bt, mb, h_sl) in group_handles:
-        groups.append(AttentionBatch(
-            tok_req=pk.view(h_req), positions=pk.view(h_pos),
-            block_table=pk.view(h_bt, (R, mb)), q_start=pk.view(h_qs), ctx_len=pk.view(h_ctx),
-            slots=pk.view(h_sl), max_ctx=max_ctx))
+    groups = [PagesView(block_table=pk.view(h_bt, (R, mb)), slots=pk.view(h_sl), page_size=page)
+              for (h_bt, mb, h_sl, page) in group_handles]
     plans = {key: Plan({name: pk.view(h, shape) for name, (h, shape) in handles.items()}, info)
              for key, handles, info in planned}
     return StepBatch(
@@ -259,5 +286,6 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
         first_position=first_pos, slot_list=slot_list,
         max_position=int(positions.max()) if T else 0,
         token_ids=pk.view(h_tok), positions=pk.view(h_pos), tok_req=pk.view(h_req),
-        want_rows=pk.view(h_want), slot_ids=pk.view(h_slot), feed=pk.view(h_feed), groups=groups,
+        want_rows=pk.view(h_want), slot_ids=pk.view(h_slot), feed=pk.view(h_feed),
+        q_offsets=pk.view(h_qs), ctx_len=pk.view(h_ctx), max_ctx=max_ctx, groups=groups,
         plans=plans, num_wanted=num_wanted, buffer=buffer)

@@ -10,8 +10,11 @@ request runs one step too many, whose token is thrown away.
 """
 from __future__ import annotations
 
+import time
 from dataclasses import dataclass
 from typing import Callable, Dict, List, Optional, Sequence as Seq
+
+import torch
 
 from ..config.engine_config import EngineConfig
 from ..sampling.sampler import Sampler, SamplingParams
@@ -37,6 +40,7 @@ class _QueuedStep:
     seqs: List[Sequence]            # the requests a token was sampled for, in row order
     places: List[int]               # where in each request's token list that token goes
     last: List[bool]                # the request reached max_new_tokens with this token
+    events: Optional[tuple] = None  # (before, after) the step's kernels on the stream, when steps are timed
 
 
 class LLMEngine:
@@ -44,6 +48,11 @@ class LLMEngine:
         self.model = model
         self.model_config = model_config
         self.config = engine_config
+        multiple = model.portion_multiple()
+        if engine_config.max_tokens_per_step < multiple:
+            raise ValueError(f"max_tokens_per_step ({engine_config.max_tokens_per_step}) is below the "
+                             f"{multiple} tokens that this model's prompt portions are multiples of: "
+                             "no portion of a longer prompt could ever be scheduled")
         self.runner = ModelRunner(model, engine_config)
         self.scheduler = Scheduler(self.runner.cache, engine_config.max_tokens_per_step,
                                    engine_config.max_seqs,
@@ -54,6 +63,9 @@ class LLMEngine:
         self._next_id = 1
         self._queued: Optional[_QueuedStep] = None
         self.eos_token_ids = tuple(getattr(model_config, "eos_token_ids", ()) or ())
+        # seconds of host time by what they went to (the runner keeps its own for the step itself)
+        self.times = {"schedule": 0.0, "sample": 0.0, "wait": 0.0}
+        self.last_step_gpu_ms: Optional[float] = None
 
     @classmethod
     def from_folder(cls, model_path: str, engine_config: Optional[EngineConfig] = None):
@@ -118,7 +130,9 @@ class LLMEngine:
     def _launch(self, before: Optional[_QueuedStep]) -> Optional[_QueuedStep]:
         """Schedule and queue one step.  Requests whose last token is still on the device
         (sampled by ``before``) are fed from there."""
+        t_in = time.perf_counter()
         sched: ScheduledStep = self.scheduler.step()
+        self.times["schedule"] += time.perf_counter() - t_in
         if sched.num_seqs == 0:
             if before is None and self.scheduler.has_unfinished_requests() and not sched.preempted:
                 raise RuntimeError("the scheduler has requests but can run none of them")
@@ -126,6 +140,10 @@ class LLMEngine:
         carry = None
         if before is not None and before.sampled is not None:
             carry = Carry(before.sampled.ids, {s.seq_id: row for row, s in enumerate(before.seqs)})
+        events = None
+        if self.config.time_steps and self.runner.device.type == "cuda":
+            events = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+            events[0].record()
         try:
             logits = self.runner.step(sched.entries, carry)
         except BaseException:
@@ -133,9 +151,15 @@ class LLMEngine:
             raise
         sampling = [seq for seq, s in zip(sched.seqs, sched.samples) if s]
         if not sampling:
-            return _QueuedStep(None, [], [], [])
+            if events is not None:
+                events[1].record()
+            return _QueuedStep(None, [], [], [], events)
+        t_in = time.perf_counter()
         sampled = self.sampler.sample_async(logits, [s.params for s in sampling],
                                             [s.num_generated for s in sampling])
+        self.times["sample"] += time.perf_counter() - t_in
+        if events is not None:
+            events[1].record()
         places, last = [], []
         for seq in sampling:
             places.append(seq.get_len())
@@ -143,7 +167,7 @@ class LLMEngine:
             if done:
                 self.scheduler.free_sequence(seq)
             last.append(done)
-        return _QueuedStep(sampled, sampling, places, last)
+        return _QueuedStep(sampled, sampling, places, last, events)
 
     def _collect(self, step: _QueuedStep) -> List[StepOutput]:
         """Read a queued step's tokens, put them where they belong and apply the stop rules
@@ -151,7 +175,13 @@ class LLMEngine:
         outputs: List[StepOutput] = []
         if step.sampled is None:
             return outputs
-        for seq, place, last, token in zip(step.seqs, step.places, step.last, step.sampled.tokens()):
+        t_in = time.perf_counter()
+        tokens = step.sampled.tokens()          # waits until the step's ids have reached the host
+        self.times["wait"] += time.perf_counter() - t_in
+        if step.events is not None:
+            step.events[1].synchronize()
+            self.last_step_gpu_ms = step.events[0].elapsed_time(step.events[1])
+        for seq, place, last, token in zip(step.seqs, step.places, step.last, tokens):
             if place >= seq.get_len():
                 continue        # the request ended on an earlier token: this one is thrown away
             seq.token_ids[place] = token
@@ -163,16 +193,28 @@ class LLMEngine:
             outputs.append(StepOutput(seq.seq_id, token, finished))
         return outputs
 
-    def stats(self) -> Dict[str, int]:
-        """Counters: steps and tokens run, graph replays, preemptions, pages and slots in use."""
-        cache = self.runner.cache
+    def stats(self) -> Dict[str, float]:
+        """Counters (steps and tokens run, graph replays and captures, preemptions, pages and
+        slots in use) and where the host's time went, in seconds since the engine was made:
+        ``schedule_s`` deciding the steps, ``reserve_s`` checking entries and taking pages,
+        ``batch_s`` laying out batches and sending them, ``launch_s`` queueing the model's
+        kernels or replaying captured steps, ``sample_s`` queueing the sampler, ``wait_s``
+        waiting for a step's tokens to reach the host (with ``run_ahead`` the GPU works on the
+        next step meanwhile).  ``last_step_gpu_ms``: the time between two events around the
+        last step whose tokens were read, when ``EngineConfig.time_steps`` is set (the
+        reference brackets its runs with events the same way, benchmarks/basic_bench.cc:27-64)."""
+        cache, runner = self.runner.cache, self.runner
         return {
-            "steps": self.runner.steps, "tokens": self.runner.tokens,
-            "graph_replays": self.runner.graph_replays,
+            "steps": runner.steps, "tokens": runner.tokens,
+            "graph_replays": runner.graph_replays, "graph_captures": runner.graph_captures,
             "preemptions": self.scheduler.num_preemptions,
             "waiting": len(self.scheduler.waiting), "running": len(self.scheduler.running),
             "pages_total": cache.num_blocks, "pages_free": cache.num_free_blocks(),
             "slots_free": cache.slots.num_free(),
+            "schedule_s": self.times["schedule"], "reserve_s": runner.times["reserve"],
+            "batch_s": runner.times["batch"], "launch_s": runner.times["launch"],
+            "sample_s": self.times["sample"], "wait_s": self.times["wait"],
+            "last_step_gpu_ms": self.last_step_gpu_ms,
         }
 
     # ------------------------------------------------------------------ whole requests

@@ -8,6 +8,7 @@ token and appends it to the sequences itself; here sampling is a stage of its ow
 """
 from __future__ import annotations
 
+import time
 from typing import Dict, Hashable, List, Optional, Sequence
 
 import numpy as np
@@ -60,19 +61,24 @@ class ModelRunner:
         self.planners = model.batch_planners()
         self.steps = 0
         self.tokens = 0
+        # seconds of host time spent in `step`, by what it went to: checking the entries and
+        # reserving pages, laying out the batch and sending it, queueing the model's kernels
+        # (or replaying the captured step)
+        self.times = {"reserve": 0.0, "batch": 0.0, "launch": 0.0}
         # decode steps replayed from HIP graphs: (requests, block-table width) -> captured step
         self.use_graphs = (config.use_graphs and self.device.type == "cuda"
                            and config.dtype == torch.bfloat16 and model.graph_safe())
         self._graphs: Dict[tuple, "_CapturedStep"] = {}
         self._graph_epoch = None
         self.graph_replays = 0
+        self.graph_captures = 0
 
     # ------------------------------------------------------------------ sizing
     def _blocks_from_free_memory(self, needs) -> int:
         probe = CacheManager(needs, self.config.block_size, 1, self.config.max_seqs)
         free, _ = torch.cuda.mem_get_info(self.device)
         return blocks_from_free_memory(
-            free, probe.bytes_per_block(self.config.dtype), probe.state_bytes(), self.config,
+            free, probe.bytes_per_block(self.config.dtype), probe.state_bytes(self.config.dtype), self.config,
             self.model.spec.max_positions)
 
     # ------------------------------------------------------------------ the step
@@ -137,6 +143,8 @@ class ModelRunner:
                              f"{self.cache.num_free_blocks()} pages free)")
         fresh: List[int] = []
         admitted: List[Hashable] = []
+        clock = time.perf_counter
+        t_in = clock()
         try:
             for e in entries:
                 if not self.cache.has(e.request):
@@ -145,9 +153,10 @@ class ModelRunner:
                 if self.cache.length(e.request) == 0:
                     fresh.append(self.cache.slot(e.request))
                 self.cache.reserve(e.request, len(e.tokens))
-            for site, state in self.cache.state.items():
-                for slot in fresh:
-                    state[slot].zero_()
+            if fresh:
+                self.cache.start_slots(fresh)
+            t_reserved = clock()
+            self.times["reserve"] += t_reserved - t_in
 
             if self.use_graphs and len(entries) <= self.config.graph_max_batch and all(
                     len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
@@ -155,9 +164,12 @@ class ModelRunner:
             else:
                 batch = build_batch(entries, self.cache, self.device,
                                     carry_rows=carry.rows if fed else None, planners=self.planners)
+                t_built = clock()
+                self.times["batch"] += t_built - t_reserved
                 if fed:
                     ops.feed_tokens(batch.token_ids, batch.feed, carry.ids)
                 logits, num_tokens = self.model.forward(batch, self._sites(batch)), batch.num_tokens
+                self.times["launch"] += clock() - t_built
         except BaseException:
             # nothing of this step counts: reserved pages go back, requests that it admitted
             # leave again (what kernels may already have written lies beyond every length)
@@ -197,25 +209,26 @@ class ModelRunner:
         # what the original does), so that a batch that shrinks by one does not need a new graph;
         # not with per-request state, which a copy would update a second time
         real = len(entries)
-        rows = real if real <= 4 or self.cache.state_sites else -(-real // 8) * 8
+        rows = real if real <= 4 or self.cache.has_fixed_state else -(-real // 8) * 8
         entries = list(entries) + [entries[0]] * (rows - real)
-        epoch = self.model.position_epoch()
-        if epoch != self._graph_epoch:      # a position table was made anew: addresses changed
+        epoch = self.model.tables_epoch()
+        if epoch != self._graph_epoch:      # a part has made a table anew: addresses changed
             self._graphs.clear()
             self._graph_epoch = epoch
         key = (rows, pad)
         captured = self._graphs.get(key)
         next_position = max(self.cache.length(e.request) for e in entries)
-        if captured is None or not self.model.positions_ready(next_position):
+        if captured is None or not self.model.ready(next_position):
+            t_in = time.perf_counter()
             batch = build_batch(entries, self.cache, self.device, pad_blocks=pad,
                                 carry_rows=carry.rows if carry else None, planners=self.planners)
             if carry:
                 ops.feed_tokens(batch.token_ids, batch.feed, carry.ids)
             sites = self._sites(batch)
             logits = self.model.forward(batch, sites)       # runs the step (and grows tables)
-            if self.model.position_epoch() != epoch:
+            if self.model.tables_epoch() != epoch:
                 self._graphs.clear()
-                self._graph_epoch = self.model.position_epoch()
+                self._graph_epoch = self.model.tables_epoch()
             if len(self._graphs) >= self.config.graph_cache_size:
                 self._graphs.pop(next(iter(self._graphs)))
             torch.cuda.synchronize(self.device)
@@ -223,28 +236,32 @@ class ModelRunner:
             with torch.cuda.graph(graph):
                 static_logits = self.model.forward(batch, sites)
             self._graphs[key] = _CapturedStep(graph, batch, sites, static_logits)
+            self.graph_captures += 1
+            self.times["launch"] += time.perf_counter() - t_in      # a capture: the step run twice
             return logits[:real]
+        t_in = time.perf_counter()
         build_batch(entries, self.cache, self.device, pad_blocks=pad, into=captured.batch.buffer,
                     refresh_only=True, carry_rows=carry.rows if carry else None, planners=self.planners)
+        t_built = time.perf_counter()
         if carry:       # outside the graph: the carry is at another address every step
             ops.feed_tokens(captured.batch.token_ids, captured.batch.feed, carry.ids)
         captured.graph.replay()
         self.graph_replays += 1
-        return captured.logits[:real].clone()      # the next replay overwrites the graph's own output
+        logits = captured.logits[:real].clone()      # the next replay overwrites the graph's own output
+        self.times["batch"] += t_built - t_in
+        self.times["launch"] += time.perf_counter() - t_built
+        return logits
 
     def _sites(self, batch: StepBatch) -> List[SiteView]:
         sites = []
         cache = self.cache
         for index, entry in enumerate(self.model.spec.run_order):
             owner = index if entry.cache_of is None else entry.cache_of
-            view = SiteView(batch=batch, index=index, writes_cache=entry.cache_of is None,
-                            page_size=cache.kernel_block)
-            if owner in cache.kv:
-                view.kv = cache.kv[owner]
-                view.attn = batch.groups[cache.site_group[owner]]
-            if owner in cache.state:
-                view.state = cache.state[owner]
-            sites.append(view)
+            stored = cache.storage.get(owner, ())
+            views = tuple(batch.groups[cache.need_group[(owner, k)]] if (owner, k) in cache.need_group else None
+                          for k in range(len(stored)))
+            sites.append(SiteView(batch=batch, index=index, writes_cache=entry.cache_of is None,
+                                  caches=stored, page_views=views))
         return sites
 
     def finish(self, request: Hashable) -> None:

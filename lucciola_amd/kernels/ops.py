@@ -45,6 +45,8 @@ _SIGNATURES = {
     "lc_qk_norm_rope_write": "piiiiippfppipppiip",
     "lc_attention_generic": "pipppipppiiiiiifipp",
     "lc_attn_bf16_supported": "iiii",
+    "lc_attn_page_granule": "",
+    "lc_gemm_bf16_runs_ring_ok": "",
     "lc_attn_decode_splits": "iii",
     "lc_attn_decode_waves": "i",
     "lc_attn_decode_bf16": "pippppppppp" + "iiiiii" + "f" + "ii" + "ippfpii" + "pii" + "p",
@@ -63,6 +65,30 @@ _SIGNATURES = {
 
 class KernelError(RuntimeError):
     pass
+
+
+def register_signatures(signatures) -> None:
+    """Entry points of the kernel library beyond the ones listed above, ``{name: kinds}`` with one
+    letter per argument (p pointer, i int, f float; they return an int, 0 for success): a part
+    that brings kernels of its own (a source file added to ``csrc``) declares them here and
+    launches them with :func:`call`; no table in this file has to know them."""
+    for name, kinds in signatures.items():
+        bad = [c for c in kinds if c not in _ARG]
+        if bad:
+            raise KernelError(f"entry point {name}: unknown argument kinds {bad} (p, i or f)")
+        if _SIGNATURES.get(name, kinds) != kinds:
+            raise KernelError(f"entry point {name} is already declared as '{_SIGNATURES[name]}'")
+        if _lib is not None:
+            _declare(_lib, name, kinds)
+        _SIGNATURES[name] = kinds
+
+
+def _declare(lib, name: str, kinds: str) -> None:
+    fn = getattr(lib, name, None)
+    if fn is None:
+        raise KernelError(f"the kernel library lacks the entry point {name}")
+    fn.restype = ctypes.c_int
+    fn.argtypes = [_ARG[c] for c in kinds]
 
 
 def _dt(t: torch.Tensor) -> int:
@@ -90,11 +116,7 @@ def library():
         lib.lc_attention_generic_workspace.restype = ctypes.c_longlong
         lib.lc_attention_generic_workspace.argtypes = [ctypes.c_int] * 5
         for name, sig in _SIGNATURES.items():
-            fn = getattr(lib, name, None)
-            if fn is None:
-                raise KernelError(f"the kernel library {path} lacks the entry point {name}")
-            fn.restype = ctypes.c_int
-            fn.argtypes = [_ARG[c] for c in sig]
+            _declare(lib, name, sig)
         _lib = lib
     return _lib
 
@@ -110,6 +132,13 @@ def _call(name: str, *args) -> None:
     rc = fn(*args)
     if rc != 0:
         raise KernelError(lib.lc_last_error().decode("utf-8", "replace"))
+
+
+def call(name: str, *args) -> None:
+    """Launch a declared entry point (see :func:`register_signatures`); raises KernelError with
+    the library's message if it reports a failure.  ``ptr(tensor)`` and ``stream()`` make the
+    pointer and stream arguments."""
+    _call(name, *args)
 
 
 def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
@@ -140,6 +169,8 @@ def _need(t: torch.Tensor, what: str, dtype=None, dim: Optional[int] = None) -> 
     if dim is not None and t.dim() != dim:
         raise KernelError(f"{what}: expected {dim} dimensions, got shape {tuple(t.shape)}")
 
+
+ptr, stream = _ptr, _stream       # public names, for parts that bring kernels of their own
 
 _c_int, _c_float = ctypes.c_int, ctypes.c_float
 
@@ -542,17 +573,28 @@ def plan_attention(layout):
             {"num_decode": int(decode.size), "all_decode": int(decode.size) == R})
 
 
-def attention_batch(generic: AttentionBatch, plan) -> AttentionBatch:
-    """``generic`` (a page group's view of the batch) with the work lists of ``plan`` (made by
-    :func:`plan_attention`; None: without, and only the generic kernel can run)."""
-    if plan is None:
-        return generic
-    done = plan.made.get(id(generic))
+def attention_page_granule() -> int:
+    """Tokens of a cache page as the matrix-core attention kernels index it: a page of a
+    multiple of it reaches them as so many pages of this size."""
+    return int(library().lc_attn_page_granule())
+
+
+def attention_batch(batch, pages, plan=None) -> AttentionBatch:
+    """The attention kernels' record of a step: from the step's batch (``engine.batch.StepBatch``:
+    tok_req, positions, q_offsets, ctx_len, max_ctx), a page group's view of it (``PagesView``:
+    block table, slots) and the work lists of ``plan`` (made by :func:`plan_attention`; None:
+    without, and only the generic kernel can run).  Made once a step and page group, kept in
+    ``pages.made``."""
+    done = pages.made.get(ATTENTION_PLAN)
     if done is None:
-        done = replace(generic, decode_tokens=plan.arrays["decode_tokens"],
-                       prefill_tiles=plan.arrays["prefill_tiles"],
-                       num_decode=plan.info["num_decode"], all_decode=plan.info["all_decode"])
-        plan.made[id(generic)] = done
+        done = AttentionBatch(tok_req=batch.tok_req, positions=batch.positions,
+                              block_table=pages.block_table, q_start=batch.q_offsets,
+                              ctx_len=batch.ctx_len, slots=pages.slots, max_ctx=batch.max_ctx)
+        if plan is not None:
+            done = replace(done, decode_tokens=plan.arrays["decode_tokens"],
+                           prefill_tiles=plan.arrays["prefill_tiles"],
+                           num_decode=plan.info["num_decode"], all_decode=plan.info["all_decode"])
+        pages.made[ATTENTION_PLAN] = done
     return done
 
 

@@ -11,6 +11,7 @@ argmax, src/qwen.cc:875-892).
 from __future__ import annotations
 
 import math
+import sys
 from typing import Callable, Dict, List, Optional
 
 import torch
@@ -19,7 +20,7 @@ from ..config.registry import BLOCKS, EMBEDDINGS, FAMILIES, HEADS, NORMS
 from ..config.specs import LayerSpec, ModelSpec, PartSpec
 from ..engine.batch import SiteView, StepBatch
 from ..parts import BuildContext, ResidualStream, build_part
-from ..weights.loader import ParamDecl, WeightSource, load_declared
+from ..weights.loader import ParamDecl, WeightSource, load_declared, precision_notices
 
 
 class _LayerParts:
@@ -41,10 +42,9 @@ class _LayerParts:
                                  f"unknown family '{family}'")
             self.by_slot[slot] = build_part(FAMILIES[family], spec.parts[slot])
         self.block = block_cls(**self.by_slot)
-        caching = [p for p in self.by_slot.values() if p.cache_need() is not None]
-        if len(caching) > 1:
-            raise ValueError(f"a layer may hold one part with a cache, this one has {len(caching)}")
-        self.cache_part = caching[0] if caching else None
+        # the parts that keep something in the cache, in the order of the block's slots: a site's
+        # view holds their memory in this order (``SiteView.caches``, ``SiteView.part(k)``)
+        self.caching = [p for p in self.by_slot.values() if p.cache_need() is not None]
 
     def __getattr__(self, slot):          # layer.mixer, layer.feed_forward_norm, ...
         try:
@@ -112,8 +112,14 @@ class CausalLM:
         spec.validate()
         self.spec = spec
         self.ctx = BuildContext(dtype=dtype, device=torch.device(device))
-        tensors = load_declared(source, declared_tensors(spec), self.ctx.device,
-                                optional=optional_names)
+        declared = declared_tensors(spec)
+        stored: Dict[str, torch.dtype] = {}
+        tensors = load_declared(source, declared, self.ctx.device, optional=optional_names,
+                                stored_dtypes=stored)
+        # what the kept dtypes cost, said once per class of tensor
+        self.load_notices = precision_notices(stored, declared, self.ctx.dtype)
+        for line in self.load_notices:
+            print(f"[lucciola_amd] {line}", file=sys.stderr, flush=True)
         self.embed, self.head_part, head_names = _end_parts(spec)
         self.embed.bind({"weight": tensors[spec.embedding_name]}, self.ctx)
         self.head_part.bind({logical: tensors[head_names[logical]]
@@ -144,12 +150,17 @@ class CausalLM:
 
     # ------------------------------------------------------------------ cache needs
     def site_needs(self) -> List[Optional[object]]:
-        """For each site of the run order: what it needs of the cache (None when it reads
-        another site's cache or needs nothing)."""
+        """For each site of the run order: what it needs of the cache: a need, a tuple of needs
+        (a layer with several caching parts) or None (it reads another site's cache or needs
+        nothing)."""
         needs = []
         for entry in self.spec.run_order:
-            part = self.layers[entry.layer].cache_part
-            needs.append(None if entry.cache_of is not None or part is None else part.cache_need())
+            caching = self.layers[entry.layer].caching
+            if entry.cache_of is not None or not caching:
+                needs.append(None)
+            else:
+                mine = tuple(part.cache_need() for part in caching)
+                needs.append(mine[0] if len(mine) == 1 else mine)
         return needs
 
     def graph_safe(self) -> bool:
@@ -174,20 +185,15 @@ class CausalLM:
             multiple = math.lcm(multiple, int(getattr(part, "portion_multiple", 1)))
         return multiple
 
-    # ------------------------------------------------------------------ position tables
-    def _position_parts(self):
-        for part in self._all_parts():
-            pos = getattr(part, "position", None)
-            if pos is not None and hasattr(pos, "generation"):
-                yield pos
+    # ------------------------------------------------------------------ tables that parts grow
+    def tables_epoch(self) -> int:
+        """Changes whenever a part has made a device table anew (``Part.tables_epoch``): kernel
+        arguments captured before that point at the old one."""
+        return sum(part.tables_epoch() for part in self._all_parts())
 
-    def position_epoch(self) -> int:
-        """Changes whenever a position table has been made anew (its address has changed)."""
-        return sum(p.generation for p in self._position_parts())
-
-    def positions_ready(self, position: int) -> bool:
-        """Whether every position table already covers ``position``."""
-        return all(p.capacity() > position for p in self._position_parts())
+    def ready(self, position: int) -> bool:
+        """Whether every part can serve ``position`` without making a table anew."""
+        return all(part.ready(position) for part in self._all_parts())
 
     # ------------------------------------------------------------------ forward
     def forward(self, batch: StepBatch, sites: List[SiteView]) -> torch.Tensor:

@@ -81,13 +81,22 @@ class Attention(Part):
             qkv[:, cols] = norm.apply(x).view(T, heads * self.d)
 
     def cache_need(self):
-        return PagedKV(self.nkv, self.d, self.window)
+        return PagedKV(self.nkv, self.d, self.window, granule=ops.attention_page_granule())
 
     def batch_planner(self):
         return ops.ATTENTION_PLAN, ops.plan_attention
 
+    def tables_epoch(self) -> int:
+        return self.position.tables_epoch() if self.position is not None else 0
+
+    def ready(self, position: int) -> bool:
+        return self.position.ready(position) if self.position is not None else True
+
     def forward(self, x: torch.Tensor, site) -> torch.Tensor:
-        attn = ops.attention_batch(site.attn, site.batch.plans.get(ops.ATTENTION_PLAN))
+        # the attention kernels' record of the step: made once a step for the page group, from
+        # the batch, the group's pages and the work lists of this part's planner
+        attn = ops.attention_batch(site.batch, site.pages, site.batch.plans.get(ops.ATTENTION_PLAN))
+        page_size = site.pages.page_size
         q_w = k_w = None
         eps = 0.0
         own_norm = self.q_norm is not None and not self.fused_qk_norm
@@ -101,15 +110,15 @@ class Attention(Part):
         # as it reads them, the kernel that would sum them is saved
         rows = x.x.shape[0] if isinstance(x, ops.ScaledRows) else x.shape[0]
         as_shares = ((table is not None or self.position is None) and not own_norm
-                     and ops.attention_takes_shares(attn, rows, self.nh, self.nkv, self.d, site.page_size,
+                     and ops.attention_takes_shares(attn, rows, self.nh, self.nkv, self.d, page_size,
                                                     self.dtype, table.shape[1] if table is not None else 0))
         qkv = ops.gemm(x, self.qkv, self.dtype, shares=as_shares)
         if own_norm:
             self._norm_heads(qkv)
         if self.position is not None and table is None:
             self.position.apply(qkv, self.nh, self.nkv, self.d, attn.positions)
-        k_cache, v_cache = site.kv
+        k_cache, v_cache = site.cache
         prologue = ops.QKPrologue(q_w, k_w, eps, table, attn.slots if site.writes_cache else None)
-        o = ops.attention(qkv, attn, k_cache, v_cache, self.nh, self.nkv, self.d, site.page_size,
+        o = ops.attention(qkv, attn, k_cache, v_cache, self.nh, self.nkv, self.d, page_size,
                           self.scale, self.window or 0, prologue)
         return ops.gemm(o, self.o, self.dtype, defer=True)

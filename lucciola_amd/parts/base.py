@@ -12,8 +12,9 @@ Interfaces (all tensors on the GPU; "act" is the engine's activation dtype):
                   return ops.ScaledRows; stream.pending may be an ops.PendingProduct
   PositionEncoding  rotary_table(max_position) -> float32 [positions, rot] or None;
                   apply(qkv, nh, nkv, d, positions) in place, when there is no table
-  Mixer           forward(x act [T, H], site: SiteView) -> act [T, H]; cache_need() -> spec;
-                  batch_planner() -> (key, plan) or None; portion_multiple
+  Mixer           forward(x act [T, H], site: SiteView) -> act [T, H]; cache_need() -> a
+                  CacheNeed or None; batch_planner() -> (key, plan) or None; portion_multiple;
+                  tables_epoch(), ready(position) where it grows device tables
   FeedForward     forward(x act [T, H]) -> act [T, H]
                   A mixer or feed-forward with takes_scaled_rows = True may be given
                   ops.ScaledRows as x (ops.gemm and ops.gemm_swiglu take them) and may return
@@ -24,7 +25,7 @@ Interfaces (all tensors on the GPU; "act" is the engine's activation dtype):
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Any, Dict
 
 import torch
@@ -38,6 +39,9 @@ from ..weights.loader import ParamDecl
 class BuildContext:
     dtype: torch.dtype      # activation dtype of the engine: bfloat16 or float32
     device: torch.device
+    # what parts of ONE model share (a position table that all its layers use): made with the
+    # model, gone with it; nothing is shared between models
+    shared: Dict[Any, Any] = field(default_factory=dict)
 
 
 class ResidualStream:
@@ -78,8 +82,21 @@ class Part:
         """Take the declared tensors (already on the device, in their kept dtype)."""
 
     def cache_need(self):
-        """Mixers: a cache spec (PagedKV, FixedState) or None."""
+        """What this part keeps in the cache: a ``cache.specs.CacheNeed`` (PagedKV, FixedState or
+        a subclass of the part's own) or None.  What the need allocates is what the part finds
+        as ``site.cache``; a paged need also finds ``site.pages`` (block table, slots, page
+        size)."""
         return None
+
+    def tables_epoch(self) -> int:
+        """A number that changes whenever this part has made a device table anew whose address
+        kernels take as an argument (a position table that has grown): steps captured before
+        are captured again.  A part that nests other parts adds theirs."""
+        return 0
+
+    def ready(self, position: int) -> bool:
+        """Whether the part can serve ``position`` without making such a table anew."""
+        return True
 
     def batch_planner(self):
         """Work lists this part's kernels want made from every step's batch, once a step and

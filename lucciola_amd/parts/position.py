@@ -8,7 +8,7 @@ float32) and the kernel looks them up; the table grows when a longer position sh
 """
 from __future__ import annotations
 
-from typing import Dict, Optional, Tuple
+from typing import Optional
 
 import torch
 
@@ -17,15 +17,13 @@ from .base import BuildContext, Part
 
 
 class _SharedTable:
-    """One table for all parts with the same rotated size, base and device (the layers of a
-    model, usually): ``generation`` counts how often it has been made anew."""
+    """One table for all parts of a model with the same rotated size and base (its layers,
+    usually), kept in the model's ``BuildContext.shared``: ``generation`` counts how often it
+    has been made anew."""
 
     def __init__(self) -> None:
         self.table: Optional[torch.Tensor] = None
         self.generation = 0
-
-
-_TABLES: Dict[Tuple[int, float, str], _SharedTable] = {}
 
 
 @POSITION_ENCODINGS.register("rotary")
@@ -41,12 +39,13 @@ class Rotary(Part):
 
     def bind(self, tensors, ctx: BuildContext) -> None:
         self._device = ctx.device
-        self._shared = _TABLES.setdefault((self.rotary_dim, self.theta, str(torch.device(ctx.device))),
-                                          _SharedTable())
+        self._shared = ctx.shared.setdefault(("rotary table", self.rotary_dim, self.theta), _SharedTable())
 
-    @property
-    def generation(self) -> int:
+    def tables_epoch(self) -> int:
         return self._shared.generation
+
+    def ready(self, position: int) -> bool:
+        return self.capacity() > position
 
     @property
     def _table(self) -> Optional[torch.Tensor]:

@@ -8,7 +8,9 @@ The reference prints a message and carries on with a null pointer when a tensor 
 
 Kept as stored: bfloat16 stays bfloat16 and a tensor stored in 32-bit stays 32-bit; float16
 and float64 become float32; integer tables become int32.  Small vectors that kernels read as
-float32 (norm weights) are widened to float32, which changes no value.
+float32 (norm weights) are widened to float32, which changes no value.  No matrix is ever
+rounded at load; what keeping a wide matrix costs in a bfloat16 engine (its products do not
+run on the matrix cores) is said once per class of tensor (:func:`precision_notices`).
 """
 from __future__ import annotations
 
@@ -155,12 +157,32 @@ def kept_dtype(stored: torch.dtype, role: str) -> Optional[torch.dtype]:
     return torch.float32
 
 
+def precision_notices(stored: Mapping[str, torch.dtype], declared: Mapping[str, ParamDecl],
+                      engine_dtype: torch.dtype) -> List[str]:
+    """What the kept dtypes mean for speed, one line per class of tensor: in a bfloat16 engine
+    a matrix that is stored wider than bfloat16 stays float32, and every product with it takes
+    the general kernel instead of the matrix cores."""
+    if engine_dtype != torch.bfloat16:
+        return []
+    classes: Dict[torch.dtype, List[str]] = {}
+    for name, dtype in stored.items():
+        decl = declared.get(name)
+        if decl is not None and decl.role == "matrix" and kept_dtype(dtype, "matrix") == torch.float32:
+            classes.setdefault(dtype, []).append(name)
+    return [f"{len(names)} matrices stored as {str(dtype).replace('torch.', '')} stay float32 (for one, {names[0]}): "
+            "in a bfloat16 engine their products run on the general kernel, without the matrix cores, "
+            "correct and many times slower; store them as bfloat16 to have the fast kernels"
+            for dtype, names in classes.items()]
+
+
 def load_declared(source: WeightSource, declared: Mapping[str, ParamDecl],
-                  device: torch.device, optional: Iterable[str] = ()) -> Dict[str, torch.Tensor]:
+                  device: torch.device, optional: Iterable[str] = (),
+                  stored_dtypes: Optional[Dict[str, torch.dtype]] = None) -> Dict[str, torch.Tensor]:
     """Check ``source`` against ``declared`` and bring every declared tensor to ``device``.
 
     ``optional`` names may be present in the source without being declared (a tied model's
-    checkpoint may still carry ``lm_head.weight``); they are not loaded.
+    checkpoint may still carry ``lm_head.weight``); they are not loaded.  ``stored_dtypes``: a
+    dict that is filled with the dtype every loaded tensor has in the source.
     """
     have = set(source.names())
     optional = set(optional)
@@ -181,6 +203,8 @@ def load_declared(source: WeightSource, declared: Mapping[str, ParamDecl],
     out: Dict[str, torch.Tensor] = {}
     for name, decl in declared.items():
         t = source.get(name)
+        if stored_dtypes is not None:
+            stored_dtypes[name] = t.dtype
         target = kept_dtype(t.dtype, decl.role)
         # one copy: to the device first (as stored), then widen there if needed
         t = t.to(device=device, non_blocking=False)

@@ -60,8 +60,8 @@ def test_slots():
 def test_groups_are_formed_by_equal_needs():
     cm = CacheManager([FULL, WINDOW, FULL, None, FixedState((3,)), WINDOW], 4, 20, 4)
     assert [g.sites for g in cm.groups] == [[0, 2], [1, 5]]
-    assert cm.state_sites == [4]
-    assert cm.site_group == {0: 0, 2: 0, 1: 1, 5: 1}
+    assert cm.has_fixed_state and [i for i, n in enumerate(cm.site_needs) if n and not n[0].paged] == [4]
+    assert cm.need_group == {(0, 0): 0, (2, 0): 0, (1, 0): 1, (5, 0): 1}
 
 
 def test_pages_follow_the_length():
@@ -159,3 +159,61 @@ def test_random_orders_of_requests(seed):
         cm.release(name)
     cm.check()
     assert all(g.pool.num_free() == 40 for g in cm.groups) and cm.slots.num_free() == 5
+
+
+def test_a_need_of_another_layout_and_two_needs_at_one_site():
+    """The manager only counts: a need that is no key/value pair (one tensor of latents per
+    site, with a kernel page of its own) makes its own memory, and a site may hold several
+    needs (a layer with two caching parts)."""
+    from dataclasses import dataclass
+    import torch
+    from lucciola_amd.cache.specs import CacheNeed
+
+    @dataclass(frozen=True)
+    class Latents(CacheNeed):
+        rank: int
+        window: int = None
+        paged = True
+
+        def kernel_page(self, page_size):
+            return 4 if page_size % 4 == 0 else page_size
+
+        def bytes_per_page(self, page_size, dtype):
+            return page_size * self.rank * 4
+
+        def allocate(self, layout, dtype, device):
+            return torch.zeros((layout.kernel_pages, layout.kernel_page, self.rank), device=device)
+
+    class Ring(CacheNeed):
+        def bytes_per_request(self, dtype):
+            return 40
+
+        def allocate(self, layout, dtype, device):
+            return {"ring": torch.ones((layout.max_seqs, 10)), "started": []}
+
+        def start(self, storage, slot):
+            storage["started"].append(slot)
+            storage["ring"][slot] = 0
+
+    ring = Ring()
+    cm = CacheManager([Latents(6), (Latents(6), FULL, ring), None, Latents(6, window=8)], 8, 10, 3)
+    assert [g.sites for g in cm.groups] == [[0, 1], [1], [3]]
+    assert [(g.kernel_page, g.pieces) for g in cm.groups] == [(4, 2), (8, 1), (4, 2)]
+    assert cm.need_group == {(0, 0): 0, (1, 0): 0, (1, 1): 1, (3, 0): 2} and cm.has_fixed_state
+    assert cm.bytes_per_block(torch.float32) == 3 * 8 * 6 * 4 + 2 * 2 * 8 * 16 * 4
+    assert cm.state_bytes() == 3 * 40
+    cm.allocate_tensors(torch.float32, "cpu")
+    assert sorted(cm.storage) == [0, 1, 3] and len(cm.storage[1]) == 3
+    assert cm.storage[0][0].shape == (20, 4, 6) and cm.storage[1][1][0].shape == (10, 2, 8, 16)
+    slot = cm.admit("a")
+    cm.start_slots([slot])
+    assert cm.storage[1][2]["started"] == [slot] and float(cm.storage[1][2]["ring"][slot].sum()) == 0
+    cm.reserve("a", 20)
+    cm.commit("a")
+    assert [len(g.tables["a"]) for g in cm.groups] == [3, 3, 3]
+    assert list(cm.groups[2].tables["a"])[0] == -1        # the window of 8 has passed the first page
+    cm.check()
+    cm.release("a")
+    assert all(g.pool.num_free() == 10 for g in cm.groups)
+    with pytest.raises(TypeError, match="not a cache need"):
+        CacheManager([object()], 8, 10, 3)

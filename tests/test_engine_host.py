@@ -54,8 +54,8 @@ def test_pages_of_several_kernel_pages(monkeypatch, key, page, family):
     steps = {"chunked": traces.chunked, "mixed": traces.mixed}[family](prompts)
     blocks = traces.max_live_tokens(steps, page) // page
     runner, weights = make(cfg, seed, page, blocks)
-    assert runner.cache.kernel_block == 16 and runner.cache.pieces == page // 16
-    assert runner.cache.kv[0][0].shape[0] == blocks * (page // 16) and runner.cache.kv[0][0].shape[2] == 16
+    assert runner.cache.groups[0].kernel_page == 16 and runner.cache.groups[0].pieces == page // 16
+    assert runner.cache.storage[0][0][0].shape[0] == blocks * (page // 16) and runner.cache.storage[0][0][0].shape[2] == 16
     got = replay(runner, steps)
     compare(got, cfg, weights, prompts, 2e-5)
     for g in runner.cache.groups:
@@ -253,3 +253,42 @@ def test_a_step_that_raises_leaves_the_cache_and_the_queues_as_they_were(monkeyp
         assert seen[i] == plain_qwen3.greedy(cfg, weights, p, 6)
     engine.runner.cache.check()
     assert not engine.runner.cache.requests
+
+
+def test_budgets_that_could_never_schedule_are_refused(monkeypatch):
+    """A step budget below the multiple that the model's prompt portions must have is refused
+    when the engine is made; a queue that holds requests none of which can ever run raises
+    instead of spinning."""
+    from lucciola_amd.sampling.sampler import SamplingParams
+    reference_ops.install(monkeypatch)
+    cfg, page, seed = configs.ALL["A"]
+    weights = random_weights(cfg, seed, std=0.3)
+    engine = host_engine(cfg, weights, page, 16, max_tokens_per_step=12, max_seqs=3)
+    model = engine.model
+    monkeypatch.setattr(type(model.layers[0].mixer), "portion_multiple", 16, raising=False)
+    assert model.portion_multiple() == 16
+    with pytest.raises(ValueError, match="below the 16 tokens"):
+        host_engine(cfg, weights, page, 16, max_tokens_per_step=12, max_seqs=3)
+    # a queue whose front request can never be cut into a portion (forced here past the check
+    # above): the engine says so instead of scheduling nothing for ever
+    monkeypatch.setattr(type(model.layers[0].mixer), "portion_multiple", 1, raising=False)
+    for ahead in (False, True):
+        engine = host_engine(cfg, weights, page, 16, max_tokens_per_step=12, max_seqs=3, run_ahead=ahead)
+        engine.scheduler.portion_multiple = 16
+        engine.add_request(list(range(40)), SamplingParams(max_new_tokens=2))
+        with pytest.raises(RuntimeError, match="can run none of them"):
+            engine.step()
+
+
+def test_stats_say_where_the_host_time_went(monkeypatch):
+    from lucciola_amd.sampling.sampler import SamplingParams
+    reference_ops.install(monkeypatch)
+    cfg, page, seed = configs.ALL["A"]
+    weights = random_weights(cfg, seed, std=0.3)
+    engine = host_engine(cfg, weights, page, 40, max_tokens_per_step=12, max_seqs=3, time_steps=True)
+    engine.generate(list(prompts_for(cfg, [9, 20], seed).values()), SamplingParams(max_new_tokens=5))
+    stats = engine.stats()
+    for key in ("schedule_s", "reserve_s", "batch_s", "launch_s", "sample_s", "wait_s"):
+        assert stats[key] > 0, key
+    assert stats["steps"] > 5 and stats["graph_captures"] == 0
+    assert stats["last_step_gpu_ms"] is None        # no device events on the CPU

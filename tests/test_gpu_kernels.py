@@ -847,3 +847,11 @@ def test_attention_decode_takes_q_k_v_as_shares_of_a_product(nh, nkv, window, ro
     b = ops.attention(ops.ProductShares(part5, torch.bfloat16).value(), mixed, kc3.clone(), vc3.clone(), nh, nkv, d,
                       16, d ** -0.5, window, ops.QKPrologue(qw, kw, 1e-6, table, slots5))
     assert torch.equal(a, b)
+
+
+def test_runs_kernel_keeps_its_ring_of_x_in_registers():
+    """The form of the runs kernel that fills a ring of registers with hand-counted loads is
+    only sound while the compiler keeps that ring in registers; the library asks its compiled
+    kernels and must find them without scratch memory (else it would quietly run the slower
+    kernel)."""
+    assert ops.library().lc_gemm_bf16_runs_ring_ok() == 1

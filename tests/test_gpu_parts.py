@@ -78,9 +78,9 @@ def test_rotary_part():
     cos, sin = cs[:, None, :24], cs[:, None, 24:]
     got = torch.cat([x[..., :24] * cos - x[..., 24:] * sin, x[..., :24] * sin + x[..., 24:] * cos], -1)
     torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-6)
-    epoch = rot.generation
+    epoch = rot.tables_epoch()
     bigger = rot.rotary_table(5000)           # grows on demand
-    assert bigger.shape[0] > 5000 and rot.generation == epoch + 1
+    assert bigger.shape[0] > 5000 and rot.tables_epoch() == epoch + 1 and rot.ready(5000)
     torch.testing.assert_close(bigger[:table.shape[0]], table)
 
 
@@ -113,8 +113,8 @@ def attention_site(part, T, page, dtype, first=0):
     cache.reserve("r", T)
     batch = build_batch([StepEntry("r", list(range(T)), [])], cache, DEV,
                         planners=dict([part.batch_planner()]))
-    return SiteView(batch=batch, index=0, writes_cache=True, page_size=cache.kernel_block, kv=cache.kv[0],
-                    attn=batch.groups[0]), cache
+    return SiteView(batch=batch, index=0, writes_cache=True, caches=cache.storage[0],
+                    page_views=(batch.groups[0],)), cache
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -127,7 +127,7 @@ def test_attention_part(dtype, nh, nkv, d, page, window):
         "qk_norm": PartSpec("rms", {"size": d, "eps": eps}),
         "position": PartSpec("rotary", {"rotary_dim": d, "theta": theta, "max_positions": 64})})
     part = build_part(MIXERS, spec)
-    assert part.cache_need() == PagedKV(nkv, d, window)
+    assert part.cache_need() == PagedKV(nkv, d, window, granule=16)
     names = {"q_proj": (nh * d, H), "k_proj": (nkv * d, H), "v_proj": (nkv * d, H), "o_proj": (H, nh * d),
              "q_norm.weight": (d,), "k_norm.weight": (d,)}
     assert {k: v.shape for k, v in part.declare().items()} == names
@@ -175,7 +175,7 @@ def test_run_order_names_a_layer_twice_and_shares_a_cache(dtype):
             steps = family(prompts)
             runner = ModelRunner(model, EngineConfig(dtype=dtype, block_size=page, max_seqs=4, device="cuda:0",
                                                      max_blocks=traces.max_live_tokens(steps, page) // page))
-            assert len(runner.cache.kv) == 3          # three sites own a cache, one borrows
+            assert len(runner.cache.storage) == 3     # three sites own a cache, one borrows
             got = replay(runner, steps)
             compare(got, cfg, weights, prompts, 2e-5 if dtype == "float32" else 3e-2, refs)
     finally:
@@ -205,11 +205,11 @@ class ToyDecay(Part):
         states = torch.empty_like(u)
         batch = site.batch
         for r, slot in enumerate(batch.slot_list):
-            s = site.state[slot]
+            s = site.cache[slot]
             for t in range(batch.q_start[r], batch.q_start[r + 1]):
                 s = self.decay * s + u[t]
                 states[t] = s
-            site.state[slot] = s
+            site.cache[slot] = s
         return ops.gemm(states.to(self.dtype), self.w_out, self.dtype)
 
 
@@ -299,9 +299,10 @@ def test_toy_architecture_with_a_stateful_mixer():
             steps = family(prompts)
             runner = ModelRunner(model, EngineConfig(dtype="float32", block_size=4, max_seqs=4, device="cuda:0",
                                                      max_blocks=traces.max_live_tokens(steps, 4) // 4))
-            assert sorted(runner.cache.state) == [0, 2, 3] and sorted(runner.cache.kv) == [1]
-            for state in runner.cache.state.values():
-                state.fill_(7.0)                       # a new request must not see an old state
+            assert sorted(runner.cache.storage) == [0, 1, 2, 3] and runner.cache.has_fixed_state
+            assert [site for g in runner.cache.groups for site in g.sites] == [1]
+            for site in (0, 2, 3):
+                runner.cache.storage[site][0].fill_(7.0)   # a new request must not see an old state
             got = replay(runner, steps)
             compare(got, TOY, weights, prompts, 2e-5, refs)
     finally:
@@ -329,8 +330,9 @@ def test_toy_architecture_through_the_engine_with_preemption():
             engine = LLMEngine(model, TOY, EngineConfig(dtype="float32", block_size=4, max_blocks=18,
                                                         max_seqs=4, max_tokens_per_step=12,
                                                         device="cuda:0", run_ahead=ahead))
-            for state in engine.runner.cache.state.values():
-                state.fill_(3.0)
+            for site, stored in engine.runner.cache.storage.items():
+                if isinstance(engine.runner.cache.site_needs[site][0], FixedState):
+                    stored[0].fill_(3.0)
             got = engine.generate(prompts, SamplingParams(max_new_tokens=20))
             assert engine.scheduler.num_preemptions > 0
             for prompt, tokens in zip(prompts, got):
@@ -685,3 +687,201 @@ def test_block_mixes_parts_that_take_scaled_rows_with_parts_that_do_not(rows):
         assert isinstance(stream.pending, ops.PendingProduct)
     assert rel(stream.h, want) < 2e-2
     assert rel(ops.value(stream.pending), pending) < 3e-2
+
+
+# ------------------------------------------------------------------ a paged cache of another layout
+from dataclasses import dataclass  # noqa: E402
+
+from lucciola_amd.cache.specs import CacheNeed  # noqa: E402
+
+
+@dataclass(frozen=True)
+class LatentPages(CacheNeed):
+    """One latent vector of ``rank`` numbers per token, in pages: a single float32 tensor
+    [pages, page, rank] per site instead of a key/value pair; ``window`` as for keys."""
+
+    rank: int
+    window: int = None
+
+    paged = True
+
+    def bytes_per_page(self, page_size, dtype):
+        return page_size * self.rank * 4
+
+    def allocate(self, layout, dtype, device):
+        return torch.full((layout.kernel_pages, layout.kernel_page, self.rank), 77.0,
+                          dtype=torch.float32, device=device)
+
+
+class ToyLatentMean(Part):
+    """c_t = W_c x_t is written to the token's place in the pages; y_t = W_o mean(c_s, s <= t),
+    read back through the block table.  Plain torch on the device: a toy, not a kernel."""
+
+    def __init__(self, hidden_size, rank):
+        super().__init__(hidden_size=hidden_size, rank=rank)
+        self.H, self.rank = hidden_size, rank
+
+    def declare(self):
+        return {"c_proj": ParamDecl((self.rank, self.H)), "o_proj": ParamDecl((self.H, self.rank))}
+
+    def bind(self, tensors, ctx):
+        self.w_c, self.w_o, self.dtype = tensors["c_proj"], tensors["o_proj"], ctx.dtype
+
+    def cache_need(self):
+        return LatentPages(self.rank)
+
+    def forward(self, x, site):
+        latents = site.cache.view(-1, self.rank)                   # every place of every page
+        pages, batch = site.pages, site.batch
+        c = ops.gemm(x, self.w_c, torch.float32)
+        latents[pages.slots.long()] = c                            # this step's tokens, at their places
+        means = torch.empty_like(c)
+        for r in range(batch.num_requests):
+            first, lo, hi = batch.first_position[r], batch.q_start[r], batch.q_start[r + 1]
+            upto = first + hi - lo
+            position = torch.arange(upto, device=x.device)
+            place = pages.block_table[r].long()[position // pages.page_size] * pages.page_size \
+                + position % pages.page_size
+            running = latents[place].cumsum(0) / (position + 1)[:, None]
+            means[lo:hi] = running[first:upto]
+        return ops.gemm(means.to(self.dtype), self.w_o, self.dtype)
+
+
+class TwoMixerBlock:
+    """h += latent_mean(norm(h)) + attention(norm(h)); h += feed_forward(norm(h)): two parts of
+    one layer keep a cache, each of its own kind."""
+
+    slots = {"latent": "mixer", "attention": "mixer", "feed_forward": "feed_forward",
+             "mixer_norm": "norm", "feed_forward_norm": "norm"}
+
+    def __init__(self, latent, attention, feed_forward, mixer_norm, feed_forward_norm):
+        self.latent, self.attention, self.feed_forward = latent, attention, feed_forward
+        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+
+    def forward(self, stream, site):
+        x = self.mixer_norm.add_norm(stream)
+        a = self.latent.forward(x, site.part(0))
+        b = ops.value(self.attention.forward(x, site.part(1)))
+        stream.pending = (a.float() + b.float()).to(a.dtype)
+        x = self.feed_forward_norm.add_norm(stream)
+        stream.pending = self.feed_forward.forward(x)
+
+
+TOY4 = {"architectures": ["Toy4ForCausalLM"], "hidden_size": 24, "vocab_size": 61, "rank": 6,
+        "eps": 1e-5, "heads": 2, "head_dim": 16}
+
+
+def toy4_spec(c):
+    norm = PartSpec("rms", {"size": c["hidden_size"], "eps": c["eps"]})
+    latent = PartSpec("toy_latent_mean", {"hidden_size": c["hidden_size"], "rank": c["rank"]})
+    attn = PartSpec("attention", {"hidden_size": c["hidden_size"], "num_heads": c["heads"],
+                                  "num_kv_heads": 1, "head_dim": c["head_dim"],
+                                  "position": PartSpec("rotary", {"rotary_dim": c["head_dim"], "theta": 100.0})})
+    ff = PartSpec("toy_scale", {"hidden_size": c["hidden_size"]})
+    plain_names = {"mixer_norm.weight": "l0.n1", "feed_forward_norm.weight": "l0.n2", "feed_forward.proj": "l0.ff",
+                   "mixer.c_proj": "l0.c", "mixer.o_proj": "l0.o"}
+    both_names = {"mixer_norm.weight": "l1.n1", "feed_forward_norm.weight": "l1.n2", "feed_forward.proj": "l1.ff",
+                  "latent.c_proj": "l1.c", "latent.o_proj": "l1.lo"}
+    both_names.update({f"attention.{k}_proj": f"l1.{k}" for k in "qkvo"})
+    layers = [prenorm_layer(latent, ff, norm, norm, plain_names),
+              LayerSpec("toy_two_mixers", {"latent": latent, "attention": attn, "feed_forward": ff,
+                                           "mixer_norm": norm, "feed_forward_norm": norm}, both_names)]
+    return ModelSpec(hidden_size=c["hidden_size"], vocab_size=c["vocab_size"], embedding_name="emb",
+                     layers=layers, run_order=[RunEntry(0), RunEntry(1), RunEntry(0)],
+                     final_norm=norm, final_norm_names={"weight": "final"}, head_name="head", init_std=0.3)
+
+
+def toy4_plain(c, w, ids):
+    w = {k: v.double() for k, v in w.items()}
+    T = len(ids)
+    h = w["emb"][torch.tensor(ids)]
+    steps = torch.arange(1, T + 1, dtype=F64)[:, None]
+    for layer in (0, 1, 0):
+        x = plain.rmsnorm(h, w[f"l{layer}.n1"], c["eps"])
+        if layer == 0:
+            a = ((x @ w["l0.c"].T).cumsum(0) / steps) @ w["l0.o"].T
+        else:
+            a = ((x @ w["l1.c"].T).cumsum(0) / steps) @ w["l1.lo"].T
+            q = plain.rope((x @ w["l1.q"].T).view(T, c["heads"], c["head_dim"]), range(T), 100.0)
+            k = plain.rope((x @ w["l1.k"].T).view(T, 1, c["head_dim"]), range(T), 100.0)
+            v = (x @ w["l1.v"].T).view(T, 1, c["head_dim"])
+            a = a + plain.attention(q, k, v, list(range(T))).reshape(T, -1) @ w["l1.o"].T
+        h = h + a
+        h = h + plain.rmsnorm(h, w[f"l{layer}.n2"], c["eps"]) @ w[f"l{layer}.ff"].T
+    return plain.rmsnorm(h, w["final"], c["eps"]) @ w["head"].T
+
+
+def test_toy_mixer_with_a_paged_cache_of_its_own_layout():
+    """A mixer whose cache is pages of ONE tensor per site (a latent vector per token), defined
+    here with its need, beside attention's key/value pages: in a layer of its own and as one of
+    two caching parts of one layer.  Registered, built, replayed in every family with so few
+    pages that they are used again (they start out holding 77), and driven through LLMEngine
+    with preemption, with no change to the package."""
+    from lucciola_amd.config.registry import BLOCKS
+    from lucciola_amd.engine.llm_engine import LLMEngine
+    from lucciola_amd.sampling.sampler import SamplingParams
+    MIXERS.register("toy_latent_mean", ToyLatentMean, replace=True)
+    FEED_FORWARDS.register("toy_scale", ToyScale, replace=True)
+    BLOCKS.register("toy_two_mixers", TwoMixerBlock, replace=True)
+    ARCHITECTURES.register("Toy4ForCausalLM", Architecture("Toy4ForCausalLM", read_config=dict,
+                                                           model_spec=toy4_spec), replace=True)
+    try:
+        spec = toy4_spec(TOY4)
+        weights = dict(random_tensors(declared_tensors(spec), 9, spec.init_std, torch.float32))
+        model = _build(spec, DictSource(weights), "float32", "cuda:0")
+        needs = model.site_needs()
+        assert needs[0] == LatentPages(6) == needs[2] and isinstance(needs[1], tuple)
+        assert needs[1][0] == LatentPages(6) and isinstance(needs[1][1], PagedKV)
+        prompts = prompts_for({"vocab_size": 61}, [25, 7, 40, 13, 31], 4)
+        refs = {n: toy4_plain(TOY4, weights, ids) for n, ids in prompts.items()}
+        for family in (traces.whole, traces.tail_decode, traces.chunked, traces.mixed):
+            steps = family(prompts)
+            blocks = traces.max_live_tokens(steps, 4) // 4
+            runner = ModelRunner(model, EngineConfig(dtype="float32", block_size=4, max_seqs=4, device="cuda:0",
+                                                     max_blocks=blocks))
+            cache = runner.cache
+            # two groups of pages: the three latent caches share one, attention has its own
+            assert [g.sites for g in cache.groups] == [[0, 1, 2], [1]]
+            assert cache.storage[0][0].shape == (blocks, 4, 6) and len(cache.storage[1]) == 2
+            assert cache.bytes_per_block(torch.float32) == 3 * 4 * 6 * 4 + 2 * 1 * 4 * 16 * 4
+            got = replay(runner, steps)
+            compare(got, TOY4, weights, prompts, 2e-5, refs)
+            assert all(g.pool.num_free() == blocks for g in cache.groups)
+        weights = dict(random_tensors(declared_tensors(spec), 9, 0.6, torch.float32))
+        model = _build(spec, DictSource(weights), "float32", "cuda:0")
+        asked = list(prompts_for({"vocab_size": 61}, [9, 14, 6, 11], 8).values())
+        for ahead in (False, True):
+            engine = LLMEngine(model, TOY4, EngineConfig(dtype="float32", block_size=4, max_blocks=18,
+                                                         max_seqs=4, max_tokens_per_step=12,
+                                                         device="cuda:0", run_ahead=ahead))
+            got = engine.generate(asked, SamplingParams(max_new_tokens=20))
+            assert engine.scheduler.num_preemptions > 0
+            for prompt, tokens in zip(asked, got):
+                ids = list(prompt)
+                for tok in tokens:
+                    assert tok == int(torch.argmax(toy4_plain(TOY4, weights, ids)[-1]))
+                    ids.append(tok)
+            engine.runner.cache.check()
+    finally:
+        MIXERS.unregister("toy_latent_mean")
+        FEED_FORWARDS.unregister("toy_scale")
+        BLOCKS.unregister("toy_two_mixers")
+        ARCHITECTURES.unregister("Toy4ForCausalLM")
+
+
+def test_kernel_signatures_can_be_registered_from_outside():
+    """A part that brings kernels of its own declares their entry points itself: here one that
+    the library already has is declared under the public door and launched through it."""
+    ops.register_signatures({"lc_attn_page_granule": ""})            # the same again: fine
+    with pytest.raises(ops.KernelError, match="already declared"):
+        ops.register_signatures({"lc_attn_page_granule": "i"})
+    with pytest.raises(ops.KernelError, match="unknown argument kinds"):
+        ops.register_signatures({"lc_new_kernel": "pq"})
+    with pytest.raises(ops.KernelError, match="lacks the entry point"):
+        ops.register_signatures({"lc_no_such_entry_point": "pi"})
+    assert "lc_no_such_entry_point" not in ops._SIGNATURES
+    ids = torch.zeros(3, dtype=torch.int32, device=DEV)
+    source = torch.tensor([2, -1, 0], dtype=torch.int32, device=DEV)
+    sampled = torch.tensor([5, 6, 7], dtype=torch.int32, device=DEV)
+    ops.call("lc_feed_tokens", ops.ptr(ids), ops.ptr(source), ops.ptr(sampled), 3, 3, ops.stream())
+    assert ids.tolist() == [7, 0, 5]

@@ -14,7 +14,7 @@ from lucciola_amd import models  # noqa: F401
 from lucciola_amd.config.registry import architecture_for
 from lucciola_amd.engine.loading import load_model
 from lucciola_amd.models.causal_lm import declared_tensors
-from lucciola_amd.weights.loader import (DictSource, FolderSource, ParamDecl, WeightsError,
+from lucciola_amd.weights.loader import (DictSource, FolderSource, ParamDecl, WeightsError, precision_notices,
                                          load_declared)
 from lucciola_amd.weights.random_init import random_tensors, write_model_folder
 from lucciola_amd.weights.safetensors_io import SafetensorsError, SafetensorsFile, write_safetensors
@@ -113,6 +113,16 @@ def test_kept_dtypes():
     with pytest.raises(WeightsError, match="wrong dtype"):
         load_declared(DictSource({"x": torch.zeros(2, dtype=torch.int64)}),
                       {"x": ParamDecl((2,))}, torch.device("cpu"))
+    # what keeping costs is said once per class of tensor, and only where it costs something
+    stored = {}
+    load_declared(source, declared, torch.device("cpu"), stored_dtypes=stored)
+    assert stored["m_f16"] == torch.float16 and stored["v_bf16"] == torch.bfloat16
+    lines = precision_notices(stored, declared, torch.bfloat16)
+    assert len(lines) == 2 and any("float32" in l and "m_f32" in l for l in lines)
+    assert any("float16" in l and "m_f16" in l and "general kernel" in l for l in lines)
+    assert precision_notices(stored, declared, torch.float32) == []
+    only_bf16 = {"m_bf16": torch.bfloat16, "v_bf16": torch.bfloat16}
+    assert precision_notices(only_bf16, declared, torch.bfloat16) == []
 
 
 @pytest.mark.parametrize("key", ["A", "B", "C", "D"])

@@ -45,19 +45,39 @@ def test_sampling_without_an_allocation():
         want = torch.full((R,), -1, dtype=torch.int32, device=dev)
         got = torch.full((R,), -2, dtype=torch.int32, device=dev)
         workspace = torch.empty(lib.lc_sample_workspace(R), dtype=torch.float32, device=dev)
-        torch.cuda.synchronize()
-        before = torch.cuda.memory_allocated(dev)
         rc = lib.lc_sample(_ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(want), _ptr(workspace),
                            R, V, stream)
         assert rc == 0, lib.lc_last_error()
+        # the first call on the device looks the array's address up; what is measured is the calls
+        # after it, by the runtime's own count of free device memory (torch's allocator would
+        # not see a hipMalloc inside the library)
         rc = lib.lc_sample_static(_ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(got), R, V, stream)
         assert rc == 0, lib.lc_last_error()
         torch.cuda.synchronize()
-        assert torch.cuda.memory_allocated(dev) == before
+        free_before = torch.cuda.mem_get_info(dev)[0]
+        for _ in range(4):
+            got.fill_(-2)
+            rc = lib.lc_sample_static(_ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(got), R, V, stream)
+            assert rc == 0, lib.lc_last_error()
+            torch.cuda.synchronize()
+            assert torch.cuda.mem_get_info(dev)[0] == free_before
         assert torch.equal(got, want), (R, V)
         assert int(got.min()) >= 0 and int(got.max()) < V
         if not sampled:
             assert torch.equal(got.long(), logits.argmax(dim=1))
+        else:
+            # against the definition, on the host in float64: greedy rows are the argmax, the others
+            # the first token whose cumulative probability exceeds the row's uniform number (a
+            # pick at a boundary that float32 sums could move may be its neighbour)
+            host, temps, us = logits.double().cpu(), temperature.cpu().tolist(), uniform.cpu().tolist()
+            for r in range(R):
+                if temps[r] <= 0:
+                    assert int(got[r]) == int(host[r].argmax())
+                    continue
+                cdf = torch.softmax(host[r] / temps[r], 0).cumsum(0)
+                pick = min(int(torch.searchsorted(cdf, torch.tensor(us[r], dtype=torch.float64), right=True)), V - 1)
+                if int(got[r]) != pick:
+                    assert abs(int(got[r]) - pick) == 1 and abs(float(cdf[min(int(got[r]), pick)]) - us[r]) < 1e-5, (r, pick)
     # more rows than the library's array holds: refused, nothing launched
     big = torch.zeros(1025, 8, device=dev)
     out = torch.full((1025,), -5, dtype=torch.int32, device=dev)
