@@ -224,10 +224,12 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
     // the numbers of the wave's first two pages: asked for now, they are back before the q/k preparation below is done
     const int pg0 = begin + wave;
     const int first_pages[2] = {pg0 < end ? table[pg0] : 0, pg0 + NW < end ? table[pg0 + NW] : 0};
+    // the page that takes the token's own k and v (asked for with the others, not when it is needed)
+    const bool owner = pro.enabled && pro.write_kv && begin <= last_page && last_page < end;
+    const int own_page = owner ? table[last_page] : 0;
 
     bf16x8 bq[1][D / 32];
     if (pro.enabled) {
-        const bool owner = pro.write_kv && begin <= last_page && last_page < end;
         const int ntask = G + (owner ? 2 : 0);            // the q heads, then k, then v
         const int half = pro.rot / 2;
         const float* cs = pro.rope ? pro.rope + (size_t)p * pro.rot : nullptr;
@@ -240,9 +242,25 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
                 if (!pro.shares) return *reinterpret_cast<const head_chunk*>(row + col);
                 const float* src = pro.shares + (size_t)t * pro.width + col;
                 floatx4 lo4 = {0.f, 0.f, 0.f, 0.f}, hi4 = {0.f, 0.f, 0.f, 0.f};
-                for (int sh = 0; sh < pro.num_shares; ++sh) {
-                    lo4 += *reinterpret_cast<const floatx4*>(src + (size_t)sh * pro.share_stride);
-                    hi4 += *reinterpret_cast<const floatx4*>(src + (size_t)sh * pro.share_stride + 4);
+                // the shares are asked for eight at a time and added in their order once all are
+                // back: one trip to memory for up to eight shares instead of one trip each (a
+                // share past the last is the last one again, loaded and not added)
+                constexpr int AT_ONCE = 8;
+                for (int s0 = 0; s0 < pro.num_shares; s0 += AT_ONCE) {
+                    floatx4 got_lo[AT_ONCE], got_hi[AT_ONCE];
+#pragma unroll
+                    for (int i = 0; i < AT_ONCE; ++i) {
+                        const float* at = src + (size_t)min(s0 + i, pro.num_shares - 1) * pro.share_stride;
+                        got_lo[i] = *reinterpret_cast<const floatx4*>(at);
+                        got_hi[i] = *reinterpret_cast<const floatx4*>(at + 4);
+                    }
+#pragma unroll
+                    for (int i = 0; i < AT_ONCE; ++i) {
+                        if (s0 + i < pro.num_shares) {
+                            lo4 += got_lo[i];
+                            hi4 += got_hi[i];
+                        }
+                    }
                 }
                 head_chunk out8;
 #pragma unroll
@@ -255,14 +273,14 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
             for (int task = threadIdx.x >> 4; task < ntask; task += 4 * NW) {
                 if (task == G + 1) {                      // v: copied, transposed into the page
                     const head_chunk raw = chunk_at((size_t)(nh + nkv + kvh) * D + 8 * j);
-                    bf16* col = v_cache + ((size_t)table[last_page] * nkv + kvh) * D * PAGE + (p % PAGE);
+                    bf16* col = v_cache + ((size_t)own_page * nkv + kvh) * D * PAGE + (p % PAGE);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) col[(size_t)(8 * j + e) * PAGE] = raw[e];
                     continue;
                 }
                 const bool is_k = task == G;
                 const size_t col = (size_t)(is_k ? nh + kvh : kvh * G + task) * D + 8 * j;
-                bf16* dst = is_k ? k_cache + (((size_t)table[last_page] * nkv + kvh) * PAGE + (p % PAGE)) * D
+                bf16* dst = is_k ? k_cache + (((size_t)own_page * nkv + kvh) * PAGE + (p % PAGE)) * D
                                  : sm_q + task * D;
                 const head_chunk done = head128_norm_rope(chunk_at(col), j,
                                                           is_k ? pro.k_w : pro.q_w, pro.eps, cs);
@@ -272,14 +290,14 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
             for (int task = wave; task < ntask; task += NW) {
                 if (task == G + 1) {                          // v: copied, transposed into the page
                     const bf16* x = row + (size_t)(nh + nkv + kvh) * D;
-                    bf16* col = v_cache + ((size_t)table[last_page] * nkv + kvh) * D * PAGE + (p % PAGE);
+                    bf16* col = v_cache + ((size_t)own_page * nkv + kvh) * D * PAGE + (p % PAGE);
                     for (int i = lane; i < D; i += 64) col[(size_t)i * PAGE] = x[i];
                     continue;
                 }
                 const bool is_k = task == G;
                 const bf16* x = row + (size_t)(is_k ? nh + kvh : kvh * G + task) * D;
                 const float* w = is_k ? pro.k_w : pro.q_w;
-                bf16* dst = is_k ? k_cache + (((size_t)table[last_page] * nkv + kvh) * PAGE + (p % PAGE)) * D
+                bf16* dst = is_k ? k_cache + (((size_t)own_page * nkv + kvh) * PAGE + (p % PAGE)) * D
                                  : sm_q + task * D;
                 float inv = 1.f;
                 if (w) {

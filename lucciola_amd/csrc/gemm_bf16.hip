@@ -610,16 +610,20 @@ constexpr int TL_K = 64;
 // reduction kernel to add in a fixed order: to part[blockIdx.y][M][N] (splitk_reduce_kernel),
 // or, if `compact`, tile by tile to part[blockIdx.y][tile - tile_base][BM][BN]
 // (tail_reduce_kernel).
-template <int BM, int BN, int TL_STAGES, int EPI, bool SPLIT, typename TO>
-__global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ x,
+template <int BM, int BN, int TL_STAGES, int EPI, bool SPLIT, typename TO, int WM = 2, int WN = 2>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16* __restrict__ x,
                                                          const bf16* __restrict__ w,
                                                          TO* __restrict__ out, float* __restrict__ part,
                                                          int M, int N, int K, int tiles_m, int tile_base,
-                                                         int tile_count, int compact) {
+                                                         int tile_count, int compact, int skew_step) {
+    // WM x WN waves, each owning (BM / WM) x (BN / WN) of the tile as TM x TN products of 32 x 32
     constexpr int S = TL_STAGES;
-    constexpr int TM = BM / 64, TN = BN / 64;
+    constexpr int NW = WM * WN;
+    constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN);
     constexpr int KS = TL_K / 16;                             // k-steps per block
-    constexpr int LPA = BM * 8 / 256, LPB = BN * 8 / 256, LP = LPA + LPB;   // load instructions per thread and stage
+    constexpr int LPA = BM * 8 / (64 * NW), LPB = BN * 8 / (64 * NW), LP = LPA + LPB;   // load instructions per thread and stage
+    static_assert(BM % (32 * WM) == 0 && BN % (32 * WN) == 0, "whole products per wave");
+    static_assert((BM * 8) % (64 * NW) == 0 && (BN * 8) % (64 * NW) == 0, "whole load instructions per wave");
     constexpr int NM = TM * TN, NR = TM + TN;                 // products and operand reads per k-step
     constexpr int A_STAGE = BM * TL_K * 2, B_STAGE = BN * TL_K * 2;          // bytes
     static_assert(S >= 2 && (S == 2 ? 2 : S - 1) * LP <= 63, "the load counter holds 63");
@@ -642,7 +646,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
+    const int wm = (wave / WN) * (BM / WM), wn = (wave % WN) * (BN / WN);
     const int lr = lane & 31, kg = lane >> 5;
     auto swz = [](int row) { return (row >> 1) & 7; };
 
@@ -650,27 +654,37 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
     const int kb0 = SPLIT ? (int)((long long)blockIdx.y * nk_all / gridDim.y) : 0;
     const int nk = (SPLIT ? (int)((long long)(blockIdx.y + 1) * nk_all / gridDim.y) : nk_all) - kb0;
 
-    // chunk p = (i * 4 + wave) * 64 + lane of a stage holds row p / 8, global chunk (p % 8) ^ swz(row)
+    // chunk p = (i * NW + wave) * 64 + lane of a stage holds row p / 8, global chunk (p % 8) ^ swz(row)
     const bf16* xg[LPA];
     const bf16* wg[LPB];
 #pragma unroll
     for (int i = 0; i < LPA; ++i) {
-        const int p = (i * 4 + wave) * 64 + lane, row = p >> 3, kc = (p & 7) ^ swz(row);
+        const int p = (i * NW + wave) * 64 + lane, row = p >> 3, kc = (p & 7) ^ swz(row);
         xg[i] = x + (size_t)min(m0 + row, M - 1) * K + (size_t)kb0 * TL_K + kc * 8;
     }
 #pragma unroll
     for (int i = 0; i < LPB; ++i) {
-        const int p = (i * 4 + wave) * 64 + lane, row = p >> 3, kc = (p & 7) ^ swz(row);
+        const int p = (i * NW + wave) * 64 + lane, row = p >> 3, kc = (p & 7) ^ swz(row);
         wg[i] = w + (size_t)min(n0 + row, N - 1) * K + (size_t)kb0 * TL_K + kc * 8;
     }
+    // With a single row of tiles (M <= BM: decode steps of 17 to 64 tokens) every workgroup
+    // streams rows of w that nobody else reads, all rows 2 K bytes apart, and all workgroups
+    // would walk k in step: at any moment the whole GPU would ask for the same few columns, which
+    // lie in the same memory channels (measured with rows padded by 128 bytes instead: 64 x 24576
+    // x 4096 takes 37.6 instead of 46.9 us).  So each workgroup starts at a k-block of its own
+    // (tile number times skew_step, modulo the number of k-blocks) and wraps around: 37.2 us.  (With several rows of tiles the workgroups that share a tile of w
+    // should read it at the same time, and do.)
+    const int skew = (!SPLIT && tiles_m == 1 && skew_step) ? (int)(((unsigned)id * (unsigned)skew_step) % (unsigned)nk) : 0;
     // load instruction idx (x first, then w) of block kb into a stage
     auto issue_one = [&](int idx, int kb, int stage) {
+        kb += skew;
+        kb -= kb >= nk ? nk : 0;
         if (idx < LPA)
             __builtin_amdgcn_global_load_lds((glb_ptr_t)(xg[idx] + kb * TL_K),
-                (lds_ptr_t)(lds + stage * A_STAGE + (idx * 4 + wave) * 1024), 16, 0, 0);
+                (lds_ptr_t)(lds + stage * A_STAGE + (idx * NW + wave) * 1024), 16, 0, 0);
         else
             __builtin_amdgcn_global_load_lds((glb_ptr_t)(wg[idx - LPA] + kb * TL_K),
-                (lds_ptr_t)(lds + S * A_STAGE + stage * B_STAGE + ((idx - LPA) * 4 + wave) * 1024), 16, 0, 0);
+                (lds_ptr_t)(lds + S * A_STAGE + stage * B_STAGE + ((idx - LPA) * NW + wave) * 1024), 16, 0, 0);
     };
     // With two stages, a block's loads are issued a block early: in the last k-step of block it,
     // once every wave has read the last of the stage, block it + 2 goes into it, behind block
@@ -937,16 +951,16 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restric
 // The tile shapes of the tiled kernel.  TILE_AUTO picks by size; the others are forced through
 // lc_gemm_bf16_force_tile (tests and tuning).
 enum : int { TILE_AUTO = -1, TILE_64x128 = 0, TILE_128x128 = 1, TILE_256x128 = 2, TILE_256x192 = 3, TILE_256x256 = 4,
-              TILE_192x128 = 5, TILE_192x256 = 6, TILE_64x64 = 7, TILE_COUNT = 8 };
+              TILE_192x128 = 5, TILE_192x256 = 6, TILE_64x64 = 7, TILE_64x96 = 8, TILE_COUNT = 9 };
 static thread_local int g_force_tile = TILE_AUTO;   // the switches are per thread: a test that flips one
                                                     // never changes what an engine's thread launches
 #define kCUs (::lc::device_cus())   // the GPU's compute units: they steer the tile plans only
 
 static int tile_bm(int t) {
-    return (t == TILE_64x128 || t == TILE_64x64) ? 64 : t == TILE_128x128 ? 128 : (t == TILE_192x128 || t == TILE_192x256) ? 192 : 256;
+    return (t == TILE_64x128 || t == TILE_64x64 || t == TILE_64x96) ? 64 : t == TILE_128x128 ? 128 : (t == TILE_192x128 || t == TILE_192x256) ? 192 : 256;
 }
 static int tile_bn(int t) {
-    return (t == TILE_256x256 || t == TILE_192x256) ? 256 : t == TILE_256x192 ? 192 : t == TILE_64x64 ? 64 : 128;
+    return (t == TILE_256x256 || t == TILE_192x256) ? 256 : t == TILE_256x192 ? 192 : t == TILE_64x64 ? 64 : t == TILE_64x96 ? 96 : 128;
 }
 static long long tile_count(int t, int M, int N) {
     return (long long)((M + tile_bm(t) - 1) / tile_bm(t)) * ((N + tile_bn(t) - 1) / tile_bn(t));
@@ -985,8 +999,14 @@ static bool whole_k_64x64(int M, int N, int K) {
     const long long tiles64 = tile_count(TILE_64x64, M, N);
     return (tiles64 >= kCUs && tiles64 <= 3 * kCUs) || (K <= 2048 && tiles64 >= 48);
 }
+// by how many k-blocks a workgroup's start moves per tile where the tiles form a single row (see the
+// kernel); measured at 64 x 24576 x 4096 in tiles of 64 x 96: 0: 46.9 us, 1: 41.2, 3: 58.8, 5 to 31
+// (odd): 37.0 to 38.2
+static thread_local int g_skew = 17;
+static thread_local int g_force_shares = 0;   // > 0: the small tiles are cut along K this many ways (tests, tuning)
 static int shares_for(int t, int M, int N, int K, bool partials_wanted = false) {
     if (t != TILE_64x128 && t != TILE_128x128 && t != TILE_64x64) return 1;
+    if (g_force_shares > 0) return g_force_shares <= K / TL_K ? g_force_shares : K / TL_K;
     if (t == TILE_64x64 && g_force_tile == TILE_AUTO && !partials_wanted && whole_k_64x64(M, N, K)) return 1;
     const long long tiles = tile_count(t, M, N);
     if (tiles >= 400) return 1;
@@ -1013,10 +1033,17 @@ static int pick_tile(int M, int N, int K, bool partials_wanted = false) {
         // tiles of 64 x 64 cut along K where there are few of them, and for shares that are
         // handed on; else tiles of 64 x 128, cut where they are few.
         if (partials_wanted) return g_small_partials ? TILE_64x64 : TILE_64x128;
-        if (whole_k_64x64(M, N, K) || tile_count(TILE_64x64, M, N) <= 128) return TILE_64x64;
+        // Where tiles of 64 x 64 would go through the CUs in one and a half rounds to two (every
+        // CU's way from L2 carries the tile's rows of x and of w, and the CUs with two tiles set
+        // the time), tiles of 64 x 96 that make one round carry less per CU: one workgroup of two
+        // waves a CU, with a deep ring of stages in place of a second workgroup (64 x 24576 x
+        // 4096 with SwiGLU: 384 tiles of 64 x 64, or 256 of 64 x 96).
+        const long long tiles64 = tile_count(TILE_64x64, M, N), tiles96 = tile_count(TILE_64x96, M, N);
+        if (tiles64 > kCUs && tiles64 <= 2 * kCUs && tiles96 <= kCUs && K >= 1024) return TILE_64x96;
+        if (whole_k_64x64(M, N, K) || tiles64 <= 128) return TILE_64x64;
         return TILE_64x128;
     }
-    const double rate[TILE_COUNT] = {0.70, 0.82, 0.90, 0.94, 1.0, 0.87, 0.94, 0.5};
+    const double rate[TILE_COUNT] = {0.70, 0.82, 0.90, 0.94, 1.0, 0.87, 0.94, 0.5, 0.5};
     int best = -1;
     double best_cost = 0.0;
     for (int t = M <= 128 ? TILE_64x128 : TILE_128x128; t < TILE_64x64; ++t) {
@@ -1199,26 +1226,30 @@ static void launch_skinny_any(const bf16* x, const bf16* w, TO* out, int M, int 
     }
 }
 
-template <int BM, int BN, int STAGES, int EPI, typename TO>
+template <int BM, int BN, int STAGES, int EPI, typename TO, int WM = 2, int WN = 2>
 static int launch_tiled(const bf16* x, const bf16* w, TO* out, float* workspace, int M, int N, int K,
                         int shares, TailPlan tail, hipStream_t s) {
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const int tiles = tiles_m * tiles_n;
     if (shares == 1 && tail.shares <= 1) {
-        gemm_tiled_kernel<BM, BN, STAGES, EPI, false, TO><<<tiles, 256, 0, s>>>(
-            x, w, out, nullptr, M, N, K, tiles_m, 0, tiles, 0);
+        gemm_tiled_kernel<BM, BN, STAGES, EPI, false, TO, WM, WN><<<tiles, 64 * WM * WN, 0, s>>>(
+            x, w, out, nullptr, M, N, K, tiles_m, 0, tiles, 0, g_skew);
         LC_LAUNCH_CHECK("gemm_tiled");
         return 0;
     }
+    if constexpr (WM != 2 || WN != 2) {
+        LC_CHECK(false, "gemm_bf16: the tile %dx%d is not cut along K", BM, BN);
+        return 0;
+    } else {
     LC_CHECK(workspace, "gemm_bf16: M=%d N=%d K=%d needs a workspace", M, N, K);
     if constexpr (BM >= 192) {
         LC_CHECK(shares == 1 && tail.rest > 0 && tail.rest < tiles, "gemm_bf16: bad tail for tile %dx%d", BM, BN);
         const int whole = tiles - tail.rest;
         gemm_tiled_kernel<BM, BN, STAGES, EPI, false, TO><<<whole, 256, 0, s>>>(
-            x, w, out, nullptr, M, N, K, tiles_m, 0, whole, 0);
+            x, w, out, nullptr, M, N, K, tiles_m, 0, whole, 0, g_skew);
         LC_LAUNCH_CHECK("gemm_tiled");
         gemm_tiled_kernel<BM, BN, STAGES, 0, true, TO><<<dim3(tail.rest, tail.shares), 256, 0, s>>>(
-            x, w, out, workspace, M, N, K, tiles_m, whole, tail.rest, 1);
+            x, w, out, workspace, M, N, K, tiles_m, whole, tail.rest, 1, g_skew);
         LC_LAUNCH_CHECK("gemm_tiled");
         tail_reduce_kernel<EPI, TO><<<dim3(tail.rest, (BM * BN + 2047) / 2048), 256, 0, s>>>(
             workspace, out, M, N, BM, BN, tiles_m, whole, tail.rest, tail.shares);
@@ -1227,12 +1258,13 @@ static int launch_tiled(const bf16* x, const bf16* w, TO* out, float* workspace,
     } else {
         LC_CHECK(tail.shares <= 1, "gemm_bf16: tile %dx%d has no tail", BM, BN);
         gemm_tiled_kernel<BM, BN, STAGES, 0, true, TO><<<dim3(tiles, shares), 256, 0, s>>>(
-            x, w, out, workspace, M, N, K, tiles_m, 0, tiles, 0);
+            x, w, out, workspace, M, N, K, tiles_m, 0, tiles, 0, g_skew);
         LC_LAUNCH_CHECK("gemm_tiled");
         const size_t work = EPI ? (size_t)M * N / 2 : (size_t)M * N;
         splitk_reduce_kernel<EPI, TO><<<(int)((work + 255) / 256), 256, 0, s>>>(workspace, out, M, N, shares);
         LC_LAUNCH_CHECK("splitk_reduce");
         return 0;
+    }
     }
 }
 
@@ -1255,6 +1287,7 @@ static int launch_bf16(const bf16* x, const bf16* w, TO* out, float* workspace, 
     case TILE_192x128: return launch_tiled<192, 128, 3, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     case TILE_192x256: return launch_tiled<192, 256, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     case TILE_64x64:   return launch_tiled<64, 64, 3, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
+    case TILE_64x96:   return launch_tiled<64, 96, 6, EPI, TO, 2, 1>(x, w, out, workspace, M, N, K, shares, tail, s);
     default:           return launch_tiled<256, 256, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     }
 }
@@ -1345,6 +1378,22 @@ LC_API int lc_gemm_bf16_runs_ring_ok() { return runs_ring_state(); }
 
 LC_API int lc_gemm_bf16_even_rows(int on) {
     g_even_rows = on ? 1 : 0;
+    return 0;
+}
+
+// The step of the k-block skew of products with a single row of tiles (0: none; 17 by default).
+// For tests and tuning.
+LC_API int lc_gemm_bf16_skew(int step) {
+    LC_CHECK(step >= 0, "gemm_bf16: bad skew %d", step);
+    g_skew = step;
+    return 0;
+}
+
+// > 0: products that go through the small tiles (64 x 64, 64 x 128, 128 x 128) are cut along K
+// this many ways, whatever their size; 0: by size again.  For tests and tuning.
+LC_API int lc_gemm_bf16_force_shares(int shares) {
+    LC_CHECK(shares >= 0 && shares <= 64, "gemm_bf16: %d shares (0 to 64)", shares);
+    g_force_shares = shares;
     return 0;
 }
 
@@ -1440,15 +1489,15 @@ LC_API int lc_gemm_bf16_partials(const void* x, const void* w, float* partials, 
     if (pick_tile(M, N, K, true) == TILE_64x64) {
         const int tiles_m = (M + 63) / 64, tiles = tiles_m * ((N + 63) / 64);
         gemm_tiled_kernel<64, 64, 3, 0, true, float><<<dim3(tiles, shares), 256, 0, stream>>>(
-            xb, wb, nullptr, partials, M, N, K, tiles_m, 0, tiles, 0);
+            xb, wb, nullptr, partials, M, N, K, tiles_m, 0, tiles, 0, g_skew);
     } else if (pick_tile(M, N, K, true) == TILE_64x128) {
         const int tiles_m = (M + 63) / 64, tiles = tiles_m * ((N + 127) / 128);
         gemm_tiled_kernel<64, 128, 3, 0, true, float><<<dim3(tiles, shares), 256, 0, stream>>>(
-            xb, wb, nullptr, partials, M, N, K, tiles_m, 0, tiles, 0);
+            xb, wb, nullptr, partials, M, N, K, tiles_m, 0, tiles, 0, g_skew);
     } else {
         const int tiles_m = (M + 127) / 128, tiles = tiles_m * ((N + 127) / 128);
         gemm_tiled_kernel<128, 128, 2, 0, true, float><<<dim3(tiles, shares), 256, 0, stream>>>(
-            xb, wb, nullptr, partials, M, N, K, tiles_m, 0, tiles, 0);
+            xb, wb, nullptr, partials, M, N, K, tiles_m, 0, tiles, 0, g_skew);
     }
     LC_LAUNCH_CHECK("gemm_tiled");
     return 0;

@@ -35,6 +35,8 @@ _SIGNATURES = {
     "lc_gemm_bf16_even_rows": "i",
     "lc_gemm_bf16_runs": "i",
     "lc_gemm_bf16_small_partials": "i",
+    "lc_gemm_bf16_force_shares": "i",
+    "lc_gemm_bf16_skew": "i",
     "lc_gemm_bf16_residual_pieces": "iii",
     "lc_gemm_bf16_piece_stride": "i",
     "lc_gemm_bf16_shares": "iii",
@@ -436,7 +438,7 @@ def _gemm_workspace(M: int, N: int, K: int, device) -> Optional[torch.Tensor]:
 
 def force_gemm_tile(tile: int) -> None:
     """Make the tiled bfloat16 product use one tile shape for every size (0: 64x128, 1: 128x128,
-    2: 256x128, 3: 256x192, 4: 256x256, 5: 192x128, 6: 192x256, 7: 64x64; -1: choose by size again).  For tests and tuning."""
+    2: 256x128, 3: 256x192, 4: 256x256, 5: 192x128, 6: 192x256, 7: 64x64, 8: 64x96; -1: choose by size again).  For tests and tuning."""
     _call("lc_gemm_bf16_force_tile", _c_int(tile))
 
 
