@@ -951,16 +951,16 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restric
 // The tile shapes of the tiled kernel.  TILE_AUTO picks by size; the others are forced through
 // lc_gemm_bf16_force_tile (tests and tuning).
 enum : int { TILE_AUTO = -1, TILE_64x128 = 0, TILE_128x128 = 1, TILE_256x128 = 2, TILE_256x192 = 3, TILE_256x256 = 4,
-              TILE_192x128 = 5, TILE_192x256 = 6, TILE_64x64 = 7, TILE_64x96 = 8, TILE_COUNT = 9 };
+              TILE_192x128 = 5, TILE_192x256 = 6, TILE_64x64 = 7, TILE_64x96 = 8, TILE_192x320 = 9, TILE_COUNT = 10 };
 static thread_local int g_force_tile = TILE_AUTO;   // the switches are per thread: a test that flips one
                                                     // never changes what an engine's thread launches
 #define kCUs (::lc::device_cus())   // the GPU's compute units: they steer the tile plans only
 
 static int tile_bm(int t) {
-    return (t == TILE_64x128 || t == TILE_64x64 || t == TILE_64x96) ? 64 : t == TILE_128x128 ? 128 : (t == TILE_192x128 || t == TILE_192x256) ? 192 : 256;
+    return (t == TILE_64x128 || t == TILE_64x64 || t == TILE_64x96) ? 64 : t == TILE_128x128 ? 128 : (t == TILE_192x128 || t == TILE_192x256 || t == TILE_192x320) ? 192 : 256;
 }
 static int tile_bn(int t) {
-    return (t == TILE_256x256 || t == TILE_192x256) ? 256 : t == TILE_256x192 ? 192 : t == TILE_64x64 ? 64 : t == TILE_64x96 ? 96 : 128;
+    return (t == TILE_256x256 || t == TILE_192x256) ? 256 : t == TILE_192x320 ? 320 : t == TILE_256x192 ? 192 : t == TILE_64x64 ? 64 : t == TILE_64x96 ? 96 : 128;
 }
 static long long tile_count(int t, int M, int N) {
     return (long long)((M + tile_bm(t) - 1) / tile_bm(t)) * ((N + tile_bn(t) - 1) / tile_bn(t));
@@ -1043,10 +1043,13 @@ static int pick_tile(int M, int N, int K, bool partials_wanted = false) {
         if (whole_k_64x64(M, N, K) || tiles64 <= 128) return TILE_64x64;
         return TILE_64x128;
     }
-    const double rate[TILE_COUNT] = {0.70, 0.82, 0.90, 0.94, 1.0, 0.87, 0.94, 0.5, 0.5};
+    const double rate[TILE_COUNT] = {0.70, 0.82, 0.90, 0.94, 1.0, 0.87, 0.94, 0.5, 0.5, 0.97};
     int best = -1;
     double best_cost = 0.0;
-    for (int t = M <= 128 ? TILE_64x128 : TILE_128x128; t < TILE_64x64; ++t) {
+    const int candidates[] = {TILE_64x128, TILE_128x128, TILE_256x128, TILE_256x192, TILE_256x256, TILE_192x128,
+                              TILE_192x256, TILE_192x320};
+    for (const int t : candidates) {
+        if (t == TILE_64x128 && M > 128) continue;
         const long long tiles = tile_count(t, M, N);
         const double area = (double)tile_bm(t) * tile_bn(t);
         const double work_us = area * K * 2.0 / (4.63e6 * rate[t]);
@@ -1288,6 +1291,7 @@ static int launch_bf16(const bf16* x, const bf16* w, TO* out, float* workspace, 
     case TILE_192x256: return launch_tiled<192, 256, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     case TILE_64x64:   return launch_tiled<64, 64, 3, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     case TILE_64x96:   return launch_tiled<64, 96, 6, EPI, TO, 2, 1>(x, w, out, workspace, M, N, K, shares, tail, s);
+    case TILE_192x320: return launch_tiled<192, 320, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     default:           return launch_tiled<256, 256, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     }
 }

@@ -282,7 +282,7 @@ def test_gemm_bf16_matrix_cores(out_dtype, M, N, K):
     close(got, want, out_dtype, scale=K ** 0.5)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9])
 @pytest.mark.parametrize("M,N,K", [(1, 16, 128), (70, 130, 128), (257, 300, 256), (300, 1000, 640),
                                    (513, 257, 384), (64, 128, 1024), (1000, 520, 2048), (100, 400, 128)])
 def test_gemm_bf16_every_tile_shape(tile, M, N, K):
