@@ -14,7 +14,7 @@ import subprocess
 import sys
 import tempfile
 import time
-from concurrent.futures import ThreadPoolExecutor, as_completed
+from concurrent.futures import FIRST_COMPLETED, ThreadPoolExecutor, wait
 from typing import List, Optional
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -114,9 +114,15 @@ def build(force: bool = True, jobs: Optional[int] = None) -> str:
     objs = []
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         futures = {pool.submit(compile_one, s): s for s in srcs}
-        for fut in as_completed(futures):
-            objs.append(fut.result())
-            _log(f"  {futures[fut]} done ({time.time() - t0:.0f} s)")
+        pending = set(futures)
+        while pending:
+            # a line every ten seconds at the least: the largest file takes half a minute
+            done, pending = wait(pending, timeout=10, return_when=FIRST_COMPLETED)
+            for fut in done:
+                objs.append(fut.result())
+                _log(f"  {futures[fut]} done ({time.time() - t0:.0f} s)")
+            if not done:
+                _log(f"  still compiling {', '.join(sorted(futures[f] for f in pending))} ({time.time() - t0:.0f} s)")
     tmp_lib = lib + f".tmp{os.getpid()}"
     cmd = [hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-fno-gpu-rdc", "-o", tmp_lib] + sorted(objs)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
