@@ -119,6 +119,9 @@ def library():
         lib.lc_attention_generic_workspace.argtypes = [ctypes.c_int] * 5
         for name, sig in _SIGNATURES.items():
             _declare(lib, name, sig)
+        if lib.lc_attn_page_granule() != ATTENTION_PAGE_GRANULE:
+            raise KernelError(f"the attention kernels of {path} are built for pages of "
+                              f"{lib.lc_attn_page_granule()} tokens, this module for {ATTENTION_PAGE_GRANULE}")
         _lib = lib
     return _lib
 
@@ -575,10 +578,15 @@ def plan_attention(layout):
             {"num_decode": int(decode.size), "all_decode": int(decode.size) == R})
 
 
+# Tokens of a cache page as the matrix-core attention kernels index it: a page of a multiple of
+# it reaches them as so many pages of this size.  The kernels say the same number
+# (lc_attn_page_granule), which is checked when the library is loaded; a model can be described
+# and its cache laid out without loading it.
+ATTENTION_PAGE_GRANULE = 16
+
+
 def attention_page_granule() -> int:
-    """Tokens of a cache page as the matrix-core attention kernels index it: a page of a
-    multiple of it reaches them as so many pages of this size."""
-    return int(library().lc_attn_page_granule())
+    return ATTENTION_PAGE_GRANULE
 
 
 def attention_batch(batch, pages, plan=None) -> AttentionBatch:

@@ -123,16 +123,12 @@ def attention_takes_shares(*args, **kwargs):
     return False
 
 
-def attention_page_granule():
-    return 16
-
-
 def feed_tokens(ids, source, sampled):
     take = source >= 0
     ids[take] = sampled[source[take].long()]
 
 
-ALL = ("feed_tokens", "attention_takes_shares", "attention_page_granule", "embedding", "rmsnorm", "rmsnorm_act", "gemm", "qk_norm_rope_write", "attention",
+ALL = ("feed_tokens", "attention_takes_shares", "embedding", "rmsnorm", "rmsnorm_act", "gemm", "qk_norm_rope_write", "attention",
        "swiglu", "sample")
 
 

@@ -274,3 +274,16 @@ def test_sharded_checkpoint(tmp_path):
     with pytest.raises(WeightsError) as info:
         FolderSource(folder)
     assert info.value.missing == [names[0]]
+
+
+def test_a_model_folder_is_written_without_the_kernel_library(tmp_path, monkeypatch):
+    """Describing a model, declaring its tensors and writing random weights is host work: none
+    of it may load (or build) the kernel library."""
+    from lucciola_amd.kernels import ops
+
+    def refuse(*args, **kwargs):
+        raise AssertionError("the kernel library was asked for")
+    monkeypatch.setattr(ops, "library", refuse)
+    cfg, _, seed = configs.ALL["C"]
+    folder = write_model_folder(str(tmp_path / "m"), cfg, seed)
+    assert sorted(os.listdir(folder)) == ["config.json", "model.safetensors"]
