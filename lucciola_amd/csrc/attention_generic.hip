@@ -84,8 +84,9 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
     int nh, int nkv, int d, int d_pow2, int page_size, float scale, int window,
     float* __restrict__ part, int part_spans) {
     __shared__ __align__(16) float qs[GH][256];
-    __shared__ float ps[GH][AG_THREADS];
+    __shared__ __align__(16) float ps[GH][AG_THREADS];
     __shared__ float scratch[GH][AG_WAVES];
+    __shared__ int pages[AG_THREADS + 1];      // the chunk's pages, looked up once a chunk
 
     const int t = blockIdx.x, tid = threadIdx.x;
     const int group = nh / nkv, batches = (group + GH - 1) / GH;
@@ -129,8 +130,13 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
             const int count = min(AG_THREADS, hi - c0 + 1);
             const bool valid = tid < count;
             float sc[GH];
+            // the numbers of the chunk's pages go to LDS first: one trip to the block table a
+            // chunk instead of one before every key's and value's own load
+            const int page0 = c0 / page_size, page_n = (c0 + count - 1) / page_size - page0 + 1;
+            for (int i = tid; i < page_n; i += AG_THREADS) pages[i] = table[page0 + i];
+            __syncthreads();
             if (vec) {
-                const int piece = tid & 3, quarter = d >> 2;
+                const int piece = tid & 3;
                 for (int pass = 0; pass < 4; ++pass) {
                     const int kc = pass * (AG_THREADS / 4) + (tid >> 2);
                     float dot[GH];
@@ -138,16 +144,25 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
                     for (int hh = 0; hh < GH; ++hh) dot[hh] = 0.f;
                     if (kc < count) {
                         const int jk = c0 + kc;
-                        const long long head = (long long)table[jk / page_size] * nkv + kvh;
-                        const T* krow = k_cache + (head * page_size + (jk % page_size)) * d + piece * quarter;
-                        for (int i = 0; i < quarter; i += 4) {
-                            float k4[4];
-                            load4(k4, krow + i);
+                        const long long head = (long long)pages[jk / page_size - page0] * nkv + kvh;
+                        // the four lanes of a key take its pieces of four entries in turn (lane
+                        // `piece` the pieces piece, piece + 4, ...): one load instruction then reads
+                        // 64 bytes in a row of each of a wave's 16 keys; four loads are asked for
+                        // before the first is used
+                        const T* krow = k_cache + (head * page_size + (jk % page_size)) * d + piece * 4;
+                        for (int i0 = 0; i0 < d; i0 += 64) {
+                            float k4[4][4];
 #pragma unroll
-                            for (int hh = 0; hh < GH; ++hh)
+                            for (int u = 0; u < 4; ++u)
+                                if (i0 + 16 * u < d) load4(k4[u], krow + i0 + 16 * u);
 #pragma unroll
-                                for (int e = 0; e < 4; ++e)
-                                    dot[hh] = fmaf(qs[hh][piece * quarter + i + e], k4[e], dot[hh]);
+                            for (int u = 0; u < 4; ++u)
+                                if (i0 + 16 * u < d)
+#pragma unroll
+                                    for (int hh = 0; hh < GH; ++hh)
+#pragma unroll
+                                        for (int e = 0; e < 4; ++e)
+                                            dot[hh] = fmaf(qs[hh][piece * 4 + i0 + 16 * u + e], k4[u][e], dot[hh]);
                         }
                     }
 #pragma unroll
@@ -166,7 +181,7 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
                 for (int hh = 0; hh < GH; ++hh) sc[hh] = 0.f;
                 if (valid) {
                     const int j = c0 + tid;
-                    const long long head = (long long)table[j / page_size] * nkv + kvh;
+                    const long long head = (long long)pages[j / page_size - page0] * nkv + kvh;
                     const T* krow = k_cache + (head * page_size + (j % page_size)) * d;
                     for (int i = 0; i < d; ++i) {
                         const float kv = to_f32(krow[i]);
@@ -201,24 +216,39 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
                 if (vec) {
                     // runs of four keys that start at a multiple of four lie in one page; a run
                     // may reach over the chunk's ends, where the keys count nothing
+                    // (four runs are asked for before the first is used; they are taken in in
+                    // their order)
                     const int last_run = (c0 + count - 1) >> 2;
-                    for (int run = (c0 >> 2) + g; run <= last_run; run += groups) {
-                        const int j4 = run * 4;
-                        const long long head = (long long)table[j4 / page_size] * nkv + kvh;
-                        float v4[4];
-                        load4(v4, v_cache + head * d * page_size + (long long)di * page_size + (j4 % page_size));
+                    for (int run0 = (c0 >> 2) + g; run0 <= last_run; run0 += 4 * groups) {
+                        float v4[4][4];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const int jj = j4 + e - c0;
-                            if (jj >= 0 && jj < count)
+                        for (int u = 0; u < 4; ++u) {
+                            const int j4 = (run0 + u * groups) * 4;
+                            if (run0 + u * groups <= last_run) {
+                                // a run may begin before the chunk's first key, in the page before its first
+                                const int pg = j4 >= c0 ? pages[j4 / page_size - page0] : table[j4 / page_size];
+                                const long long head = (long long)pg * nkv + kvh;
+                                load4(v4[u], v_cache + head * d * page_size + (long long)di * page_size + (j4 % page_size));
+                            }
+                        }
 #pragma unroll
-                                for (int hh = 0; hh < GH; ++hh) acc[hh] = fmaf(ps[hh][jj], v4[e], acc[hh]);
+                        for (int u = 0; u < 4; ++u) {
+                            const int j4 = (run0 + u * groups) * 4;
+                            if (run0 + u * groups <= last_run) {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) {
+                                    const int jj = j4 + e - c0;
+                                    if (jj >= 0 && jj < count)
+#pragma unroll
+                                        for (int hh = 0; hh < GH; ++hh) acc[hh] = fmaf(ps[hh][jj], v4[u][e], acc[hh]);
+                                }
+                            }
                         }
                     }
                 } else {
                     for (int jj = g; jj < count; jj += groups) {
                         const int j = c0 + jj;
-                        const long long head = (long long)table[j / page_size] * nkv + kvh;
+                        const long long head = (long long)pages[j / page_size - page0] * nkv + kvh;
                         const float v = to_f32(v_cache[head * d * page_size + (long long)di * page_size + (j % page_size)]);
 #pragma unroll
                         for (int hh = 0; hh < GH; ++hh) acc[hh] = fmaf(ps[hh][jj], v, acc[hh]);
