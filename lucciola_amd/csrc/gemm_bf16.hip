@@ -951,16 +951,17 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restric
 // The tile shapes of the tiled kernel.  TILE_AUTO picks by size; the others are forced through
 // lc_gemm_bf16_force_tile (tests and tuning).
 enum : int { TILE_AUTO = -1, TILE_64x128 = 0, TILE_128x128 = 1, TILE_256x128 = 2, TILE_256x192 = 3, TILE_256x256 = 4,
-              TILE_192x128 = 5, TILE_192x256 = 6, TILE_64x64 = 7, TILE_64x96 = 8, TILE_192x320 = 9, TILE_COUNT = 10 };
+              TILE_192x128 = 5, TILE_192x256 = 6, TILE_64x64 = 7, TILE_64x96 = 8, TILE_192x320 = 9, TILE_64x224 = 10,
+              TILE_64x128_ONE = 11, TILE_64x160 = 12, TILE_COUNT = 13 };
 static thread_local int g_force_tile = TILE_AUTO;   // the switches are per thread: a test that flips one
                                                     // never changes what an engine's thread launches
 #define kCUs (::lc::device_cus())   // the GPU's compute units: they steer the tile plans only
 
 static int tile_bm(int t) {
-    return (t == TILE_64x128 || t == TILE_64x64 || t == TILE_64x96) ? 64 : t == TILE_128x128 ? 128 : (t == TILE_192x128 || t == TILE_192x256 || t == TILE_192x320) ? 192 : 256;
+    return (t == TILE_64x128 || t == TILE_64x64 || t == TILE_64x96 || t == TILE_64x224 || t == TILE_64x128_ONE || t == TILE_64x160) ? 64 : t == TILE_128x128 ? 128 : (t == TILE_192x128 || t == TILE_192x256 || t == TILE_192x320) ? 192 : 256;
 }
 static int tile_bn(int t) {
-    return (t == TILE_256x256 || t == TILE_192x256) ? 256 : t == TILE_192x320 ? 320 : t == TILE_256x192 ? 192 : t == TILE_64x64 ? 64 : t == TILE_64x96 ? 96 : 128;
+    return (t == TILE_256x256 || t == TILE_192x256) ? 256 : t == TILE_192x320 ? 320 : t == TILE_256x192 ? 192 : t == TILE_64x64 ? 64 : t == TILE_64x96 ? 96 : t == TILE_64x224 ? 224 : t == TILE_64x160 ? 160 : 128;
 }
 static long long tile_count(int t, int M, int N) {
     return (long long)((M + tile_bm(t) - 1) / tile_bm(t)) * ((N + tile_bn(t) - 1) / tile_bn(t));
@@ -1033,17 +1034,22 @@ static int pick_tile(int M, int N, int K, bool partials_wanted = false) {
         // tiles of 64 x 64 cut along K where there are few of them, and for shares that are
         // handed on; else tiles of 64 x 128, cut where they are few.
         if (partials_wanted) return g_small_partials ? TILE_64x64 : TILE_64x128;
-        // Where tiles of 64 x 64 would go through the CUs in one and a half rounds to two (every
-        // CU's way from L2 carries the tile's rows of x and of w, and the CUs with two tiles set
-        // the time), tiles of 64 x 96 that make one round carry less per CU: one workgroup of two
-        // waves a CU, with a deep ring of stages in place of a second workgroup (64 x 24576 x
-        // 4096 with SwiGLU: 384 tiles of 64 x 64, or 256 of 64 x 96).
-        const long long tiles64 = tile_count(TILE_64x64, M, N), tiles96 = tile_count(TILE_64x96, M, N);
-        if (tiles64 > kCUs && tiles64 <= 2 * kCUs && tiles96 <= kCUs && K >= 1024) return TILE_64x96;
+        // Where tiles of 64 x 64 would go through the CUs in more than one round (every CU's way
+        // from L2 carries the tile's rows of x and of w, and the CUs with the most tiles set the
+        // time), wider tiles that make a single round carry less per CU: one workgroup of two
+        // waves a CU, with a deep ring of stages in place of a second workgroup.  The narrowest
+        // of the widths 96, 128, 160 and 224 that fits N into one round is taken (64 x 24576 x
+        // 4096 with SwiGLU: 384 tiles of 64 x 64 49.3 us, 256 of 64 x 96 37.5; 64 x 51200 x 5120:
+        // 400 tiles of 64 x 128 in two rounds 109 us, 229 of 64 x 224 96).
+        const long long tiles64 = tile_count(TILE_64x64, M, N);
+        if (tiles64 > kCUs && K >= 1024) {
+            for (const int t : {TILE_64x96, TILE_64x128_ONE, TILE_64x160, TILE_64x224})
+                if (tile_count(t, M, N) <= kCUs) return t;
+        }
         if (whole_k_64x64(M, N, K) || tiles64 <= 128) return TILE_64x64;
         return TILE_64x128;
     }
-    const double rate[TILE_COUNT] = {0.70, 0.82, 0.90, 0.94, 1.0, 0.87, 0.94, 0.5, 0.5, 0.97};
+    const double rate[TILE_COUNT] = {0.70, 0.82, 0.90, 0.94, 1.0, 0.87, 0.94, 0.5, 0.5, 0.97, 0.6, 0.6, 0.6};
     int best = -1;
     double best_cost = 0.0;
     const int candidates[] = {TILE_64x128, TILE_128x128, TILE_256x128, TILE_256x192, TILE_256x256, TILE_192x128,
@@ -1292,6 +1298,9 @@ static int launch_bf16(const bf16* x, const bf16* w, TO* out, float* workspace, 
     case TILE_64x64:   return launch_tiled<64, 64, 3, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     case TILE_64x96:   return launch_tiled<64, 96, 6, EPI, TO, 2, 1>(x, w, out, workspace, M, N, K, shares, tail, s);
     case TILE_192x320: return launch_tiled<192, 320, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
+    case TILE_64x224:  return launch_tiled<64, 224, 4, EPI, TO, 2, 1>(x, w, out, workspace, M, N, K, shares, tail, s);
+    case TILE_64x128_ONE: return launch_tiled<64, 128, 5, EPI, TO, 2, 1>(x, w, out, workspace, M, N, K, shares, tail, s);
+    case TILE_64x160:  return launch_tiled<64, 160, 4, EPI, TO, 2, 1>(x, w, out, workspace, M, N, K, shares, tail, s);
     default:           return launch_tiled<256, 256, 2, EPI, TO>(x, w, out, workspace, M, N, K, shares, tail, s);
     }
 }

@@ -441,7 +441,8 @@ def _gemm_workspace(M: int, N: int, K: int, device) -> Optional[torch.Tensor]:
 
 def force_gemm_tile(tile: int) -> None:
     """Make the tiled bfloat16 product use one tile shape for every size (0: 64x128, 1: 128x128,
-    2: 256x128, 3: 256x192, 4: 256x256, 5: 192x128, 6: 192x256, 7: 64x64, 8: 64x96, 9: 192x320; -1: choose by size again).  For tests and tuning."""
+    2: 256x128, 3: 256x192, 4: 256x256, 5: 192x128, 6: 192x256, 7: 64x64, 8: 64x96, 9: 192x320, 10: 64x224,
+    11: 64x128 in one round, 12: 64x160; -1: choose by size again).  For tests and tuning."""
     _call("lc_gemm_bf16_force_tile", _c_int(tile))
 
 

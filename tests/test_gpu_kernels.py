@@ -272,7 +272,8 @@ def test_sampling_follows_the_distribution():
                                    (65, 128, 128), (128, 257, 512), (300, 1000, 640), (2048, 512, 1024),
                                    (3, 151936 // 8, 256), (33, 4096, 4096), (64, 6144, 1024), (48, 100, 128),
                                    (20, 24576, 256), (600, 3000, 256), (2, 331, 512), (13, 16400, 256),
-                                   (16, 24576, 128), (12, 16384, 2048), (40, 24576, 1024), (64, 20000, 1152)])
+                                   (16, 24576, 128), (12, 16384, 2048), (40, 24576, 1024), (64, 20000, 1152),
+                                   (33, 30000, 1024), (64, 38000, 1024), (50, 51200, 1024)])
 def test_gemm_bf16_matrix_cores(out_dtype, M, N, K):
     x = rnd(M, K, dtype=torch.bfloat16, seed=60)
     w = rnd(N, K, dtype=torch.bfloat16, seed=61)
@@ -282,7 +283,7 @@ def test_gemm_bf16_matrix_cores(out_dtype, M, N, K):
     close(got, want, out_dtype, scale=K ** 0.5)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12])
 @pytest.mark.parametrize("M,N,K", [(1, 16, 128), (70, 130, 128), (257, 300, 256), (300, 1000, 640),
                                    (513, 257, 384), (64, 128, 1024), (1000, 520, 2048), (100, 400, 128)])
 def test_gemm_bf16_every_tile_shape(tile, M, N, K):
