@@ -68,6 +68,9 @@ def main(argv=None) -> int:
     ap.add_argument("--wait-for-tokens", action="store_true",
                     help="read every step's tokens before the next step is queued (by default the "
                          "next step is queued first and takes them on the device)")
+    ap.add_argument("--stats", action="store_true",
+                    help="at the end, print the engine's counters and where the host's time went "
+                         "(LLMEngine.stats(), with the GPU time of the last step) as JSON on standard error")
     args = ap.parse_args(argv)
 
     if args.random_config:
@@ -90,7 +93,12 @@ def main(argv=None) -> int:
     engine = LLMEngine.from_folder(args.model, EngineConfig(
         dtype=args.dtype, block_size=args.block_size, max_blocks=args.max_blocks,
         max_tokens_per_step=args.max_tokens_per_step, max_seqs=args.max_seqs, device=args.device,
-        memory_fraction=args.mem_fraction, run_ahead=not args.wait_for_tokens))
+        memory_fraction=args.mem_fraction, run_ahead=not args.wait_for_tokens, time_steps=args.stats))
+
+    def report() -> None:
+        if args.stats:
+            print(json.dumps(engine.stats()), file=sys.stderr, flush=True)
+
     print(f"model ready: {len(engine.model.layers)} layers, {engine.runner.cache.num_blocks} pages "
           f"of {args.block_size} tokens", file=sys.stderr, flush=True)
 
@@ -130,6 +138,7 @@ def main(argv=None) -> int:
         outputs = engine.generate(prompts, [params(i) for i in range(len(prompts))])
         for out, text in zip(outputs, as_text):
             print(tokenizer.decode(out) if text else " ".join(str(t) for t in out), flush=True)
+        report()
         return 0
 
     # interactive: a request per line, generated ids streamed as they come
@@ -154,6 +163,7 @@ def main(argv=None) -> int:
         except ValueError as exc:
             print(f"error: {exc}", file=sys.stderr, flush=True)
         count += 1
+    report()
     return 0
 
 

@@ -502,9 +502,11 @@ def test_command_line_and_async_engine(tmp_path):
            "--max-blocks", "32", "--block-size", str(page), "--max-new-tokens", "6"]
     for p in prompts:
         cmd += ["--prompt-ids", ",".join(map(str, p))]
-    proc = subprocess.run(cmd, cwd=ROOT, text=True, capture_output=True, timeout=600)
+    proc = subprocess.run(cmd + ["--stats"], cwd=ROOT, text=True, capture_output=True, timeout=600)
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert [[int(t) for t in line.split()] for line in proc.stdout.strip().splitlines()] == want
+    stats = json.loads(proc.stderr.strip().splitlines()[-1])       # --stats: the last line on standard error
+    assert stats["steps"] >= 6 and stats["launch_s"] > 0 and stats["last_step_gpu_ms"] > 0
     # interactive: a request per line until "exit"
     proc = subprocess.run(cmd[:cmd.index("--prompt-ids")], cwd=ROOT, text=True, capture_output=True,
                           timeout=600, input=" ".join(map(str, prompts[0])) + "\nexit\n")
