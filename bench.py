@@ -65,6 +65,24 @@ SIZES_06B = dict(num_hidden_layers=28, hidden_size=1024, num_attention_heads=16,
                  max_position_embeddings=40960, initializer_range=0.02)
 
 
+SIZES_17B = dict(num_hidden_layers=28, hidden_size=2048, num_attention_heads=16,
+                 num_key_value_heads=8, head_dim=128, intermediate_size=6144, vocab_size=151936,
+                 rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
+                 max_position_embeddings=40960, initializer_range=0.02)
+
+SIZES_4B = dict(num_hidden_layers=36, hidden_size=2560, num_attention_heads=32,
+                num_key_value_heads=8, head_dim=128, intermediate_size=9728, vocab_size=151936,
+                rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
+                max_position_embeddings=40960, initializer_range=0.02)
+
+SIZES_14B = dict(num_hidden_layers=40, hidden_size=5120, num_attention_heads=40,
+                 num_key_value_heads=8, head_dim=128, intermediate_size=17408, vocab_size=151936,
+                 rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
+                 max_position_embeddings=40960, initializer_range=0.02)
+
+SIZES = {"8b": SIZES_8B, "32b": SIZES_32B, "0.6b": SIZES_06B, "1.7b": SIZES_17B, "4b": SIZES_4B, "14b": SIZES_14B}
+
+
 def say(text):
     print(f"[bench] {text}", file=sys.stderr, flush=True)
 
@@ -313,8 +331,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=8192)
-    ap.add_argument("--model", default="8b", choices=["8b", "32b", "0.6b"],
-                    help="layer sizes: Qwen3-8B-shaped (the default line), 32B- or 0.6B-shaped")
+    ap.add_argument("--model", default="8b", choices=sorted(SIZES),
+                    help="layer sizes: Qwen3-8B-shaped (the default line), or another size of the family")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the model has (0: all)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
@@ -360,7 +378,7 @@ def main() -> int:
         print(json.dumps(line), flush=True)
         return 0
 
-    sizes = {"8b": SIZES_8B, "32b": SIZES_32B, "0.6b": SIZES_06B}[args.model]
+    sizes = SIZES[args.model]
     points = [int(p) for p in args.points.split(",") if p]
     others = args.others == 1 or (args.others == -1 and args.model == "8b" and not args.layers
                                   and args.dtype == "bf16")
