@@ -514,7 +514,6 @@ def test_command_line_and_async_engine(tmp_path):
     assert [int(t) for t in proc.stdout.split()] == want[0]
 
     # text: a vocab.json beside the weights (every byte a token), the chat format with ids of this vocabulary
-    import json
     from lucciola_amd.text.vocab_tokenizer import ChatFormat, VocabTokenizer, byte_alphabet
     vocab = {c: b for b, c in enumerate(byte_alphabet())}
     with open(os.path.join(folder, "vocab.json"), "w", encoding="utf-8") as fh:
