@@ -46,6 +46,7 @@ _SIGNATURES = {
     "lc_gemm_bf16_scaled_rows_supported": "iii",
     "lc_qk_norm_rope_write": "piiiiippfppipppiip",
     "lc_attention_generic": "pipppipppiiiiiifipp",
+    "lc_attention_generic_rows": "i",
     "lc_attn_bf16_supported": "iiii",
     "lc_attn_page_granule": "",
     "lc_gemm_bf16_runs_ring_ok": "",

@@ -187,6 +187,14 @@ def test_attention_mixed_batch(dtype, nh, nkv, d, page, window):
                                                    batch.block_table.cpu()),
                          kc.cpu(), vc.cpu(), nh, nkv, d, page, d ** -0.5, window)
     close(got, want, dtype, atol=attention_atol(dtype, vc))
+    # the general kernel with several rows to a workgroup: rows of one request together, the others
+    # (a workgroup's rows straddle two requests) one after the other; every row the same bits
+    lib = ops.library()
+    lib.lc_attention_generic_rows(4)
+    try:
+        assert torch.equal(ops.attention(qkv, batch, kc, vc, nh, nkv, d, page, d ** -0.5, window), got)
+    finally:
+        lib.lc_attention_generic_rows(0)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -209,6 +217,20 @@ def test_attention_general_kernel_same_bits_alone_and_in_a_prompt(dtype, nh, nkv
     assert torch.equal(kc2, kc) and torch.equal(few.block_table, batch.block_table)
     tail = ops.attention(qkv[-alone:].contiguous(), few, kc, vc, nh, nkv, d, page, d ** -0.5, window)
     assert torch.equal(tail, got[-alone:])
+    # several rows of the prompt to a workgroup, which share every key and value they load (what a
+    # large prompt gets by itself); once with an odd number of rows, whose last workgroup has one
+    lib = ops.library()
+    lib.lc_attention_generic_rows(4)
+    try:
+        shared = ops.attention(qkv, batch, kc, vc, nh, nkv, d, page, d ** -0.5, window)
+        odd = ops.attention(qkv[1:].contiguous(), AttentionBatch(batch.tok_req[1:].contiguous(),
+                                                                 batch.positions[1:].contiguous(),
+                                                                 batch.block_table),
+                            kc, vc, nh, nkv, d, page, d ** -0.5, window)
+    finally:
+        lib.lc_attention_generic_rows(0)
+    assert torch.equal(shared, got)
+    assert torch.equal(odd, got[1:])
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
