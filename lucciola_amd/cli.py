@@ -46,7 +46,7 @@ def main(argv=None) -> int:
     ap.add_argument("--seed", "--sample-seed", dest="seed", type=int, default=0,
                     help="of the sampler, or of --random-config")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32", "bf16", "fp32"])
-    ap.add_argument("--max-tokens-per-step", type=int, default=576)
+    ap.add_argument("--max-tokens-per-step", type=int, default=2048)
     ap.add_argument("--max-seqs", type=int, default=256)
     ap.add_argument("--ignore-eos", action="store_true")
     ap.add_argument("--prompt-ids", action="append", default=[],

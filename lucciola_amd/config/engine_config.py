@@ -35,7 +35,10 @@ class EngineConfig:
     max_blocks: int = 0             # pages in each pool; 0: size from free memory
     memory_fraction: float = 0.90   # of free device memory, when max_blocks == 0
     memory_reserve: int = 500 << 20
-    max_tokens_per_step: int = 576
+    # tokens a step may run: decode tokens and portions of prompts together.  The reference cuts
+    # prompts at 576 (src/scheduler.cc:48); 256 CUs want more rows to a product (an 8B-shaped
+    # 2,048-token prompt runs at 68 k tokens a second whole and at 46 k in portions of 576)
+    max_tokens_per_step: int = 2048
     max_seqs: int = 256             # live requests (also the number of state slots)
     device: str = "cuda:0"
     use_graphs: bool = True         # replay decode steps from HIP graphs (bfloat16 on the GPU)

@@ -23,7 +23,7 @@ from .llm_engine import LLMEngine
 
 class AsyncEngine:
     def __init__(self, model_path: str, max_blocks: int = 0, block_size: int = 16,
-                 dtype="bfloat16", max_tokens_per_step: int = 576, max_seqs: int = 256,
+                 dtype="bfloat16", max_tokens_per_step: int = 2048, max_seqs: int = 256,
                  device: str = "cuda:0", engine: Optional[LLMEngine] = None,
                  tokenizer: Optional[VocabTokenizer] = None,
                  chat_format: Optional[ChatFormat] = ChatFormat()):

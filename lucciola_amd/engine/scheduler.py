@@ -3,7 +3,7 @@ tokens each.  Host code only; it decides from the cache manager's bookkeeping.
 
 What is kept from the reference (src/scheduler.cc:42-139): running requests are served first,
 one decode token each; then prompts are cut into portions under what is left of the step's
-token budget (576 there, src/scheduler.cc:48), first come first served; the step that feeds a
+token budget (576 there, src/scheduler.cc:48; 2,048 by default here), first come first served; the step that feeds a
 prompt's last token makes its request running, and that step's logits give its first new
 token (src/scheduler.cc:113-117).
 
@@ -53,7 +53,7 @@ class ScheduledStep:
 
 
 class Scheduler:
-    def __init__(self, cache: CacheManager, max_tokens_per_step: int = 576,
+    def __init__(self, cache: CacheManager, max_tokens_per_step: int = 2048,
                  max_seqs: Optional[int] = None, max_model_len: int = 0, portion_multiple: int = 1):
         self.cache = cache
         self.max_tokens_per_step = int(max_tokens_per_step)
