@@ -1013,8 +1013,11 @@ static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* 
     // One workgroup per request and kv head (no shares): requests of unequal length leave the
     // long ones running alone at the end, each at the pace its waves draw on memory; eight
     // waves double that (64 requests of 16 to 2,176 tokens: 59 instead of 65 us; equal lengths
-    // take the same time either way, short shares are slower with eight).
-    const int waves = g_decode_waves ? g_decode_waves : (splits == 1 && max_blocks >= 32 ? 8 : 4);
+    // take the same time either way, short shares are slower with eight).  From four workgroups
+    // a CU on, four waves: all of them are on the CUs at once instead of in two rounds (128
+    // requests of 1,024 tokens: 116 instead of 125 us; 96 requests: 95 against 93).
+    const int waves = g_decode_waves ? g_decode_waves
+                      : (splits == 1 && max_blocks >= 32 && (long long)ND * nkv < 4ll * device_cus() ? 8 : 4);
     if (waves == 8)
         attn_decode_kernel<D, 8><<<grid, 512, 0, s>>>(qkv, q_stride, k, v, out, part_o, part_ml,
                                                       decode_tokens, tok_req, positions, table, max_blocks,

@@ -1049,7 +1049,10 @@ static int pick_tile(int M, int N, int K, bool partials_wanted = false) {
         if (whole_k_64x64(M, N, K) || tiles64 <= 128) return TILE_64x64;
         return TILE_64x128;
     }
-    const double rate[TILE_COUNT] = {0.70, 0.82, 0.90, 0.94, 1.0, 0.87, 0.94, 0.5, 0.5, 0.97, 0.6, 0.6, 0.6};
+    // (tiles of 64 x 128 for 65 to 128 rows: every tile of w's rows reads all of x again, 96 x
+    // 24576 x 4096 with SwiGLU takes 57 us in them and 52 as 192 tiles of 192 x 128 in one round,
+    // 128 rows 62 and 50)
+    const double rate[TILE_COUNT] = {0.55, 0.82, 0.90, 0.94, 1.0, 0.87, 0.94, 0.5, 0.5, 0.97, 0.6, 0.6, 0.6};
     int best = -1;
     double best_cost = 0.0;
     const int candidates[] = {TILE_64x128, TILE_128x128, TILE_256x128, TILE_256x192, TILE_256x256, TILE_192x128,
