@@ -26,7 +26,7 @@ batch and launching, plus queueing the sampler; ``host_split_ms`` has the parts,
 for the engine's loop from ``LLMEngine.stats()``).  ``points`` holds, in tokens a second:
 decode at the other batch sizes at the headline's context (``decode_b1``, ``decode_b64``) and
 at a context of 1,024 tokens (``decode_b1_ctx1024``, ...: the length of the prompts that the
-baseline's runs decode after), the same batch driven through ``LLMEngine`` and its scheduler
+baseline's runs decode after; there also a batch of 256, ``decode_b256_ctx1024``), the same batch driven through ``LLMEngine`` and its scheduler
 after real prompts of the context length (``decode_b8_engine``), the 2,048-token prompt fed in
 portions of 576, the reference's step budget (src/scheduler.cc:48; ``prefill_576``), and the
 other shapes (``32b_decode_b1``, ``32b_decode_b32``, ``32b_prefill_2048``, ``0.6b_mixed``).
@@ -91,7 +91,7 @@ class ModelBench:
     """One model with random weights and a cache for its largest run, and the timed runs."""
 
     def __init__(self, sizes, layers, dtype, dev, block_size, max_batch, max_context, prefill_tokens,
-                 run_ahead, spare_steps):
+                 run_ahead, spare_steps, max_seqs=0):
         import torch
         from lucciola_amd.config.engine_config import EngineConfig
         from lucciola_amd.engine.loading import random_model
@@ -109,7 +109,7 @@ class ModelBench:
         t0 = time.time()
         self.model, self.mcfg = random_model(cfg, seed=0, dtype=self.dtype, device=dev)
         self.runner = ModelRunner(self.model, EngineConfig(dtype=self.dtype, block_size=block_size,
-                                                           max_blocks=blocks, max_seqs=max_batch + 2, device=dev))
+                                                           max_blocks=blocks, max_seqs=max(max_batch, max_seqs) + 2, device=dev))
         for ((k, v),) in self.runner.cache.storage.values():
             k.normal_(0, 0.5)
             v.normal_(0, 0.5)
@@ -337,6 +337,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--points", default="1,64", help="further decode batch sizes (comma list, '' for none)")
+    ap.add_argument("--short-points", default="256",
+                    help="further batch sizes measured at the short context only (those that fit the cache)")
     ap.add_argument("--short-context", type=int, default=1024,
                     help="also decode at this context, at the headline's batch and the batches of --points (0: skip)")
     ap.add_argument("--block-size", type=int, default=16)
@@ -383,9 +385,14 @@ def main() -> int:
     others = args.others == 1 or (args.others == -1 and args.model == "8b" and not args.layers
                                   and args.dtype == "bf16")
     point_steps = max(args.steps, 50)
-    bench = ModelBench(sizes, args.layers, args.dtype, dev, args.block_size, max([args.batch] + points),
+    short_points = [int(p) for p in args.short_points.split(",") if p] if args.short_context else []
+    most = max([args.batch] + points)
+    # the larger batches of the short context must fit the cache that the longest run needs
+    short_points = [b for b in short_points
+                    if b * (args.short_context + point_steps + 16) <= most * max(args.context, args.short_context)]
+    bench = ModelBench(sizes, args.layers, args.dtype, dev, args.block_size, most,
                        max(args.context, args.short_context), args.prefill_tokens, args.run_ahead,
-                       spare_steps=point_steps + args.warmup + 8)
+                       spare_steps=point_steps + args.warmup + 8, max_seqs=max([0] + short_points))
     values, fractions = {}, {}
 
     # The prompt and the other decode points first, the headline after them: a GPU that has just been handed its weights
@@ -400,7 +407,7 @@ def main() -> int:
         say(f"decode batch {b}: {r['ms']:.3f} ms/step (gpu {r['gpu_ms']:.3f}, host {r['host_ms']:.3f}), "
             f"{r['frac']:.3f} of the HBM peak")
     if args.short_context and args.short_context != args.context:
-        for b in sorted(set(points + [args.batch]), reverse=True):
+        for b in sorted(set(points + [args.batch] + short_points), reverse=True):
             r = bench.decode_run(b, args.short_context, point_steps, 3)
             key = f"decode_b{b}_ctx{args.short_context}"
             values[key], fractions[key] = round(r["tps"], 2), round(r["frac"], 4)
