@@ -1,211 +1,158 @@
-// out[M, N] = x[M, K] . w[N, K]^T for any sizes and any mix of float32 / bfloat16 operands,
-// accumulated with float32 FMAs (no matrix-core instruction, so that with float32 operands it
-// is a true 32-bit product).  The weight layout is the checkpoint's: [out_features,
-// in_features] row-major, applied as y = x . W^T without bias (reference:
-// src/kernels/linear.cu:24-27, one thread per output element; here LDS-tiled 64x64x16 with a
-// 4x4 register tile per thread; up to 16 rows: 16x64x16 with four rows of a column per thread).
+// out[M, N] = x[M, K] . w[N, K]^T for any sizes and any mix of float32 / bfloat16 operands, as a
+// true 32-bit product: the operands are widened to float32 and multiplied on the matrix cores in
+// float32 (v_mfma_f32_16x16x4_f32: float32 products, float32 sums, no reduced-precision mode).
+// The weight layout is the checkpoint's: [out_features, in_features] row-major, applied as
+// y = x . W^T without bias (reference: src/kernels/linear.cu:24-27, one thread per output
+// element; here tiles of 128 x 128, 64 x 64 or, for up to 16 rows, 16 x 64, staged through LDS
+// 16 k at a time, four waves with a grid of 16 x 16 products each).
 //
 // The order of the additions is a function of the output element alone: K is cut into chunks of
-// 256; within a chunk the products are added one after the other from 0, and the chunks' sums
-// are added one after the other from 0.  With few tiles (a decode step: up to 64 rows and a
-// narrow N) the chunks are shared out over workgroups, which leave their sums in a workspace,
-// and a second kernel adds them in the same order: a row's result has the same bits whether it
-// is computed alone or among thousands.
+// 256; within a chunk the element's sum takes four k at a time, in order (one matrix
+// instruction each, the same in every tile shape), and the chunks' sums are added one after the
+// other from 0.  With few tiles (a decode step: up to 64 rows and a narrow N) the chunks are
+// shared out over workgroups, which leave their sums in a workspace, and a second kernel adds
+// them in the same order: a row's result has the same bits whether it is computed alone or
+// among thousands.
 #include "common.h"
 
 namespace lc {
 
 constexpr int GB_M = 64, GB_N = 64, GB_K = 16;
 constexpr int GB_CHUNK = 256;   // k elements whose products are added up before they join the total
+constexpr int GB_PAD = 16;      // a row of a stage is its tile's rows and 16 floats: the four k that a wave reads
+                                // at once (16 lanes each) then lie in different banks
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
+// Tile BM x BN, WM x WN waves, each with (BM / 16 / WM) x (BN / 16 / WN) products of 16 x 16.
 // part == nullptr: out = x . w^T.  Else blockIdx.z owns the chunks [z * per, (z + 1) * per) and
 // writes each chunk's sums to part[chunk][M][N].
-template <typename TX, typename TW, typename TO>
-__global__ __launch_bounds__(256) void gemm_generic_kernel(const TX* __restrict__ x,
+template <typename TX, typename TW, typename TO, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(256, 2) void gemm_generic_kernel(const TX* __restrict__ x,
                                                            const TW* __restrict__ w,
                                                            TO* __restrict__ out, int M, int N,
                                                            int K, float* __restrict__ part, int per) {
-    __shared__ float xs[GB_K][GB_M + 4];
-    __shared__ float ws[GB_K][GB_N + 4];
-    const int tid = threadIdx.x;
-    const int m0 = blockIdx.y * GB_M, n0 = blockIdx.x * GB_N;
-    const int tm = (tid / 16) * 4, tn = (tid % 16) * 4;
+    static_assert(WM * WN == 4, "four waves");
+    constexpr int TM = BM / 16 / WM, TN = BN / 16 / WN;
+    constexpr int XL = (BM * 4 + 255) / 256, WL = (BN * 4 + 255) / 256;   // 16-byte pieces a thread loads per stage
+    __shared__ float xs[2][GB_K][BM + GB_PAD];     // two stages: one is filled while the other is multiplied
+    __shared__ float ws[2][GB_K][BN + GB_PAD];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int wm = (wave / WN) * (BM / WM), wn = (wave % WN) * (BN / WN);
     const int chunks = (K + GB_CHUNK - 1) / GB_CHUNK;
     const int c_begin = part ? blockIdx.z * per : 0;
     const int c_end = part ? min(c_begin + per, chunks) : chunks;
-    float total[4][4] = {};
+    floatx4 total[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) total[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // loader mapping: 64 rows x 16 k; a thread loads 4 consecutive k of one row of x and of w,
-    // a step ahead of the products that use them (the loads of step k0 + 16 are in flight while
-    // step k0 is multiplied)
+    // loader mapping: rows x 16 k; a thread loads 4 consecutive k of a row (of up to XL rows of x
+    // and WL of w, 64 apart), a step ahead of the products that use them (the loads of step
+    // k0 + 16 are in flight while step k0 is multiplied)
     const int lrow = tid / 4, lk = (tid % 4) * 4;
-    const bool x_row = m0 + lrow < M, w_row = n0 + lrow < N;
-    const TX* xp = x + (size_t)min(m0 + lrow, M - 1) * K + lk;
-    const TW* wp = w + (size_t)min(n0 + lrow, N - 1) * K + lk;
     // whole 16-byte (8-byte) pieces where the row length allows it
     const bool vec = (K & 3) == 0 && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
-    float xr[4], wr[4];
-    auto fetch = [&](int k0) {
-        if (vec && k0 + lk + 3 < K) {
-            load4(xr, xp + k0);
-            load4(wr, wp + k0);
-        } else {
+    float xr[XL][4], wr[WL][4];
+    auto fetch_rows = [&](auto* rows_ptr, int first, int limit, int tile_rows, int count, float (*dst)[4], int k0) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int k = k0 + lk + j;
-                xr[j] = k < K ? to_f32(xp[k0 + j]) : 0.f;
-                wr[j] = k < K ? to_f32(wp[k0 + j]) : 0.f;
-            }
-        }
-        if (!x_row) { xr[0] = xr[1] = xr[2] = xr[3] = 0.f; }
-        if (!w_row) { wr[0] = wr[1] = wr[2] = wr[3] = 0.f; }
-    };
-    if (c_begin < c_end) fetch(c_begin * GB_CHUNK);
-    for (int c = c_begin; c < c_end; ++c) {
-        float acc[4][4] = {};
-        const int k_end = min(K, (c + 1) * GB_CHUNK);
-        for (int k0 = c * GB_CHUNK; k0 < k_end; k0 += GB_K) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                xs[lk + j][lrow] = xr[j];
-                ws[lk + j][lrow] = wr[j];
-            }
-            __syncthreads();
-            {   // the step after this one, which may be the first of the next chunk
-                const int next = k0 + GB_K;
-                if (next < k_end || c + 1 < c_end) fetch(next < k_end ? next : (c + 1) * GB_CHUNK);
-            }
-#pragma unroll
-            for (int kk = 0; kk < GB_K; ++kk) {
-                float a[4], b[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) a[i] = xs[kk][tm + i];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) b[j] = ws[kk][tn + j];
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
-            }
-            __syncthreads();
-        }
-        if (part) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int m = m0 + tm + i;
-                if (m >= M) continue;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int n = n0 + tn + j;
-                    if (n < N) part[((size_t)c * M + m) * N + n] = acc[i][j];
-                }
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) total[i][j] = __fadd_rn(total[i][j], acc[i][j]);
-        }
-    }
-    if (part) return;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int m = m0 + tm + i;
-        if (m >= M) continue;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int n = n0 + tn + j;
-            if (n < N) out[(size_t)m * N + n] = from_f32<TO>(total[i][j]);
-        }
-    }
-}
-
-// The same product for up to 16 rows of x (a decode step): tiles of 16 x 64, a thread owns four
-// rows of one column and reads four k of both operands at a time.  Every output element sees
-// the same operations in the same order as in the kernel above.
-constexpr int GF_M = 16;
-
-template <typename TX, typename TW, typename TO>
-__global__ __launch_bounds__(256) void gemm_generic_few_kernel(const TX* __restrict__ x,
-                                                               const TW* __restrict__ w,
-                                                               TO* __restrict__ out, int M, int N,
-                                                               int K, float* __restrict__ part, int per) {
-    __shared__ __align__(16) float xs[GF_M][GB_K];
-    __shared__ __align__(16) float ws[GB_N][GB_K + 4];
-    const int tid = threadIdx.x;
-    const int m0 = blockIdx.y * GF_M, n0 = blockIdx.x * GB_N;
-    const int tn = tid % GB_N, tm = (tid / GB_N) * 4;
-    const int chunks = (K + GB_CHUNK - 1) / GB_CHUNK;
-    const int c_begin = part ? blockIdx.z * per : 0;
-    const int c_end = part ? min(c_begin + per, chunks) : chunks;
-    float total[4] = {};
-
-    const int lrow = tid / 4, lk = (tid % 4) * 4;
-    const bool x_loader = lrow < GF_M, x_row = x_loader && m0 + lrow < M, w_row = n0 + lrow < N;
-    const TX* xp = x + (size_t)min(m0 + lrow, M - 1) * K + lk;
-    const TW* wp = w + (size_t)min(n0 + lrow, N - 1) * K + lk;
-    const bool vec = (K & 3) == 0 && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
-    float xr[4] = {}, wr[4];
-    auto fetch = [&](int k0) {
-        if (vec && k0 + lk + 3 < K) {
-            if (x_row) load4(xr, xp + k0);
-            load4(wr, wp + k0);
-        } else {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int k = k0 + lk + j;
-                xr[j] = (x_row && k < K) ? to_f32(xp[k0 + j]) : 0.f;
-                wr[j] = k < K ? to_f32(wp[k0 + j]) : 0.f;
-            }
-        }
-        if (!x_row) { xr[0] = xr[1] = xr[2] = xr[3] = 0.f; }
-        if (!w_row) { wr[0] = wr[1] = wr[2] = wr[3] = 0.f; }
-    };
-    if (c_begin < c_end) fetch(c_begin * GB_CHUNK);
-    for (int c = c_begin; c < c_end; ++c) {
-        float acc[4] = {};
-        const int k_end = min(K, (c + 1) * GB_CHUNK);
-        for (int k0 = c * GB_CHUNK; k0 < k_end; k0 += GB_K) {
-            if (x_loader) *reinterpret_cast<float4*>(&xs[lrow][lk]) = make_float4(xr[0], xr[1], xr[2], xr[3]);
-            *reinterpret_cast<float4*>(&ws[lrow][lk]) = make_float4(wr[0], wr[1], wr[2], wr[3]);
-            __syncthreads();
-            {
-                const int next = k0 + GB_K;
-                if (next < k_end || c + 1 < c_end) fetch(next < k_end ? next : (c + 1) * GB_CHUNK);
-            }
-#pragma unroll
-            for (int kk = 0; kk < GB_K; kk += 4) {
-                const float4 b = *reinterpret_cast<const float4*>(&ws[tn][kk]);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float4 a = *reinterpret_cast<const float4*>(&xs[tm + i][kk]);
-                    acc[i] = fmaf(a.x, b.x, acc[i]);
-                    acc[i] = fmaf(a.y, b.y, acc[i]);
-                    acc[i] = fmaf(a.z, b.z, acc[i]);
-                    acc[i] = fmaf(a.w, b.w, acc[i]);
-                }
-            }
-            __syncthreads();
-        }
-        const int n = n0 + tn;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int m = m0 + tm + i;
-            if (part) {
-                if (m < M && n < N) part[((size_t)c * M + m) * N + n] = acc[i];
+        for (int u = 0; u < count; ++u) {
+            const int row = lrow + 64 * u;
+            const bool live = row < tile_rows && first + row < limit;
+            const auto* p = rows_ptr + (size_t)min(first + row, limit - 1) * K + lk;
+            if (vec && k0 + lk + 3 < K) {
+                load4(dst[u], p + k0);
             } else {
-                total[i] = __fadd_rn(total[i], acc[i]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) dst[u][j] = k0 + lk + j < K ? to_f32(p[k0 + j]) : 0.f;
             }
+            if (!live) { dst[u][0] = dst[u][1] = dst[u][2] = dst[u][3] = 0.f; }
         }
+    };
+    auto fetch = [&](int k0) {
+        fetch_rows(x, m0, M, BM, XL, xr, k0);
+        fetch_rows(w, n0, N, BN, WL, wr, k0);
+    };
+    auto put = [&](int stage) {
+#pragma unroll
+        for (int u = 0; u < XL; ++u)
+            if (lrow + 64 * u < BM)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) xs[stage][lk + j][lrow + 64 * u] = xr[u][j];
+#pragma unroll
+        for (int u = 0; u < WL; ++u)
+            if (lrow + 64 * u < BN)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) ws[stage][lk + j][lrow + 64 * u] = wr[u][j];
+    };
+    // every step of 16 k, over all of this workgroup's chunks, is a stage: stage s is written to
+    // LDS while stage s - 1 is multiplied, one barrier a stage
+    int stage = 0;
+    if (c_begin < c_end) {
+        fetch(c_begin * GB_CHUNK);
+        put(0);
+    }
+    for (int c = c_begin; c < c_end; ++c) {
+        floatx4 acc[TM][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+        const int k_end = min(K, (c + 1) * GB_CHUNK);
+        for (int k0 = c * GB_CHUNK; k0 < k_end; k0 += GB_K) {
+            __syncthreads();            // this stage is written; the other has been read by everybody
+            const int next = k0 + GB_K;
+            const bool more = next < k_end || c + 1 < c_end;
+            if (more) fetch(next < k_end ? next : (c + 1) * GB_CHUNK);
+            // lane l brings x[row l % 16][k l / 16] of each of its tiles, and w likewise; all of
+            // the stage's operands are asked for before the first product
+            float a[4][TM], b[4][TN];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i) a[q][i] = xs[stage][4 * q + (lane >> 4)][wm + 16 * i + (lane & 15)];
+#pragma unroll
+                for (int j = 0; j < TN; ++j) b[q][j] = ws[stage][4 * q + (lane >> 4)][wn + 16 * j + (lane & 15)];
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[q][i], b[q][j], acc[i][j], 0, 0, 0);
+            stage ^= 1;
+            if (more) put(stage);
+        }
+        // lane l holds the rows 4 (l / 16) + r and the column l % 16 of each of its tiles
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (part) {
+                        const int m = m0 + wm + 16 * i + 4 * (lane >> 4) + r, n = n0 + wn + 16 * j + (lane & 15);
+                        if (m < M && n < N) part[((size_t)c * M + m) * N + n] = acc[i][j][r];
+                    } else {
+                        total[i][j][r] = __fadd_rn(total[i][j][r], acc[i][j][r]);
+                    }
+                }
     }
     if (part) return;
-    const int n = n0 + tn;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int m = m0 + tm + i;
-        if (m < M && n < N) out[(size_t)m * N + n] = from_f32<TO>(total[i]);
-    }
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = m0 + wm + 16 * i + 4 * (lane >> 4) + r, n = n0 + wn + 16 * j + (lane & 15);
+                if (m < M && n < N) out[(size_t)m * N + n] = from_f32<TO>(total[i][j][r]);
+            }
 }
+
+constexpr int GF_M = 16;        // rows of the tile for a decode step's few rows
 
 // out = the chunks' sums part[c][M][N] added one after the other from 0, as the kernel above
 // adds them when it keeps them to itself
@@ -241,30 +188,35 @@ static int launch_generic(const void* x, const void* w, void* out, int M, int N,
     const int per = chunks_per_workgroup(M, N, K);
     const int chunks = (K + GB_CHUNK - 1) / GB_CHUNK;
     const bool few = M <= GF_M;
+    // tiles of 128 x 128 where they fill the card (they bring half as many bytes into a CU per product)
+    const bool large = per == 0 && M > GB_M && (long long)((N + 127) / 128) * ((M + 127) / 128) >= device_cus();
+    float* part = nullptr;
+    int shares = 1;
     if (per > 0) {
         LC_CHECK(workspace, "gemm: M=%d N=%d K=%d needs a workspace", M, N, K);
-        dim3 grid((N + GB_N - 1) / GB_N, few ? 1 : (M + GB_M - 1) / GB_M, (chunks + per - 1) / per);
-        if (few)
-            gemm_generic_few_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>((const TX*)x, (const TW*)w, (TO*)out, M,
-                                                                          N, K, workspace, per);
-        else
-            gemm_generic_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>((const TX*)x, (const TW*)w, (TO*)out, M, N,
-                                                                      K, workspace, per);
-        LC_LAUNCH_CHECK("gemm_generic");
+        part = workspace;
+        shares = (chunks + per - 1) / per;
+    }
+    if (few) {
+        dim3 grid((N + GB_N - 1) / GB_N, 1, shares);
+        gemm_generic_kernel<TX, TW, TO, GF_M, GB_N, 1, 4><<<grid, 256, 0, stream>>>(
+            (const TX*)x, (const TW*)w, (TO*)out, M, N, K, part, per);
+    } else if (large) {
+        dim3 grid((N + 127) / 128, (M + 127) / 128, 1);
+        gemm_generic_kernel<TX, TW, TO, 128, 128, 2, 2><<<grid, 256, 0, stream>>>(
+            (const TX*)x, (const TW*)w, (TO*)out, M, N, K, nullptr, 0);
+    } else {
+        dim3 grid((N + GB_N - 1) / GB_N, (M + GB_M - 1) / GB_M, shares);
+        gemm_generic_kernel<TX, TW, TO, GB_M, GB_N, 2, 2><<<grid, 256, 0, stream>>>(
+            (const TX*)x, (const TW*)w, (TO*)out, M, N, K, part, per);
+    }
+    LC_LAUNCH_CHECK("gemm_generic");
+    if (per > 0) {
         const size_t MN = (size_t)M * N;
         gemm_generic_sum_kernel<TO><<<(int)((MN + 255) / 256 < 4096 ? (MN + 255) / 256 : 4096), 256, 0, stream>>>(
             workspace, (TO*)out, MN, chunks);
         LC_LAUNCH_CHECK("gemm_generic_sum");
-        return 0;
     }
-    dim3 grid((N + GB_N - 1) / GB_N, few ? 1 : (M + GB_M - 1) / GB_M);
-    if (few)
-        gemm_generic_few_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>((const TX*)x, (const TW*)w, (TO*)out, M, N,
-                                                                      K, nullptr, 0);
-    else
-        gemm_generic_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>((const TX*)x, (const TW*)w, (TO*)out, M, N, K,
-                                                                  nullptr, 0);
-    LC_LAUNCH_CHECK("gemm_generic");
     return 0;
 }
 
