@@ -300,9 +300,9 @@ __device__ __forceinline__ void attend_rows(
             if (pv_active) {
                 if constexpr (vec) {
                     // runs of four keys that start at a multiple of four lie in one page; a run
-                    // may reach over the chunk's ends, where the keys count nothing
-                    // (four runs are asked for before the first is used; they are taken in in
-                    // their order)
+                    // may reach over the chunk's ends, where the keys count nothing (two runs
+                    // of each of the thread's dims are asked for before the first is used; they
+                    // are taken in in their order).
                     // Nothing in the loop is left out by a branch: a run behind the chunk's last is
                     // the last run once more, and a key outside the chunk counts as a value of
                     // zero with the weight of a key inside it (p >= 0, so the sum is only ever
