@@ -1019,10 +1019,13 @@ static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* 
     // One workgroup a CU or fewer (one to four requests): eight waves halve each wave's walk
     // (one request of 8,192 tokens with its join 13.4 instead of 14.6 us, four of 1,024 10.1
     // instead of 10.9).
+    // Shares of up to 1,024 keys likewise (8 requests of 1,024 tokens in four shares 13.0
+    // instead of 14.0 us, 16 of 2,048 in two 28.2 instead of 28.9); longer shares stream as well
+    // with four waves, or better (8 requests of 8,192 tokens 45.7 against 47.9).
     const long long workgroups = (long long)ND * nkv * splits;
     const int waves = g_decode_waves ? g_decode_waves
                       : (splits == 1 && max_blocks >= 32 && workgroups < 4ll * device_cus()) ? 8
-                      : (splits > 1 && workgroups <= device_cus()) ? 8 : 4;
+                      : (splits > 1 && workgroups <= device_cus() && max_blocks * PAGE <= 1024 * splits) ? 8 : 4;
     if (waves == 8)
         attn_decode_kernel<D, 8><<<grid, 512, 0, s>>>(qkv, q_stride, k, v, out, part_o, part_ml,
                                                       decode_tokens, tok_req, positions, table, max_blocks,
@@ -1110,19 +1113,26 @@ LC_API int lc_attn_decode_waves(int waves) {
     return 0;
 }
 
-// Into how many shares the decode kernel cuts a request's pages.  Two workgroups fit on a CU
-// (measured to beat four), 512 on the GPU, and from about 384 on they draw all that memory
-// gives.  So: as many shares as keep the workgroups within 512 (one more, and a second round
-// of workgroups has to wait for the first: 3 requests in 22 shares each took 31 us, in 21 26);
-// with 257 to 383 workgroups of whole requests, three shares each (40 requests: 252 instead
-// of 282 us), with 384 to 447 two (48 requests: 291 instead of 305); from 448 on none.  A share has
-// 8 pages or more, and there are at most 32.
+// Into how many shares the decode kernel cuts a request's pages.  Up to one workgroup of whole
+// requests a CU: as many shares as give every CU one workgroup and no more (8 requests of 8,192
+// tokens: 45.7 us in four shares each, 49.8 in eight, 50.3 in six; 4 requests 28.2 in eight,
+// 30.7 in sixteen; 16 requests 102.8 in two, 106.6 in four; 24 requests 150.7 whole, 161.2 in
+// two; a workgroup more than the CUs, and a second round has to wait for the first: 3 requests
+// in 22 shares each took 31 us, in 21 26).  With 257 to 383 workgroups of whole requests, three
+// shares each (40 requests: 252 instead of 282 us), with 384 to 447 two (48 requests: 291
+// instead of 305); from 448 on none.  A share has 8 pages or more, and there are at most 32.
+static thread_local int g_force_splits = 0;    // > 0: this many shares where the pages allow (tests, tuning)
+LC_API int lc_attn_decode_force_splits(int splits) {
+    g_force_splits = splits > 0 ? splits : 0;
+    return 0;
+}
 LC_API int lc_attn_decode_splits(int num_decode, int nkv, int max_ctx) {
     if (num_decode <= 0) return 1;
     const int pages = (max_ctx + PAGE - 1) / PAGE;
+    if (g_force_splits > 0) return g_force_splits < pages ? (g_force_splits > 32 ? 32 : g_force_splits) : (pages > 32 ? 32 : pages);
     const long long base = (long long)num_decode * nkv;
     const int cus = device_cus();       // the thresholds were measured with 256 of them
-    long long splits = base >= cus * 7 / 4 ? 1 : base >= cus * 3 / 2 ? 2 : base > cus ? 3 : 2 * cus / base;
+    long long splits = base >= cus * 7 / 4 ? 1 : base >= cus * 3 / 2 ? 2 : base > cus ? 3 : cus / base;
     const int most = (pages + 7) / 8;
     if (splits > most) splits = most;
     if (splits > 32) splits = 32;

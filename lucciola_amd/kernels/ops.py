@@ -52,6 +52,7 @@ _SIGNATURES = {
     "lc_gemm_bf16_runs_ring_ok": "",
     "lc_attn_decode_splits": "iii",
     "lc_attn_decode_waves": "i",
+    "lc_attn_decode_force_splits": "i",
     "lc_attn_decode_bf16": "pippppppppp" + "iiiiii" + "f" + "ii" + "ippfpii" + "pii" + "p",
     "lc_attn_decode_takes_shares": "ii",
     "lc_gemm_bf16_sum_shares": "ppiiiip",
