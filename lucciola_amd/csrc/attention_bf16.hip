@@ -1025,7 +1025,8 @@ static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* 
     const long long workgroups = (long long)ND * nkv * splits;
     const int waves = g_decode_waves ? g_decode_waves
                       : (splits == 1 && max_blocks >= 32 && workgroups < 4ll * device_cus()) ? 8
-                      : (splits > 1 && workgroups <= device_cus() && max_blocks * PAGE <= 1024 * splits) ? 8 : 4;
+                      : (splits > 1 && workgroups <= device_cus() && max_blocks * PAGE <= 1024 * splits) ? 8
+                      : (splits == 2 && workgroups > 2ll * device_cus()) ? 8 : 4;   // two shares of more requests than CUs
     if (waves == 8)
         attn_decode_kernel<D, 8><<<grid, 512, 0, s>>>(qkv, q_stride, k, v, out, part_o, part_ml,
                                                       decode_tokens, tok_req, positions, table, max_blocks,
@@ -1114,13 +1115,20 @@ LC_API int lc_attn_decode_waves(int waves) {
 }
 
 // Into how many shares the decode kernel cuts a request's pages.  Up to one workgroup of whole
-// requests a CU: as many shares as give every CU one workgroup and no more (8 requests of 8,192
+// requests a CU: the number that costs least when the CUs take the workgroups in rounds, which is
+// mostly what gives every CU one workgroup and no more (12 requests of 8,192 tokens are better
+// off with five shares each, two rounds of 102 pages, than with two, one round of 256: 82.5
+// against 97.1 us) (8 requests of 8,192
 // tokens: 45.7 us in four shares each, 49.8 in eight, 50.3 in six; 4 requests 28.2 in eight,
 // 30.7 in sixteen; 16 requests 102.8 in two, 106.6 in four; 24 requests 150.7 whole, 161.2 in
 // two; a workgroup more than the CUs, and a second round has to wait for the first: 3 requests
-// in 22 shares each took 31 us, in 21 26).  With 257 to 383 workgroups of whole requests, three
-// shares each (40 requests: 252 instead of 282 us), with 384 to 447 two (48 requests: 291
-// instead of 305); from 448 on none.  A share has 8 pages or more, and there are at most 32.
+// in 22 shares each took 31 us, in 21 26).  With more workgroups of whole requests than CUs:
+// three shares each while all of them fit on the CUs at once, four four-wave workgroups a CU (40
+// requests of 8,192 tokens: 249 instead of 271 us; 44 requests of 4,096 in three shares each,
+// 1,056 workgroups, 162, whole 152, in two shares of eight waves 146); beyond that, up to one
+// and a half workgroups a CU and from 4,096 tokens on, two shares of eight waves (48 requests
+// of 8,192 tokens: 289 us, 311 with four waves, 302 whole); else none (52 requests of 4,096
+// tokens: 164 whole, 175 in two shares).  A share has 8 pages or more, and there are at most 32.
 static thread_local int g_force_splits = 0;    // > 0: this many shares where the pages allow (tests, tuning)
 LC_API int lc_attn_decode_force_splits(int splits) {
     g_force_splits = splits > 0 ? splits : 0;
@@ -1132,11 +1140,24 @@ LC_API int lc_attn_decode_splits(int num_decode, int nkv, int max_ctx) {
     if (g_force_splits > 0) return g_force_splits < pages ? (g_force_splits > 32 ? 32 : g_force_splits) : (pages > 32 ? 32 : pages);
     const long long base = (long long)num_decode * nkv;
     const int cus = device_cus();       // the thresholds were measured with 256 of them
-    long long splits = base >= cus * 7 / 4 ? 1 : base >= cus * 3 / 2 ? 2 : base > cus ? 3 : cus / base;
-    const int most = (pages + 7) / 8;
-    if (splits > most) splits = most;
-    if (splits > 32) splits = 32;
-    if (splits < 1) splits = 1;
+    int most = (pages + 7) / 8;
+    if (most > 32) most = 32;
+    if (most < 1) most = 1;
+    long long splits = 1;
+    if (base <= cus) {
+        // the CUs work through the workgroups in rounds; a workgroup costs its pages and about as
+        // much as 32 pages more to start, look up, prepare q and leave its sums
+        long long best = -1;
+        for (int s = 1; s <= most; ++s) {
+            const long long rounds = (base * s + cus - 1) / cus;
+            if (rounds > 2) break;      // more than two workgroups a CU were slower whenever measured
+            const long long cost = rounds * ((pages + s - 1) / s + 32);
+            if (best < 0 || cost < best) { best = cost; splits = s; }
+        }
+    } else {
+        splits = 3 * base <= 4 * cus ? 3 : (2 * base <= 3 * cus && pages >= 256) ? 2 : 1;
+        if (splits > most) splits = most;
+    }
     return (int)splits;
 }
 
