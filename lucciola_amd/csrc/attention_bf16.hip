@@ -1007,8 +1007,8 @@ template <int D>
 static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* out,
                          float* part_o, float* part_ml, const int* decode_tokens, const int* tok_req,
                          const int* positions, const int* table, int max_blocks, int ND, int nh,
-                         int nkv, float scale_log2, int window, int splits, DecodePrologue pro,
-                         hipStream_t s) {
+                         int nkv, float scale_log2, int window, int splits, bool even_lengths,
+                         DecodePrologue pro, hipStream_t s) {
     dim3 grid(splits, nkv, ND);
     // One workgroup per request and kv head (no shares): requests of unequal length leave the
     // long ones running alone at the end, each at the pace its waves draw on memory; eight
@@ -1016,17 +1016,21 @@ static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* 
     // take the same time either way, short shares are slower with eight).  From four workgroups
     // a CU on, four waves: all of them are on the CUs at once instead of in two rounds (128
     // requests of 1,024 tokens: 116 instead of 125 us; 96 requests: 95 against 93).
-    // One workgroup a CU or fewer (one to four requests): eight waves halve each wave's walk
-    // (one request of 8,192 tokens with its join 13.4 instead of 14.6 us, four of 1,024 10.1
-    // instead of 10.9).
-    // Shares of up to 1,024 keys likewise (8 requests of 1,024 tokens in four shares 13.0
-    // instead of 14.0 us, 16 of 2,048 in two 28.2 instead of 28.9); longer shares stream as well
-    // with four waves, or better (8 requests of 8,192 tokens 45.7 against 47.9).
+    // One workgroup a CU or fewer: eight waves, which keep twice the loads in flight on the CU
+    // (with cold caches, as in a step: 8 requests of 8,192 tokens in four shares each 55.8
+    // instead of 57.4 us, 16 in two 104.7 instead of 107.4, one request with its join 16.1 instead
+    // of 17.2, 8 of 1,024 tokens 15.7 instead of 16.8).  Two shares of more requests than CUs
+    // likewise.
     const long long workgroups = (long long)ND * nkv * splits;
+    // Whole requests of about the same length, more of them than CUs: nobody is left running
+    // alone, and four waves a workgroup are as good or better (with cold caches 48 requests of
+    // 1,024 tokens 48.8 instead of 53.5 us, 64 requests 58.9 instead of 61.7, 32 of 8,192 192
+    // instead of 194).
+    const bool alone_at_the_end = !even_lengths || workgroups <= device_cus();
     const int waves = g_decode_waves ? g_decode_waves
-                      : (splits == 1 && max_blocks >= 32 && workgroups < 4ll * device_cus()) ? 8
-                      : (splits > 1 && workgroups <= device_cus() && max_blocks * PAGE <= 1024 * splits) ? 8
-                      : (splits == 2 && workgroups > 2ll * device_cus()) ? 8 : 4;   // two shares of more requests than CUs
+                      : (splits == 1 && max_blocks >= 32 && workgroups < 4ll * device_cus() && alone_at_the_end) ? 8
+                      : (splits > 1 && workgroups <= device_cus()) ? 8
+                      : (splits == 2 && workgroups > 2ll * device_cus()) ? 8 : 4;
     if (waves == 8)
         attn_decode_kernel<D, 8><<<grid, 512, 0, s>>>(qkv, q_stride, k, v, out, part_o, part_ml,
                                                       decode_tokens, tok_req, positions, table, max_blocks,
@@ -1123,8 +1127,9 @@ LC_API int lc_attn_decode_waves(int waves) {
 // 30.7 in sixteen; 16 requests 102.8 in two, 106.6 in four; 24 requests 150.7 whole, 161.2 in
 // two; a workgroup more than the CUs, and a second round has to wait for the first: 3 requests
 // in 22 shares each took 31 us, in 21 26).  With more workgroups of whole requests than CUs:
-// three shares each while all of them fit on the CUs at once, four four-wave workgroups a CU (40
-// requests of 8,192 tokens: 249 instead of 271 us; 44 requests of 4,096 in three shares each,
+// three shares each from 2,048 tokens on and while all of them fit on the CUs at once, four
+// four-wave workgroups a CU (40 requests of 8,192 tokens: 249 instead of 271 us, of 1,024 tokens
+// 47.3 against 44.7 whole; 44 requests of 4,096 in three shares each,
 // 1,056 workgroups, 162, whole 152, in two shares of eight waves 146); beyond that, up to one
 // and a half workgroups a CU and from 4,096 tokens on, two shares of eight waves (48 requests
 // of 8,192 tokens: 289 us, 311 with four waves, 302 whole); else none (52 requests of 4,096
@@ -1151,11 +1156,14 @@ LC_API int lc_attn_decode_splits(int num_decode, int nkv, int max_ctx) {
         for (int s = 1; s <= most; ++s) {
             const long long rounds = (base * s + cus - 1) / cus;
             if (rounds > 2) break;      // more than two workgroups a CU were slower whenever measured
-            const long long cost = rounds * ((pages + s - 1) / s + 32);
+            // (two rounds, which are four-wave workgroups, count a tenth more than twice one round of
+            // eight-wave workgroups: with cold caches 12 requests of 8,192 tokens take 81.5 us in
+            // two shares each, 84.3 in five)
+            const long long cost = (rounds == 1 ? 10 : 22) * ((pages + s - 1) / s + 32);
             if (best < 0 || cost < best) { best = cost; splits = s; }
         }
     } else {
-        splits = 3 * base <= 4 * cus ? 3 : (2 * base <= 3 * cus && pages >= 256) ? 2 : 1;
+        splits = (3 * base <= 4 * cus && pages >= 128) ? 3 : (2 * base <= 3 * cus && pages >= 256) ? 2 : 1;
         if (splits > most) splits = most;
     }
     return (int)splits;
@@ -1182,7 +1190,7 @@ LC_API int lc_attn_decode_bf16(const void* qkv, int q_stride, void* k_cache, voi
                                void* out, float* part_o, float* part_ml, const int* decode_tokens,
                                const int* tok_req, const int* positions, const int* block_table,
                                int max_blocks, int num_decode, int nh, int nkv, int d, int page_size,
-                               float scale, int window, int splits, int prologue, const float* q_w,
+                               float scale, int window, int splits, int even_lengths, int prologue, const float* q_w,
                                const float* k_w, float eps, const float* rope_table, int rot,
                                int write_kv, const float* qkv_shares, int num_shares, int share_rows,
                                hipStream_t stream) {
@@ -1207,7 +1215,7 @@ LC_API int lc_attn_decode_bf16(const void* qkv, int q_stride, void* k_cache, voi
     const float sl2 = scale * 1.4426950408889634f;
 #define CALL(DD) launch_decode<DD>((const bf16*)qkv, q_stride, (bf16*)k_cache, (bf16*)v_cache,             \
         (bf16*)out, part_o, part_ml, decode_tokens, tok_req, positions, block_table, max_blocks,           \
-        num_decode, nh, nkv, sl2, window, splits, pro, stream)
+        num_decode, nh, nkv, sl2, window, splits, even_lengths != 0, pro, stream)
     LC_DISPATCH_D(d, CALL)
 #undef CALL
     return 0;

@@ -53,7 +53,7 @@ _SIGNATURES = {
     "lc_attn_decode_splits": "iii",
     "lc_attn_decode_waves": "i",
     "lc_attn_decode_force_splits": "i",
-    "lc_attn_decode_bf16": "pippppppppp" + "iiiiii" + "f" + "ii" + "ippfpii" + "pii" + "p",
+    "lc_attn_decode_bf16": "pippppppppp" + "iiiiii" + "f" + "iii" + "ippfpii" + "pii" + "p",
     "lc_attn_decode_takes_shares": "ii",
     "lc_gemm_bf16_sum_shares": "ppiiiip",
     "lc_attn_prefill_bf16": "pippppp" + "iiiiii" + "f" + "i" + "ipfpi" + "ipp" + "p",
@@ -548,6 +548,7 @@ class AttentionBatch:
     prefill_tiles: Optional[torch.Tensor] = None   # [NT, 4]: request, first token row, rows, first position
     max_ctx: int = 0                               # longest cached length in the batch
     all_decode: bool = False
+    even_lengths: bool = False                     # the decoding requests' lengths are within half of their mean
 
 
 PREFILL_TILE = 64               # query rows of one work item of the prefill attention kernel
@@ -577,8 +578,14 @@ def plan_attention(layout):
                 tile_list.append((r, q_start[r] + t0, min(PREFILL_TILE, n - t0), first[r] + t0))
         tile_list.sort(key=lambda t: -(t[3] + t[2]))
         tiles = np.asarray(tile_list, dtype=np.int32).reshape(-1, 4)
+    # lengths after this step of the requests that decode: a hint for the decode kernel (how
+    # it lays its work out, never what it computes); a captured step keeps the hint of its capture
+    lengths = np.asarray(first, dtype=np.int64) + 1
+    if not layout.single:
+        lengths = lengths[np.diff(np.asarray(q_start, dtype=np.int64)) == 1]
+    even = bool(lengths.size) and int(lengths.max()) * int(lengths.size) <= 1.5 * int(lengths.sum())
     return ({"decode_tokens": decode, "prefill_tiles": tiles},
-            {"num_decode": int(decode.size), "all_decode": int(decode.size) == R})
+            {"num_decode": int(decode.size), "all_decode": int(decode.size) == R, "even_lengths": even})
 
 
 # Tokens of a cache page as the matrix-core attention kernels index it: a page of a multiple of
@@ -606,7 +613,8 @@ def attention_batch(batch, pages, plan=None) -> AttentionBatch:
         if plan is not None:
             done = replace(done, decode_tokens=plan.arrays["decode_tokens"],
                            prefill_tiles=plan.arrays["prefill_tiles"],
-                           num_decode=plan.info["num_decode"], all_decode=plan.info["all_decode"])
+                           num_decode=plan.info["num_decode"], all_decode=plan.info["all_decode"],
+                           even_lengths=plan.info["even_lengths"])
         pages.made[ATTENTION_PLAN] = done
     return done
 
@@ -702,7 +710,7 @@ def attention(qkv, batch: AttentionBatch, k_cache: torch.Tensor,
             _call("lc_attn_decode_bf16", _ptr(qkv if shares is None else None), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
                   _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(batch.decode_tokens),
                   _ptr(batch.tok_req), _ptr(batch.positions), _ptr(batch.block_table), mb, nd, nh,
-                  nkv, d, page_size, scale, window, splits,
+                  nkv, d, page_size, scale, window, splits, 1 if batch.even_lengths else 0,
                   1 if in_kernel else 0,
                   _ptr(prologue.q_weight if in_kernel else None),
                   _ptr(prologue.k_weight if in_kernel else None),
