@@ -548,7 +548,7 @@ class AttentionBatch:
     prefill_tiles: Optional[torch.Tensor] = None   # [NT, 4]: request, first token row, rows, first position
     max_ctx: int = 0                               # longest cached length in the batch
     all_decode: bool = False
-    even_lengths: bool = False                     # the decoding requests' lengths are within half of their mean
+    even_lengths: bool = False                     # the longest decoding request is within a tenth of the mean length
 
 
 PREFILL_TILE = 64               # query rows of one work item of the prefill attention kernel
@@ -584,7 +584,7 @@ def plan_attention(layout):
     lengths = np.asarray(first, dtype=np.int64) + 1
     if not layout.single:
         lengths = lengths[np.diff(np.asarray(q_start, dtype=np.int64)) == 1]
-    even = bool(lengths.size) and int(lengths.max()) * int(lengths.size) <= 1.5 * int(lengths.sum())
+    even = bool(lengths.size) and int(lengths.max()) * int(lengths.size) <= 1.1 * int(lengths.sum())
     if lengths.size > 1 and int(lengths.max()) != int(lengths.min()):
         # the decode kernel's workgroups start in the order of this list: the longest requests first,
         # so that none of them starts late and runs on alone at the end (64 requests of 16 to 2,200
