@@ -1056,9 +1056,13 @@ static int pick_tile(int M, int N, int K, bool partials_wanted = false) {
     int best = -1;
     double best_cost = 0.0;
     const int candidates[] = {TILE_64x128, TILE_128x128, TILE_256x128, TILE_256x192, TILE_256x256, TILE_192x128,
-                              TILE_192x256, TILE_192x320};
+                              TILE_192x256, TILE_192x320, TILE_64x64};
     for (const int t : candidates) {
         if (t == TILE_64x128 && M > 128) continue;
+        // 64 x 64 above 256 rows: for the narrow products of a portion of a prompt, which have few
+        // larger tiles (2,048 x 1024 x 2048 with the norm that follows: 24.6 us in 512 whole tiles of
+        // 64 x 64, 31.2 as tiles of 128 x 128 cut along K four ways; 576 x 1024 x 3072 18.7 against 22.3)
+        if (t == TILE_64x64 && M <= 256) continue;
         const long long tiles = tile_count(t, M, N);
         const double area = (double)tile_bm(t) * tile_bn(t);
         const double work_us = area * K * 2.0 / (4.63e6 * rate[t]);
@@ -1338,6 +1342,14 @@ LC_API int lc_gemm_bf16_force_tile(int tile) {
     LC_CHECK(tile >= TILE_AUTO && tile < TILE_COUNT, "gemm_bf16: no tile shape %d", tile);
     g_force_tile = tile;
     return 0;
+}
+
+// The tile shape that a product of these sizes goes through (the numbers of lc_gemm_bf16_force_tile;
+// -1: up to 16 rows, which the skinny kernels take), and into how many shares of K it is cut;
+// partials: as lc_gemm_bf16_partials would do it.  For tests and tuning.
+LC_API int lc_gemm_bf16_tile(int M, int N, int K, int partials) {
+    if (!lc_gemm_bf16_supported(M, N, K) || (M <= 16 && g_force_tile == TILE_AUTO)) return -1;
+    return pick_tile(M, N, K, partials != 0);
 }
 
 // float32 words of workspace that lc_gemm_bf16 needs for these sizes (0: none).

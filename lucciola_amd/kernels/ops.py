@@ -40,6 +40,7 @@ _SIGNATURES = {
     "lc_gemm_bf16_residual_pieces": "iii",
     "lc_gemm_bf16_piece_stride": "i",
     "lc_gemm_bf16_shares": "iii",
+    "lc_gemm_bf16_tile": "iiii",
     "lc_gemm_bf16_partials": "pppiiip",
     "lc_gemm_bf16_residual": "ppppppiiip",
     "lc_gemm_bf16_scaled_rows": "pppiiiipifp",
