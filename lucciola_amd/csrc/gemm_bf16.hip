@@ -1062,10 +1062,16 @@ static int pick_tile(int M, int N, int K, bool partials_wanted = false) {
         // 64 x 64 above 256 rows: for the narrow products of a portion of a prompt, which have few
         // larger tiles (2,048 x 1024 x 2048 with the norm that follows: 24.6 us in 512 whole tiles of
         // 64 x 64, 31.2 as tiles of 128 x 128 cut along K four ways; 576 x 1024 x 3072 18.7 against 22.3)
-        if (t == TILE_64x64 && M <= 256) continue;
+        // (up to 256 rows only for a w of up to 32 MB: 128 x 4096 x 4096 with its norm 19.2 us against 21.1 in
+        // tiles of 64 x 128; on a large w every tile of 64 rows of w reads all of x again: 128 x 24576 x 4096
+        // 61.8 against 50.8 in tiles of 192 x 128.  Measured over the four products of six model sizes at 96 to
+        // 4,096 rows, the shape picked is within 8 % of the best of all shapes in 208 of 216 cases.)
+        if (t == TILE_64x64 && M <= 256 && (long long)N * K > (1ll << 24)) continue;
         const long long tiles = tile_count(t, M, N);
         const double area = (double)tile_bm(t) * tile_bn(t);
-        const double work_us = area * K * 2.0 / (4.63e6 * rate[t]);
+        // (tiles of 64 x 64 do better than their rate on a small w, which stays in the caches)
+        const double r = (t == TILE_64x64 && (long long)N * K <= (1ll << 24)) ? 0.62 : rate[t];
+        const double work_us = area * K * 2.0 / (4.63e6 * r);
         double cost;
         if (tile_bm(t) >= 192) {
             const double round_us = work_us + 3.0;
