@@ -1187,7 +1187,10 @@ static SkinnyPlan skinny_plan(int M, int N, int K, int epilogue) {
     // (measured at 8 rows: 201 MB of w 41.8 -> 38.7 us, 100 MB 24.8 -> 22.3, 1.2 GB 221 -> 213; 50 MB 12.4 -> 13.5 and
     // 34 MB 9.8 -> 10.1: the ring's start and the barrier of every stage cost the small ones more than the runs gain)
     // With one or two rows of x the kernel above, one tile a workgroup, is the faster one (1.2 GB of w: 196 against 206 us).
-    if (g_runs && g_force_skinny < 0 && K % SR_K == 0 && (g_runs > 1 || (M >= 4 && (long long)N * K >= (1ll << 25)))) {
+    // (a long K, as the down products have, gains from a smaller w on: 2560 x 9728 16.0 instead of 17.7 us at 8 rows,
+    // 2048 x 6144 12.0 instead of 13.1)
+    const bool large = (long long)N * K >= (1ll << 25) || (K >= 6144 && (long long)N * K >= (1ll << 23));
+    if (g_runs && g_force_skinny < 0 && K % SR_K == 0 && (g_runs > 1 || (M >= 4 && large))) {
         // tiles of 16 rows, or of as many as give every CU the same number (the SwiGLU epilogue keeps whole blocks of 16)
         p.runs = true;
         p.shape = SKINNY_PLAIN;
