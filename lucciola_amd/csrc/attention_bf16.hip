@@ -835,13 +835,16 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_wide_kernel(
     const int half_of = (total + 1) / 2;
     const int task = (total <= resident && number >= half_of) ? total - 1 - (number - half_of) : number;
     const int tile_index = task / gridDim.x, heads_index = task - tile_index * gridDim.x;
-    const int h = heads_index * 2 + (wave >> 1);
+    // the pairs of heads of one kv head; with an odd number of heads a kv head, the last pair is
+    // a single head, and the two waves of its other half only help to bring keys and values in
+    const int pairs = (G + 1) / 2;
+    const int kvh = heads_index / pairs, in_kv = (heads_index - kvh * pairs) * 2 + (wave >> 1);
+    const int h = min(kvh * G + in_kv, nh - 1);
     const int wrow = (wave & 1) * 32;
-    const int kvh = (heads_index * 2) / G;
     {
         const int* tile = tiles + (size_t)tile_index * 4;
         const int req = tile[0], row0 = tile[1], rows = tile[2], pos0 = tile[3];
-        const bool active = wrow < rows;
+        const bool active = wrow < rows && in_kv < G;
         const int* table = block_table + (size_t)req * max_blocks;
 
         const int my = wrow + q;
@@ -1066,8 +1069,11 @@ static int launch_prefill(const bf16* qkv, int q_stride, const bf16* k, const bf
     if constexpr (D == 128) {
         // heads of 128 in pairs, every tile's keys walked by one workgroup: the kernel built from
         // the wide products
-        if (g_prefill_wide && (nh / nkv) % 2 == 0 && splits == 1) {
-            attn_prefill_wide_kernel<D><<<dim3(nh / 2, NT), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
+        // (an odd number of heads a kv head from 3 on: the last pair is a single head, which leaves a CU's
+        // matrix cores half idle for a sixth of the pairs of five heads, where one head a workgroup in the
+        // kernel below takes 1.6 times as long for all of them)
+        if (g_prefill_wide && ((nh / nkv) % 2 == 0 || nh / nkv >= 3) && splits == 1) {
+            attn_prefill_wide_kernel<D><<<dim3(nkv * ((nh / nkv + 1) / 2), NT), 256, 0, s>>>(qkv, q_stride, k, v, out, tiles, table,
                                                                        max_blocks, nh, nkv, scale_log2, window, pro, resident);
             LC_LAUNCH_CHECK("attn_prefill_wide");
             return 0;

@@ -177,7 +177,7 @@ def paged_case(lengths, new, nh, nkv, d, page, dtype, seed, spare=3):
 @pytest.mark.parametrize("nh,nkv,d,page,window", [
     (4, 2, 16, 4, 0), (6, 2, 48, 16, 0), (8, 1, 32, 8, 0), (5, 5, 80, 16, 0), (32, 8, 128, 16, 0),
     (6, 2, 48, 16, 24), (4, 4, 64, 8, 5), (2, 1, 256, 16, 0), (4, 2, 64, 16, 0), (6, 2, 96, 16, 24),
-    (16, 1, 32, 16, 0), (32, 8, 128, 16, 40), (12, 4, 128, 16, 7)])
+    (16, 1, 32, 16, 0), (32, 8, 128, 16, 40), (12, 4, 128, 16, 7), (10, 2, 128, 16, 0), (5, 1, 128, 16, 33)])
 def test_attention_mixed_batch(dtype, nh, nkv, d, page, window):
     lengths = [1, 300, 17, 64, 130]
     new = [1, 1, 17, 2, 70]
@@ -481,10 +481,11 @@ def test_slow_paths_say_so_once(capfd):
     assert "no matrix-core" not in capfd.readouterr().err
 
 
-@pytest.mark.parametrize("nh,nkv,window", [(8, 2, 0), (4, 2, 100), (6, 1, 33), (2, 1, 0)])
+@pytest.mark.parametrize("nh,nkv,window", [(8, 2, 0), (4, 2, 100), (6, 1, 33), (2, 1, 0), (10, 2, 0), (3, 1, 50),
+                                           (15, 3, 0)])
 def test_attention_prefill_of_heads_of_128_in_pairs(nh, nkv, window):
-    """Heads of 128 with an even number of heads per kv head go to the prefill kernel built from
-    32x32x16 products: whole prompts, portions after a history, rows that do not fill a tile,
+    """Heads of 128 go in pairs of one kv head (of an odd number from three on, the last pair is
+    a single head) to the prefill kernel built from 32x32x16 products: whole prompts, portions after a history, rows that do not fill a tile,
     a window whose edge cuts through groups of keys, against the plain formulas and against the
     general kernel."""
     d = 128
