@@ -153,11 +153,13 @@ __device__ __forceinline__ void attend_range(AttnState<D, QT>& st, const bf16x8 
                                              const int* __restrict__ table, int begin, int end,
                                              int step, int nkv, int kvh, const int (&lo)[QT],
                                              const int (&hi)[QT], float scale_log2, int lane,
-                                             const int (&first_pages)[2]) {
-    // first_pages: table[begin] and table[begin + step], where they exist
+                                             const int (&first_pages)[2], PageRegs<D>& cur,
+                                             bool loaded) {
+    // first_pages: table[begin] and table[begin + step], where they exist; loaded: the caller
+    // has asked for the first page's keys and values (into cur) already
     if (begin >= end) return;
-    PageRegs<D> cur, nxt;
-    load_page<D>(cur, k_cache, v_cache, first_pages[0], nkv, kvh, lane);
+    PageRegs<D> nxt;
+    if (!loaded) load_page<D>(cur, k_cache, v_cache, first_pages[0], nkv, kvh, lane);
     int next_page = first_pages[1];
     for (int pg = begin; pg < end; pg += step) {
         const bool more = pg + step < end;
@@ -201,19 +203,21 @@ template <int D, int NW>
 __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
     const bf16* __restrict__ qkv, int q_stride, bf16* k_cache, bf16* v_cache,
     bf16* __restrict__ out, float* __restrict__ part_o,
-    float* __restrict__ part_ml, const int* __restrict__ decode_tokens,
-    const int* __restrict__ tok_req, const int* __restrict__ positions,
+    float* __restrict__ part_ml, const int4* __restrict__ decode_rows,
     const int* __restrict__ block_table, int max_blocks, int nh, int nkv, float scale_log2,
     int window, int splits, DecodePrologue pro) {
-    __shared__ float sm_o[NW][D * 16];
+    constexpr int ROW = D + 4;       // a head's D sums lie together; the padding spreads the heads over the banks
+    __shared__ __attribute__((aligned(16))) float sm_o[NW][16 * ROW];
     __shared__ float sm_m[NW][16], sm_l[NW][16];
     __shared__ __attribute__((aligned(16))) bf16 sm_q[16 * D];
 
     const int split = blockIdx.x, kvh = blockIdx.y, di = blockIdx.z;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int q = lane & 15, kg = lane >> 4;
-    const int t = decode_tokens[di];
-    const int req = tok_req[t], p = positions[t];
+    // the token's row in the batch, its request's row of the block table and its position come
+    // in one load: every look-up that hangs on another is a trip to memory before the first key
+    const int4 mine = decode_rows[di];
+    const int t = mine.x, req = mine.y, p = mine.z;
     const int G = nh / nkv;
     const int j_lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int first_page = j_lo / PAGE, last_page = p / PAGE;
@@ -227,6 +231,12 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
     // the page that takes the token's own k and v (asked for with the others, not when it is needed)
     const bool owner = pro.enabled && pro.write_kv && begin <= last_page && last_page < end;
     const int own_page = owner ? table[last_page] : 0;
+
+    // the wave's first page is asked for before q is prepared, so that the two trips to memory
+    // run side by side; not the page that this workgroup is about to write the token's own k and v into
+    PageRegs<D> first;
+    const bool early = pg0 < end && !(owner && pg0 == last_page);
+    if (early) load_page<D>(first, k_cache, v_cache, first_pages[0], nkv, kvh, lane);
 
     bf16x8 bq[1][D / 32];
     if (pro.enabled) {
@@ -282,8 +292,9 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
                 const size_t col = (size_t)(is_k ? nh + kvh : kvh * G + task) * D + 8 * j;
                 bf16* dst = is_k ? k_cache + (((size_t)own_page * nkv + kvh) * PAGE + (p % PAGE)) * D
                                  : sm_q + task * D;
-                const head_chunk done = head128_norm_rope(chunk_at(col), j,
-                                                          is_k ? pro.k_w : pro.q_w, pro.eps, cs);
+                // the weights and the table's row are asked for before the raw entries are waited for
+                const Head128Constants consts = head128_constants(j, is_k ? pro.k_w : pro.q_w, cs);
+                const head_chunk done = head128_norm_rope(chunk_at(col), j, consts, pro.eps);
                 *reinterpret_cast<head_chunk*>(dst + 8 * j) = done;
             }
         } else {
@@ -337,38 +348,43 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
     init_state<D, 1>(st);
     const int lo[1] = {j_lo}, hi[1] = {p};
     attend_range<D, 1>(st, bq, k_cache, v_cache, table, begin + wave, end, NW, nkv, kvh, lo, hi,
-                       scale_log2, lane, first_pages);
+                       scale_log2, lane, first_pages, first, early);
 
     // the waves' results meet in LDS
     float l = st.l[0];
     l = column_sum(l);
     if (kg == 0) { sm_m[wave][q] = st.m[0]; sm_l[wave][q] = l; }
+    if (q < G) {
 #pragma unroll
-    for (int tt = 0; tt < D / 16; ++tt)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) sm_o[wave][(tt * 16 + kg * 4 + v) * 16 + q] = st.o[0][tt][v];
+        for (int tt = 0; tt < D / 16; ++tt)
+            *reinterpret_cast<floatx4*>(&sm_o[wave][q * ROW + tt * 16 + kg * 4]) = st.o[0][tt];
+    }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < D * 16; idx += 64 * NW) {
-        const int dim = idx >> 4, qq = idx & 15;
-        if (qq >= G) continue;
+    // four sums of a head a thread
+    for (int idx = threadIdx.x; idx < G * (D / 4); idx += 64 * NW) {
+        const int qq = idx / (D / 4), dim = (idx % (D / 4)) * 4;
         float m_all = sm_m[0][qq];
 #pragma unroll
         for (int w = 1; w < NW; ++w) m_all = fmaxf(m_all, sm_m[w][qq]);
-        float o = 0.f, lsum = 0.f;
+        floatx4 o = {0.f, 0.f, 0.f, 0.f};
+        float lsum = 0.f;
         if (m_all != -INFINITY) {
 #pragma unroll
             for (int w = 0; w < NW; ++w) {
                 const float f = (sm_m[w][qq] == -INFINITY) ? 0.f : exp2f(sm_m[w][qq] - m_all);
-                o += f * sm_o[w][idx];
+                o += f * *reinterpret_cast<const floatx4*>(&sm_o[w][qq * ROW + dim]);
                 lsum += f * sm_l[w][qq];
             }
         }
         const int h = kvh * G + qq;
         if (splits == 1) {
-            out[((size_t)t * nh + h) * D + dim] = static_cast<bf16>(o / lsum);
+            short4v packed;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) packed[v] = bf16_bits(o[v] / lsum);
+            *reinterpret_cast<short4v*>(out + ((size_t)t * nh + h) * D + dim) = packed;
         } else {
             const size_t slot = ((size_t)di * nh + h) * splits + split;
-            part_o[slot * D + dim] = o;
+            *reinterpret_cast<floatx4*>(part_o + slot * D + dim) = o;
             if (dim == 0) { part_ml[slot * 2] = m_all; part_ml[slot * 2 + 1] = lsum; }
         }
     }
@@ -420,11 +436,11 @@ __device__ __forceinline__ void join_shares(const float* __restrict__ part_o,
 template <int D>
 __global__ __launch_bounds__(128) void attn_decode_join_kernel(const float* __restrict__ part_o,
                                                                const float* __restrict__ part_ml,
-                                                               const int* __restrict__ decode_tokens,
+                                                               const int4* __restrict__ decode_rows,
                                                                bf16* __restrict__ out, int nh,
                                                                int splits) {
     const int di = blockIdx.x, h = blockIdx.y;
-    const int t = decode_tokens[di];
+    const int t = decode_rows[di].x;
     join_shares<D>(part_o, part_ml, ((size_t)di * nh + h) * splits, splits, out + ((size_t)t * nh + h) * D);
 }
 
@@ -1008,8 +1024,8 @@ static thread_local int g_decode_waves = 0;   // 0: by the launch's shape
 
 template <int D>
 static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* out,
-                         float* part_o, float* part_ml, const int* decode_tokens, const int* tok_req,
-                         const int* positions, const int* table, int max_blocks, int ND, int nh,
+                         float* part_o, float* part_ml, const int4* decode_rows,
+                         const int* table, int max_blocks, int ND, int nh,
                          int nkv, float scale_log2, int window, int splits, bool even_lengths,
                          DecodePrologue pro, hipStream_t s) {
     dim3 grid(splits, nkv, ND);
@@ -1036,16 +1052,16 @@ static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* 
                       : (splits == 2 && workgroups > 2ll * device_cus()) ? 8 : 4;
     if (waves == 8)
         attn_decode_kernel<D, 8><<<grid, 512, 0, s>>>(qkv, q_stride, k, v, out, part_o, part_ml,
-                                                      decode_tokens, tok_req, positions, table, max_blocks,
+                                                      decode_rows, table, max_blocks,
                                                       nh, nkv, scale_log2, window, splits, pro);
     else
         attn_decode_kernel<D, 4><<<grid, 256, 0, s>>>(qkv, q_stride, k, v, out, part_o, part_ml,
-                                                      decode_tokens, tok_req, positions, table, max_blocks,
+                                                      decode_rows, table, max_blocks,
                                                       nh, nkv, scale_log2, window, splits, pro);
     LC_LAUNCH_CHECK("attn_decode");
     if (splits > 1) {
         attn_decode_join_kernel<D><<<dim3(ND, nh), 128, 0, s>>>(
-            part_o, part_ml, decode_tokens, out, nh, splits);
+            part_o, part_ml, decode_rows, out, nh, splits);
         LC_LAUNCH_CHECK("attn_decode_join");
     }
     return 0;
@@ -1193,8 +1209,8 @@ LC_API int lc_attn_decode_takes_shares(int d, int rot) { return d == 128 && (rot
 // (q_w, k_w, rope_table may be null; rot entries of a head rotate) and, if write_kv != 0, writes
 // the tokens' k and v to the cache.  Otherwise qkv is ready and the cache holds the tokens.
 LC_API int lc_attn_decode_bf16(const void* qkv, int q_stride, void* k_cache, void* v_cache,
-                               void* out, float* part_o, float* part_ml, const int* decode_tokens,
-                               const int* tok_req, const int* positions, const int* block_table,
+                               void* out, float* part_o, float* part_ml, const int* decode_rows,
+                               const int* block_table,
                                int max_blocks, int num_decode, int nh, int nkv, int d, int page_size,
                                float scale, int window, int splits, int even_lengths, int prologue, const float* q_w,
                                const float* k_w, float eps, const float* rope_table, int rot,
@@ -1213,14 +1229,15 @@ LC_API int lc_attn_decode_bf16(const void* qkv, int q_stride, void* k_cache, voi
     LC_CHECK(!qkv_shares || (num_shares >= 1 && share_rows >= 1 && q_stride % 4 == 0 && (uintptr_t)qkv_shares % 16 == 0),
              "attn_decode_bf16: bad shares (%d of %d rows)", num_shares, share_rows);
     if (qkv_shares && !qkv) qkv = qkv_shares;      // never read, but not null
-    LC_CHECK(qkv && k_cache && v_cache && out && decode_tokens && tok_req && positions && block_table,
+    LC_CHECK(qkv && k_cache && v_cache && out && decode_rows && block_table,
              "attn_decode_bf16: null pointer");
+    LC_CHECK((uintptr_t)decode_rows % 16 == 0, "attn_decode_bf16: the decode rows must be 16-byte aligned");
     LC_CHECK(splits >= 1 && splits <= 65535 && (splits == 1 || (part_o && part_ml)),
              "attn_decode_bf16: %d shares need a workspace", splits);
     LC_CHECK(q_stride % 8 == 0 && (uintptr_t)qkv % 16 == 0, "attn_decode_bf16: q must be 16-byte aligned");
     const float sl2 = scale * 1.4426950408889634f;
 #define CALL(DD) launch_decode<DD>((const bf16*)qkv, q_stride, (bf16*)k_cache, (bf16*)v_cache,             \
-        (bf16*)out, part_o, part_ml, decode_tokens, tok_req, positions, block_table, max_blocks,           \
+        (bf16*)out, part_o, part_ml, (const int4*)decode_rows, block_table, max_blocks,                     \
         num_decode, nh, nkv, sl2, window, splits, even_lengths != 0, pro, stream)
     LC_DISPATCH_D(d, CALL)
 #undef CALL

@@ -102,30 +102,50 @@ __device__ __forceinline__ float row16_sum(float v, int j) {
     return v;
 }
 
-// x: the lane's 8 entries (raw).  w: the norm's 128 weights or null.  cs: the position's row of
-// the rotary table (64 cosines, then 64 sines) or null.  Entry i pairs with entry i + 64.
-__device__ __forceinline__ head_chunk head128_norm_rope(head_chunk x, int j, const float* __restrict__ w,
-                                                        float eps, const float* __restrict__ cs) {
+// What head128_norm_rope needs beside the raw entries, for the lane that holds entries 8 j to
+// 8 j + 7 of a head of 128: the norm's weights there (w: all 128, or null) and the cosines and sines
+// of the entries' pairs (cs: the position's row of the rotary table, 64 cosines, then 64 sines, or
+// null).  A function of its own so that a caller can ask for them before the raw entries are there.
+struct Head128Constants {
+    float w[8], c[8], s[8];
+    bool normed, rotated;
+};
+__device__ __forceinline__ Head128Constants head128_constants(int j, const float* __restrict__ w,
+                                                              const float* __restrict__ cs) {
+    Head128Constants k;
+    k.normed = w != nullptr;
+    k.rotated = cs != nullptr;
+    const int i0 = 8 * (j & 7);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        k.w[e] = w ? w[8 * j + e] : 1.f;
+        k.c[e] = cs ? cs[i0 + e] : 1.f;
+        k.s[e] = cs ? cs[64 + i0 + e] : 0.f;
+    }
+    return k;
+}
+
+// x: the lane's 8 entries (raw).  Entry i pairs with entry i + 64.
+__device__ __forceinline__ head_chunk head128_norm_rope(head_chunk x, int j, const Head128Constants& k,
+                                                        float eps) {
     float f[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) f[e] = static_cast<float>(x[e]);
-    if (w) {
+    if (k.normed) {
         float ss = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) ss = __fmaf_rn(f[e], f[e], ss);
         ss = row16_sum(ss, j);
         const float inv = rsqrtf(ss / 128.f + eps);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) f[e] = __fmul_rn(__fmul_rn(f[e], inv), w[8 * j + e]);
+        for (int e = 0; e < 8; ++e) f[e] = __fmul_rn(__fmul_rn(f[e], inv), k.w[e]);
     }
-    if (cs) {
-        const int i0 = 8 * (j & 7);
+    if (k.rotated) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const float other = row_move<0x128>(f[e]);        // the partner entry, 64 further on or back
-            const float c = cs[i0 + e], sn = cs[64 + i0 + e];
             // first half: a c - b s (a own, b partner); second half: a s + b c (b own, a partner)
-            const float own_c = __fmul_rn(f[e], c), other_s = __fmul_rn(other, sn);
+            const float own_c = __fmul_rn(f[e], k.c[e]), other_s = __fmul_rn(other, k.s[e]);
             f[e] = (j < 8) ? __fsub_rn(own_c, other_s) : __fadd_rn(other_s, own_c);
         }
     }
@@ -133,6 +153,12 @@ __device__ __forceinline__ head_chunk head128_norm_rope(head_chunk x, int j, con
 #pragma unroll
     for (int e = 0; e < 8; ++e) out[e] = static_cast<bf16>(f[e]);
     return out;
+}
+
+// The same with the weights (or null) and the table's row (or null) where they lie.
+__device__ __forceinline__ head_chunk head128_norm_rope(head_chunk x, int j, const float* __restrict__ w,
+                                                        float eps, const float* __restrict__ cs) {
+    return head128_norm_rope(x, j, head128_constants(j, w, cs), eps);
 }
 
 // Compute units of the GPU.  They only steer how work is laid over the device (tile plans, the

@@ -54,7 +54,7 @@ _SIGNATURES = {
     "lc_attn_decode_splits": "iii",
     "lc_attn_decode_waves": "i",
     "lc_attn_decode_force_splits": "i",
-    "lc_attn_decode_bf16": "pippppppppp" + "iiiiii" + "f" + "iii" + "ippfpii" + "pii" + "p",
+    "lc_attn_decode_bf16": "pippppppp" + "iiiiii" + "f" + "iii" + "ippfpii" + "pii" + "p",
     "lc_attn_decode_takes_shares": "ii",
     "lc_gemm_bf16_sum_shares": "ppiiiip",
     "lc_attn_prefill_bf16": "pippppp" + "iiiiii" + "f" + "i" + "ipfpi" + "ipp" + "p",
@@ -545,7 +545,7 @@ class AttentionBatch:
     ctx_len: Optional[torch.Tensor] = None
     slots: Optional[torch.Tensor] = None
     num_decode: int = 0
-    decode_tokens: Optional[torch.Tensor] = None   # [ND] token rows of length-1 portions
+    decode_rows: Optional[torch.Tensor] = None     # [ND, 4] of the length-1 portions: token row, request, position, 0
     prefill_tiles: Optional[torch.Tensor] = None   # [NT, 4]: request, first token row, rows, first position
     max_ctx: int = 0                               # longest cached length in the batch
     all_decode: bool = False
@@ -558,19 +558,19 @@ ATTENTION_PLAN = "paged_attention"
 
 def plan_attention(layout):
     """The work lists of the attention kernels for one step's batch (a planner in the sense of
-    ``Part.batch_planner``): the token rows of the portions of length one, which the decode
-    kernel serves, and the tiles of up to PREFILL_TILE query rows that the longer portions are
+    ``Part.batch_planner``): the portions of length one, which the decode kernel serves, four
+    numbers each (token row, request, position, 0: all a workgroup needs to know of its token in
+    one load, not one look-up after the other), and the tiles of up to PREFILL_TILE query rows that the longer portions are
     cut into, four numbers each (request, first token row, rows, first position).  The tiles
     that see the most keys come first: the kernel's workgroups start in this order, and whoever
     is done takes the longest that is left (the order changes no tile's result).  The decoding
     rows likewise come longest request first."""
     R, q_start, first = layout.num_requests, layout.q_start, layout.first_position
     if layout.single:
-        decode = np.arange(R, dtype=np.int32)
+        singles = np.arange(R, dtype=np.int64)
         tiles = np.zeros((0, 4), dtype=np.int32)
     else:
-        decode = np.asarray([q_start[r] for r in range(R) if q_start[r + 1] - q_start[r] == 1],
-                            dtype=np.int32)
+        singles = np.asarray([r for r in range(R) if q_start[r + 1] - q_start[r] == 1], dtype=np.int64)
         tile_list = []
         for r in range(R):
             n = q_start[r + 1] - q_start[r]
@@ -582,17 +582,19 @@ def plan_attention(layout):
         tiles = np.asarray(tile_list, dtype=np.int32).reshape(-1, 4)
     # lengths after this step of the requests that decode: a hint for the decode kernel (how
     # it lays its work out, never what it computes); a captured step keeps the hint of its capture
-    lengths = np.asarray(first, dtype=np.int64) + 1
-    if not layout.single:
-        lengths = lengths[np.diff(np.asarray(q_start, dtype=np.int64)) == 1]
+    lengths = np.asarray(first, dtype=np.int64)[singles] + 1
+    decode = np.zeros((singles.size, 4), dtype=np.int32)
+    decode[:, 0] = np.asarray(q_start, dtype=np.int64)[singles]
+    decode[:, 1] = singles
+    decode[:, 2] = lengths - 1
     even = bool(lengths.size) and int(lengths.max()) * int(lengths.size) <= 1.1 * int(lengths.sum())
     if lengths.size > 1 and int(lengths.max()) != int(lengths.min()):
         # the decode kernel's workgroups start in the order of this list: the longest requests first,
         # so that none of them starts late and runs on alone at the end (64 requests of 16 to 2,200
         # tokens: 58 instead of 70 us a layer; the order changes no token's result)
         decode = decode[np.argsort(-lengths, kind="stable")]
-    return ({"decode_tokens": decode, "prefill_tiles": tiles},
-            {"num_decode": int(decode.size), "all_decode": int(decode.size) == R, "even_lengths": even})
+    return ({"decode_rows": decode, "prefill_tiles": tiles},
+            {"num_decode": int(singles.size), "all_decode": int(singles.size) == R, "even_lengths": even})
 
 
 # Tokens of a cache page as the matrix-core attention kernels index it: a page of a multiple of
@@ -618,7 +620,7 @@ def attention_batch(batch, pages, plan=None) -> AttentionBatch:
                               block_table=pages.block_table, q_start=batch.q_offsets,
                               ctx_len=batch.ctx_len, slots=pages.slots, max_ctx=batch.max_ctx)
         if plan is not None:
-            done = replace(done, decode_tokens=plan.arrays["decode_tokens"],
+            done = replace(done, decode_rows=plan.arrays["decode_rows"],
                            prefill_tiles=plan.arrays["prefill_tiles"],
                            num_decode=plan.info["num_decode"], all_decode=plan.info["all_decode"],
                            even_lengths=plan.info["even_lengths"])
@@ -645,7 +647,7 @@ def attention_takes_shares(batch: AttentionBatch, T: int, nh: int, nkv: int, d: 
     single tokens in bfloat16, whose decode kernel prepares whole heads of 128 itself and sums
     the shares as it reads them."""
     lib = library()
-    return bool(dtype == torch.bfloat16 and batch.decode_tokens is not None
+    return bool(dtype == torch.bfloat16 and batch.decode_rows is not None
                 and batch.prefill_tiles is not None and batch.num_decode == T and T > 0
                 and lib.lc_attn_bf16_supported(nh, nkv, d, page_size)
                 and lib.lc_attn_decode_takes_shares(d, rot))
@@ -682,7 +684,7 @@ def attention(qkv, batch: AttentionBatch, k_cache: torch.Tensor,
     _need(batch.block_table, "block table", torch.int32, 2)
     _check_caches(k_cache, v_cache, nkv, page_size, d)
     lib = library()
-    fast = (qkv.dtype == torch.bfloat16 and batch.decode_tokens is not None
+    fast = (qkv.dtype == torch.bfloat16 and batch.decode_rows is not None
             and batch.prefill_tiles is not None and lib.lc_attn_bf16_supported(nh, nkv, d, page_size))
     if qkv.dtype == torch.bfloat16 and not fast:
         _say_once(("attention", nh, nkv, d, page_size),
@@ -715,8 +717,8 @@ def attention(qkv, batch: AttentionBatch, k_cache: torch.Tensor,
                 part_o = torch.empty((nd * nh * splits * d,), dtype=torch.float32, device=qkv.device)
                 part_ml = torch.empty((nd * nh * splits * 2,), dtype=torch.float32, device=qkv.device)
             _call("lc_attn_decode_bf16", _ptr(qkv if shares is None else None), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
-                  _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(batch.decode_tokens),
-                  _ptr(batch.tok_req), _ptr(batch.positions), _ptr(batch.block_table), mb, nd, nh,
+                  _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(batch.decode_rows),
+                  _ptr(batch.block_table), mb, nd, nh,
                   nkv, d, page_size, scale, window, splits, 1 if batch.even_lengths else 0,
                   1 if in_kernel else 0,
                   _ptr(prologue.q_weight if in_kernel else None),

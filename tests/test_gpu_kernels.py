@@ -159,7 +159,7 @@ def paged_case(lengths, new, nh, nkv, d, page, dtype, seed, spare=3):
         q_start.append(q_start[-1] + k)
     T = len(tok_req)
     qkv = rnd(T, (nh + 2 * nkv) * d, dtype=dtype, seed=seed + 3)
-    dec = [q_start[r] for r in range(R) if new[r] == 1]
+    dec = [[q_start[r], r, lengths[r] - 1, 0] for r in range(R) if new[r] == 1]
     tiles = []
     for r in range(R):
         if new[r] > 1:
@@ -168,7 +168,7 @@ def paged_case(lengths, new, nh, nkv, d, page, dtype, seed, spare=3):
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
     batch = AttentionBatch(tok_req=i32(tok_req), positions=i32(positions), block_table=table.to(DEV),
                            q_start=i32(q_start), ctx_len=i32(lengths), num_decode=len(dec),
-                           decode_tokens=i32(dec), prefill_tiles=i32(tiles).view(-1, 4),
+                           decode_rows=i32(dec).view(-1, 4), prefill_tiles=i32(tiles).view(-1, 4),
                            max_ctx=max(lengths), all_decode=len(dec) == R)
     return qkv, batch, kc, vc
 
