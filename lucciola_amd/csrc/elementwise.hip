@@ -130,26 +130,41 @@ __global__ __launch_bounds__(THREADS) void rmsnorm_vec_kernel(
     const T* dr = (delta && !shares) ? delta + (size_t)src * n : nullptr;
     const float* pr = shares ? reinterpret_cast<const float*>(delta) + (size_t)src * n : nullptr;
     const int chunks = n / 8;
-    Pack8<float> hv[CHUNKS];
+    Pack8<float> hv[CHUNKS], wv[CHUNKS];
     Pack8<T> dv[CHUNKS];
+    // everything the row needs is asked for at once, the weights too: one trip to memory
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
         const int chunk = threadIdx.x + c * THREADS;
         if (chunk < chunks) {
             hv[c] = *reinterpret_cast<const Pack8<float>*>(hr + chunk * 8);
             if (dr) dv[c] = *reinterpret_cast<const Pack8<T>*>(dr + chunk * 8);
+            wv[c] = *reinterpret_cast<const Pack8<float>*>(w + chunk * 8);
         }
     }
     if (pr) {   // the shares of the branch's product, in their order, then the stream
+        // up to AT_ONCE shares are asked for together and added in their order once they are
+        // back (a share past the last is the last one again, loaded and not added): a loop
+        // that adds each share as it arrives makes one trip to memory per share
+        constexpr int AT_ONCE = CHUNKS == 1 ? 8 : 4;
 #pragma unroll
         for (int c = 0; c < CHUNKS; ++c) {
             const int chunk = threadIdx.x + c * THREADS;
             if (chunk < chunks) {
                 Pack8<float> sum = *reinterpret_cast<const Pack8<float>*>(pr + chunk * 8);
-                for (int s = 1; s < shares; ++s) {
-                    const Pack8<float> part = *reinterpret_cast<const Pack8<float>*>(pr + s * share_stride + chunk * 8);
+                for (int s0 = 1; s0 < shares; s0 += AT_ONCE) {
+                    Pack8<float> part[AT_ONCE];
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) sum.set(i, sum.get(i) + part.get(i));
+                    for (int a = 0; a < AT_ONCE; ++a)
+                        part[a] = *reinterpret_cast<const Pack8<float>*>(
+                            pr + (size_t)min(s0 + a, shares - 1) * share_stride + chunk * 8);
+#pragma unroll
+                    for (int a = 0; a < AT_ONCE; ++a) {
+                        if (s0 + a < shares) {
+#pragma unroll
+                            for (int i = 0; i < 8; ++i) sum.set(i, sum.get(i) + part[a].get(i));
+                        }
+                    }
                 }
 #pragma unroll
                 for (int i = 0; i < 8; ++i) hv[c].set(i, hv[c].get(i) + sum.get(i));
@@ -179,10 +194,9 @@ __global__ __launch_bounds__(THREADS) void rmsnorm_vec_kernel(
     for (int c = 0; c < CHUNKS; ++c) {
         const int chunk = threadIdx.x + c * THREADS;
         if (chunk < chunks) {
-            const Pack8<float> wv = *reinterpret_cast<const Pack8<float>*>(w + chunk * 8);
             Pack8<T> ov;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) ov.set(i, hv[c].get(i) * inv * wv.get(i));
+            for (int i = 0; i < 8; ++i) ov.set(i, hv[c].get(i) * inv * wv[c].get(i));
             *reinterpret_cast<Pack8<T>*>(o + chunk * 8) = ov;
         }
     }
