@@ -1235,6 +1235,8 @@ LC_API int lc_attn_decode_bf16(const void* qkv, int q_stride, void* k_cache, voi
     LC_CHECK(splits >= 1 && splits <= 65535 && (splits == 1 || (part_o && part_ml)),
              "attn_decode_bf16: %d shares need a workspace", splits);
     LC_CHECK(q_stride % 8 == 0 && (uintptr_t)qkv % 16 == 0, "attn_decode_bf16: q must be 16-byte aligned");
+    LC_CHECK(!prologue || ((uintptr_t)q_w % 16 == 0 && (uintptr_t)k_w % 16 == 0 && (uintptr_t)rope_table % 16 == 0),
+             "attn_decode_bf16: the norms' weights and the rotary table must be 16-byte aligned");
     const float sl2 = scale * 1.4426950408889634f;
 #define CALL(DD) launch_decode<DD>((const bf16*)qkv, q_stride, (bf16*)k_cache, (bf16*)v_cache,             \
         (bf16*)out, part_o, part_ml, (const int4*)decode_rows, block_table, max_blocks,                     \

@@ -105,7 +105,8 @@ __device__ __forceinline__ float row16_sum(float v, int j) {
 // What head128_norm_rope needs beside the raw entries, for the lane that holds entries 8 j to
 // 8 j + 7 of a head of 128: the norm's weights there (w: all 128, or null) and the cosines and sines
 // of the entries' pairs (cs: the position's row of the rotary table, 64 cosines, then 64 sines, or
-// null).  A function of its own so that a caller can ask for them before the raw entries are there.
+// null), both 16-byte aligned.  A function of its own so that a caller can ask for them before the
+// raw entries are there.
 struct Head128Constants {
     float w[8], c[8], s[8];
     bool normed, rotated;
@@ -115,12 +116,25 @@ __device__ __forceinline__ Head128Constants head128_constants(int j, const float
     Head128Constants k;
     k.normed = w != nullptr;
     k.rotated = cs != nullptr;
+    // w and cs are 16-byte aligned: four entries a load
+    typedef float float4v __attribute__((ext_vector_type(4)));
     const int i0 = 8 * (j & 7);
+    float4v w0 = {1.f, 1.f, 1.f, 1.f}, w1 = w0, c0 = w0, c1 = w0, s0 = {0.f, 0.f, 0.f, 0.f}, s1 = s0;
+    if (w) {
+        w0 = *reinterpret_cast<const float4v*>(w + 8 * j);
+        w1 = *reinterpret_cast<const float4v*>(w + 8 * j + 4);
+    }
+    if (cs) {
+        c0 = *reinterpret_cast<const float4v*>(cs + i0);
+        c1 = *reinterpret_cast<const float4v*>(cs + i0 + 4);
+        s0 = *reinterpret_cast<const float4v*>(cs + 64 + i0);
+        s1 = *reinterpret_cast<const float4v*>(cs + 64 + i0 + 4);
+    }
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        k.w[e] = w ? w[8 * j + e] : 1.f;
-        k.c[e] = cs ? cs[i0 + e] : 1.f;
-        k.s[e] = cs ? cs[64 + i0 + e] : 0.f;
+    for (int e = 0; e < 4; ++e) {
+        k.w[e] = w0[e]; k.w[4 + e] = w1[e];
+        k.c[e] = c0[e]; k.c[4 + e] = c1[e];
+        k.s[e] = s0[e]; k.s[4 + e] = s1[e];
     }
     return k;
 }

@@ -499,7 +499,8 @@ LC_API int lc_qk_norm_rope_write(void* qkv, int dt, int T, int nh, int nkv, int 
              "qk_norm_rope_write: cache write needs v_cache and a page size");
     if (!rope_table) rot = 0;
     if (dt == DT_BF16 && d == 128 && (rot == 0 || rot == 128) && (q_w == nullptr) == (k_w == nullptr) &&
-        (uintptr_t)qkv % 16 == 0 && (uintptr_t)k_cache % 16 == 0) {
+        (uintptr_t)qkv % 16 == 0 && (uintptr_t)k_cache % 16 == 0 && (uintptr_t)q_w % 16 == 0 &&
+        (uintptr_t)k_w % 16 == 0 && (uintptr_t)rope_table % 16 == 0) {
         if (first_head == nh && k_cache && slots) {
             kv_norm_rope_write128_kernel<<<dim3((T + 15) / 16, nkv), 256, 0, stream>>>(
                 (bf16*)qkv, T, nh, nkv, k_w, eps, positions, rope_table, (bf16*)k_cache, (bf16*)v_cache,
