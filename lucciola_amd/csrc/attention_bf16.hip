@@ -172,6 +172,81 @@ __device__ __forceinline__ void attend_range(AttnState<D, QT>& st, const bf16x8 
     }
 }
 
+// The same walk with two pages in flight beside the one being multiplied, for the decode kernel:
+// where a request's pages are one workgroup's alone (requests of unequal length, whose long ones
+// run on at the end) a wave's pace is what it keeps in flight.  The compiler counts the loads it
+// knows of and, across a loop's back edge, waits for all of them; so a page's loads are inline
+// assembly that it does not count, the waits are counted here, and three sets of page registers
+// take turns, unrolled, so that no set is ever copied.  A set is written by the hardware long
+// after the statement that names it: nothing may touch it between its loads and the counted wait
+// that is followed by page_landed (a spilled set would store what the registers held before;
+// the library asks its compiled kernels for their scratch size and takes the walk above if there
+// is any).  The page numbers come through scalar loads (their addresses are the same for the whole wave),
+// which the counter of the vector loads does not see.
+template <int D>
+__device__ __forceinline__ void load_page_uncounted(PageRegs<D>& r, const bf16* k_cache, const bf16* v_cache,
+                                                    int page, int nkv, int kvh, int lane) {
+    const size_t head = (size_t)page * nkv + kvh;
+    const bf16* kb = k_cache + (head * PAGE + (lane & 15)) * D + (lane >> 4) * 8;
+    const bf16* vb = v_cache + (head * D + (lane & 15)) * PAGE + (lane >> 4) * 4;
+#pragma unroll
+    for (int i = 0; i < D / 32; ++i)
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r.k[i]) : "v"(kb + i * 32) : "memory");
+#pragma unroll
+    for (int i = 0; i < D / 16; ++i)
+        asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(r.v[i]) : "v"(vb + i * 16 * PAGE) : "memory");
+}
+template <int D>
+__device__ __forceinline__ void page_landed(PageRegs<D>& r) {
+#pragma unroll
+    for (int i = 0; i < D / 32; ++i) asm volatile("" : "+v"(r.k[i]));
+#pragma unroll
+    for (int i = 0; i < D / 16; ++i) asm volatile("" : "+v"(r.v[i]));
+}
+
+// p0: the first page's registers; if first_loaded, the caller has asked for the page already, with
+// ordinary loads (they stay in flight across code of the caller's that the compiler is free to
+// arrange).  They are waited for here before the first uncounted load is issued, so that from
+// then on the compiler knows of no load in flight and adds no wait of its own to the loop.
+template <int D, int QT>
+__device__ __forceinline__ void attend_range_deep(AttnState<D, QT>& st, const bf16x8 (&bq)[QT][D / 32],
+                                                  const bf16* k_cache, const bf16* v_cache,
+                                                  const int* __restrict__ table, int begin, int end,
+                                                  int step, int nkv, int kvh, const int (&lo)[QT],
+                                                  const int (&hi)[QT], float scale_log2, int lane,
+                                                  PageRegs<D>& p0, bool first_loaded) {
+    if (begin >= end) return;
+    constexpr int LOADS = D / 32 + D / 16;            // of one page
+    static_assert(2 * LOADS <= 63, "the counter of loads in flight has six bits");
+    const int count = (end - begin + step - 1) / step;
+    PageRegs<D> p1, p2;
+    const int second = count > 1 ? table[begin + step] : 0;
+    int ahead = count > 2 ? table[begin + 2 * step] : 0;      // the page of the next loads
+    if (!first_loaded) load_page<D>(p0, k_cache, v_cache, table[begin], nkv, kvh, lane);
+    wait_vmcnt<0>();
+    page_landed<D>(p0);
+    if (count > 1) load_page_uncounted<D>(p1, k_cache, v_cache, second, nkv, kvh, lane);
+    // page i, in `cur`; the loads of page i + 2 go into `third`, which page i - 1 has left
+    auto turn = [&](PageRegs<D>& cur, PageRegs<D>& third, int i) {
+        if (i + 2 < count) {
+            load_page_uncounted<D>(third, k_cache, v_cache, ahead, nkv, kvh, lane);
+            if (i + 3 < count) ahead = table[begin + (i + 3) * step];
+            wait_vmcnt<2 * LOADS>();
+        } else if (i + 1 < count) {
+            wait_vmcnt<LOADS>();
+        } else {
+            wait_vmcnt<0>();
+        }
+        page_landed<D>(cur);
+        attend_page<D, QT>(st, cur, bq, (begin + i * step) * PAGE, lo, hi, scale_log2, lane);
+    };
+    for (int i = 0; i < count; i += 3) {
+        turn(p0, p2, i);
+        if (i + 1 < count) turn(p1, p0, i + 1);
+        if (i + 2 < count) turn(p2, p1, i + 2);
+    }
+}
+
 // ------------------------------------------------------------------------------- decode
 // What an attention kernel does to the raw q (the decode kernel also: k, v) of its tokens before
 // it attends, when the step has no separate kernel for it: RMSNorm over the head (weights optional), rotary
@@ -199,7 +274,8 @@ struct DecodePrologue {
 // cache before anyone in the workgroup reads that page.
 // NW waves take the pages of the workgroup's share in turn, each with one page in flight beside
 // the one it works on: a workgroup draws on memory at NW times a wave's pace.
-template <int D, int NW>
+// DEEP: the walk with two pages in flight (attend_range_deep).
+template <int D, int NW, bool DEEP>
 __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
     const bf16* __restrict__ qkv, int q_stride, bf16* k_cache, bf16* v_cache,
     bf16* __restrict__ out, float* __restrict__ part_o,
@@ -212,7 +288,8 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
     __shared__ __attribute__((aligned(16))) bf16 sm_q[16 * D];
 
     const int split = blockIdx.x, kvh = blockIdx.y, di = blockIdx.z;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // the same for the whole wave: its page numbers are scalar loads
     const int q = lane & 15, kg = lane >> 4;
     // the token's row in the batch, its request's row of the block table and its position come
     // in one load: every look-up that hangs on another is a trip to memory before the first key
@@ -347,8 +424,12 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
     AttnState<D, 1> st;
     init_state<D, 1>(st);
     const int lo[1] = {j_lo}, hi[1] = {p};
-    attend_range<D, 1>(st, bq, k_cache, v_cache, table, begin + wave, end, NW, nkv, kvh, lo, hi,
-                       scale_log2, lane, first_pages, first, early);
+    if (DEEP)
+        attend_range_deep<D, 1>(st, bq, k_cache, v_cache, table, begin + wave, end, NW, nkv, kvh, lo, hi,
+                                scale_log2, lane, first, early);
+    else
+        attend_range<D, 1>(st, bq, k_cache, v_cache, table, begin + wave, end, NW, nkv, kvh, lo, hi,
+                           scale_log2, lane, first_pages, first, early);
 
     // the waves' results meet in LDS
     float l = st.l[0];
@@ -1021,6 +1102,22 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_wide_kernel(
 }
 
 static thread_local int g_decode_waves = 0;   // 0: by the launch's shape
+static thread_local int g_decode_deep = 1;    // 0: never the walk with two pages in flight (tests, tuning)
+
+// Whether the decode kernel that walks with two pages in flight keeps its page registers in
+// registers: 1 yes, 0 it spills (its uncounted loads would not be safe), -1 could not ask.
+template <int D>
+static int decode_deep_state() {
+    static const int state = [] {
+        hipFuncAttributes attr;
+        if (hipFuncGetAttributes(&attr, (const void*)attn_decode_kernel<D, 4, true>) != hipSuccess) {
+            (void)hipGetLastError();
+            return -1;
+        }
+        return attr.localSizeBytes != 0 ? 0 : 1;
+    }();
+    return state;
+}
 
 template <int D>
 static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* out,
@@ -1050,14 +1147,22 @@ static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* 
                       : (splits == 1 && max_blocks >= 32 && workgroups < 4ll * device_cus() && alone_at_the_end) ? 8
                       : (splits > 1 && workgroups <= device_cus()) ? 8
                       : (splits == 2 && workgroups > 2ll * device_cus()) ? 8 : 4;
-    if (waves == 8)
-        attn_decode_kernel<D, 8><<<grid, 512, 0, s>>>(qkv, q_stride, k, v, out, part_o, part_ml,
-                                                      decode_rows, table, max_blocks,
-                                                      nh, nkv, scale_log2, window, splits, pro);
-    else
-        attn_decode_kernel<D, 4><<<grid, 256, 0, s>>>(qkv, q_stride, k, v, out, part_o, part_ml,
-                                                      decode_rows, table, max_blocks,
-                                                      nh, nkv, scale_log2, window, splits, pro);
+    // Two pages in flight beside the one being multiplied where the workgroups have four waves (many
+    // workgroups, or whole requests of even lengths): with cold caches 64 requests of 8,192 tokens
+    // 375 -> 359 us (6.0 TB/s), of 1,024 tokens 55.1 -> 53.1, 256 of 1,024 210.8 -> 208.1.  Not with
+    // eight waves: their launches are short shares or requests of unequal length, whose long ones run
+    // on alone at the end at the pace at which a wave works through a page (about 1.5 us, two waves
+    // a SIMD), not at what it has in flight (one request of 8,192 tokens among 63 of 512: 103.9 us
+    // with one page ahead, 108.5 with two; 16 requests of 100 to 8,000: 58.3 and 60.3).
+    const bool deep = waves == 4 && g_decode_deep && decode_deep_state<D>() == 1;
+#define LC_DECODE(NW, DEEP)                                                                             \
+    attn_decode_kernel<D, NW, DEEP><<<grid, 64 * NW, 0, s>>>(qkv, q_stride, k, v, out, part_o, part_ml, \
+                                                             decode_rows, table, max_blocks, nh, nkv,   \
+                                                             scale_log2, window, splits, pro)
+    if (waves == 8) LC_DECODE(8, false);
+    else if (deep) LC_DECODE(4, true);
+    else LC_DECODE(4, false);
+#undef LC_DECODE
     LC_LAUNCH_CHECK("attn_decode");
     if (splits > 1) {
         attn_decode_join_kernel<D><<<dim3(ND, nh), 128, 0, s>>>(
@@ -1134,6 +1239,26 @@ LC_API int lc_attn_prefill_wide(int on) {
 }
 
 // Waves of a decode workgroup (4 or 8; 0: chosen by the launch's shape).  For tests and tuning.
+// 0: the decode kernel walks its pages with one page in flight beside the one it multiplies, 1
+// (the default): with two where its workgroups have four waves and the kernel keeps its registers.
+// Returns the setting before.
+LC_API int lc_attn_decode_deep(int on) {
+    const int before = g_decode_deep;
+    g_decode_deep = on ? 1 : 0;
+    return before;
+}
+// Whether the kernels of heads of d walk with two pages in flight when the switch is on (1), or
+// cannot (0: a page register spills; -1: the runtime could not be asked; -2: no such head size).
+LC_API int lc_attn_decode_deep_ok(int d) {
+    switch (d) {
+        case 32: return decode_deep_state<32>();
+        case 64: return decode_deep_state<64>();
+        case 96: return decode_deep_state<96>();
+        case 128: return decode_deep_state<128>();
+        default: return -2;
+    }
+}
+
 LC_API int lc_attn_decode_waves(int waves) {
     LC_CHECK(waves == 0 || waves == 4 || waves == 8, "attn_decode: %d waves (0, 4 or 8)", waves);
     g_decode_waves = waves;

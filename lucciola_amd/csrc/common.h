@@ -175,6 +175,15 @@ __device__ __forceinline__ head_chunk head128_norm_rope(head_chunk x, int j, con
     return head128_norm_rope(x, j, head128_constants(j, w, cs), eps);
 }
 
+// Waits with a count of the wave's own: at most N of its youngest memory loads (vmcnt), or LDS and
+// scalar-memory operations (lgkmcnt), may still be in flight; the other counters are left alone.
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));
+}
+template <int N> __device__ __forceinline__ void wait_lgkmcnt() {
+    __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));
+}
+
 // Compute units of the GPU.  They only steer how work is laid over the device (tile plans, the
 // number of shares); no result depends on them.
 int device_cus();

@@ -55,13 +55,6 @@ __device__ __forceinline__ float swiglu_f(float g, float u) {
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef __attribute__((address_space(1))) const void* glb_ptr_t;
 
-template <int N> __device__ __forceinline__ void wait_vmcnt() {
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));   // other counters untouched
-}
-template <int N> __device__ __forceinline__ void wait_lgkmcnt() {
-    __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));
-}
-
 // ------------------------------------------------------------------------------- skinny
 constexpr int SK_KBLOCK = 128; // k elements per wave iteration
 

@@ -53,6 +53,8 @@ _SIGNATURES = {
     "lc_gemm_bf16_runs_ring_ok": "",
     "lc_attn_decode_splits": "iii",
     "lc_attn_decode_waves": "i",
+    "lc_attn_decode_deep": "i",
+    "lc_attn_decode_deep_ok": "i",
     "lc_attn_decode_force_splits": "i",
     "lc_attn_decode_bf16": "pippppppp" + "iiiiii" + "f" + "iii" + "ippfpii" + "pii" + "p",
     "lc_attn_decode_takes_shares": "ii",

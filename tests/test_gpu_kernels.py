@@ -521,18 +521,21 @@ def test_attention_prefill_of_heads_of_128_in_pairs(nh, nkv, window):
 @pytest.mark.parametrize("nh,nkv,d,window,rot,normed", [(32, 8, 128, 0, 128, True), (6, 2, 96, 24, 96, True),
                                                         (8, 1, 64, 0, 32, False), (4, 4, 32, 0, 0, True),
                                                         (16, 1, 32, 0, 32, True)])
-@pytest.mark.parametrize("waves", [0, 4, 8])
-def test_attention_decode_with_prologue_in_the_kernel(nh, nkv, d, window, rot, normed, waves):
+@pytest.mark.parametrize("waves,deep", [(0, 1), (4, 1), (4, 0), (8, 1)])
+def test_attention_decode_with_prologue_in_the_kernel(nh, nkv, d, window, rot, normed, waves, deep):
     """A step of single tokens with raw q, k, v: the decode kernel norms, rotates and writes
     the cache itself.  Output and cache must equal those of the separate kernel followed by
     the plain decode kernel, for short and long contexts (one or many shares of the pages),
     a token at a page's first and last place, part of the head rotated or none; with workgroups
-    of four and of eight waves."""
-    ops.library().lc_attn_decode_waves(waves)
+    of four and of eight waves, the four-wave ones with two pages in flight and with one."""
+    lib = ops.library()
+    lib.lc_attn_decode_waves(waves)
+    lib.lc_attn_decode_deep(deep)
     try:
         decode_prologue_case(nh, nkv, d, window, rot, normed)
     finally:
-        ops.library().lc_attn_decode_waves(0)
+        lib.lc_attn_decode_waves(0)
+        lib.lc_attn_decode_deep(1)
 
 
 def decode_prologue_case(nh, nkv, d, window, rot, normed):
@@ -812,16 +815,24 @@ def test_attention_prefill_shares_of_the_keys(nh, nkv, d, window, lengths, new):
     close(got, want, torch.bfloat16, atol=attention_atol(torch.bfloat16, vc))
 
 
-@pytest.mark.parametrize("nh,nkv,d,window", [(32, 8, 128, 0), (6, 2, 96, 700), (8, 1, 64, 0)])
-def test_attention_decode_of_many_requests_of_unequal_length(nh, nkv, d, window):
+@pytest.mark.parametrize("nh,nkv,d,window", [(32, 8, 128, 0), (6, 2, 96, 700), (8, 1, 64, 0), (4, 2, 32, 0)])
+@pytest.mark.parametrize("waves", [0, 4])
+def test_attention_decode_of_many_requests_of_unequal_length(nh, nkv, d, window, waves):
     """So many requests that each gets one workgroup per kv head (of eight waves then), lengths
-    from one token to thousands."""
+    from one token to thousands; also with workgroups of four waves, which walk their pages
+    with two in flight: every number of pages a wave, from none on, the first and the last turn
+    of the three sets of page registers."""
     rng = random.Random(5)
     lengths = [rng.choice([1, 15, 16, 17, 100, 700, 2100, 3000]) for _ in range(70)]
+    lengths[:14] = [16 * 4 * n + k for n in range(7) for k in (1, 16)]     # 0 to 6 whole rounds of four waves, and one page more
     qkv, batch, kc, vc = paged_case(lengths, [1] * len(lengths), nh, nkv, d, 16, torch.bfloat16, seed=95)
     if nkv >= 8:
         assert ops.library().lc_attn_decode_splits(len(lengths), nkv, max(lengths)) == 1
-    got = ops.attention(qkv, batch, kc, vc, nh, nkv, d, 16, d ** -0.5, window)
+    ops.library().lc_attn_decode_waves(waves)
+    try:
+        got = ops.attention(qkv, batch, kc, vc, nh, nkv, d, 16, d ** -0.5, window)
+    finally:
+        ops.library().lc_attn_decode_waves(0)
     want = ref.attention(qkv.cpu(), AttentionBatch(batch.tok_req.cpu(), batch.positions.cpu(),
                                                    batch.block_table.cpu()),
                          kc.cpu(), vc.cpu(), nh, nkv, d, 16, d ** -0.5, window)
@@ -871,6 +882,15 @@ def test_attention_decode_takes_q_k_v_as_shares_of_a_product(nh, nkv, window, ro
     b = ops.attention(ops.ProductShares(part5, torch.bfloat16).value(), mixed, kc3.clone(), vc3.clone(), nh, nkv, d,
                       16, d ** -0.5, window, ops.QKPrologue(qw, kw, 1e-6, table, slots5))
     assert torch.equal(a, b)
+
+
+def test_decode_attention_keeps_its_page_registers_in_registers():
+    """The decode kernel's walk with two pages in flight fills its page registers with loads that
+    the compiler does not count; that is only sound while none of them is spilled.  The library asks
+    its compiled kernels and must find them without scratch memory (else it would quietly walk with
+    one page in flight)."""
+    for d in (32, 64, 96, 128):
+        assert ops.library().lc_attn_decode_deep_ok(d) == 1
 
 
 def test_runs_kernel_keeps_its_ring_of_x_in_registers():
