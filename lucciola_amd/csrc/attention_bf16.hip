@@ -279,7 +279,7 @@ template <int D, int NW, bool DEEP>
 __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
     const bf16* __restrict__ qkv, int q_stride, bf16* k_cache, bf16* v_cache,
     bf16* __restrict__ out, float* __restrict__ part_o,
-    float* __restrict__ part_ml, const int4* __restrict__ decode_rows,
+    float* __restrict__ part_ml, const int4* __restrict__ decode_rows, const int* __restrict__ items,
     const int* __restrict__ block_table, int max_blocks, int nh, int nkv, float scale_log2,
     int window, int splits, DecodePrologue pro) {
     constexpr int ROW = D + 4;       // a head's D sums lie together; the padding spreads the heads over the banks
@@ -287,20 +287,39 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
     __shared__ float sm_m[NW][16], sm_l[NW][16];
     __shared__ __attribute__((aligned(16))) bf16 sm_q[16 * D];
 
-    const int split = blockIdx.x, kvh = blockIdx.y, di = blockIdx.z;
+    // Two ways to share the work out.  Without `items`, the grid is (shares, kv heads, rows) and every
+    // row's pages are cut into `splits` equal shares.  With `items` (eight numbers each: token row,
+    // request, position, row, first page, end page, the row's number of shares, 0), the grid is (items,
+    // kv heads): a list made on the host from the requests' lengths, which gives a long request more
+    // shares than a short one; an item of no shares is a spare that does nothing.
+    const int kvh = blockIdx.y;
+    int split = blockIdx.x, di = blockIdx.z, my_shares = splits, item_begin = 0, item_end = 0;
+    int4 mine;
+    if (items) {
+        const int4* it = reinterpret_cast<const int4*>(items) + (size_t)blockIdx.x * 2;
+        mine = it[0];
+        const int4 range = it[1];
+        di = mine.w;
+        item_begin = range.x;
+        item_end = range.y;
+        my_shares = range.z;
+        split = 0;
+        if (my_shares == 0) return;
+    } else {
+        // the token's row in the batch, its request's row of the block table and its position come
+        // in one load: every look-up that hangs on another is a trip to memory before the first key
+        mine = decode_rows[di];
+    }
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // the same for the whole wave: its page numbers are scalar loads
     const int q = lane & 15, kg = lane >> 4;
-    // the token's row in the batch, its request's row of the block table and its position come
-    // in one load: every look-up that hangs on another is a trip to memory before the first key
-    const int4 mine = decode_rows[di];
     const int t = mine.x, req = mine.y, p = mine.z;
     const int G = nh / nkv;
     const int j_lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int first_page = j_lo / PAGE, last_page = p / PAGE;
     const int per = (last_page - first_page + splits) / splits;   // ceil(pages / splits)
-    const int begin = first_page + split * per;
-    const int end = min(begin + per, last_page + 1);
+    const int begin = items ? max(first_page, item_begin) : first_page + split * per;
+    const int end = items ? min(item_end, last_page + 1) : min(begin + per, last_page + 1);
     const int* table = block_table + (size_t)req * max_blocks;
     // the numbers of the wave's first two pages: asked for now, they are back before the q/k preparation below is done
     const int pg0 = begin + wave;
@@ -458,13 +477,13 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
             }
         }
         const int h = kvh * G + qq;
-        if (splits == 1) {
+        if (my_shares == 1) {
             short4v packed;
 #pragma unroll
             for (int v = 0; v < 4; ++v) packed[v] = bf16_bits(o[v] / lsum);
             *reinterpret_cast<short4v*>(out + ((size_t)t * nh + h) * D + dim) = packed;
         } else {
-            const size_t slot = ((size_t)di * nh + h) * splits + split;
+            const size_t slot = items ? (size_t)blockIdx.x * nh + h : ((size_t)di * nh + h) * splits + split;
             *reinterpret_cast<floatx4*>(part_o + slot * D + dim) = o;
             if (dim == 0) { part_ml[slot * 2] = m_all; part_ml[slot * 2 + 1] = lsum; }
         }
@@ -474,7 +493,7 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(
 template <int D, int MOST>
 __device__ __forceinline__ void join_shares_of(const float* __restrict__ part_o,
                                                const float* __restrict__ part_ml, size_t base,
-                                               int splits, bf16* __restrict__ out_row) {
+                                               size_t stride, int splits, bf16* __restrict__ out_row) {
     __shared__ float f[64];
     __shared__ float inv_l;
     const int tid = threadIdx.x;
@@ -482,11 +501,11 @@ __device__ __forceinline__ void join_shares_of(const float* __restrict__ part_o,
     float early[MOST];
     if (tid < D) {
 #pragma unroll
-        for (int s = 0; s < MOST; ++s) early[s] = s < splits ? part_o[(base + s) * D + tid] : 0.f;
+        for (int s = 0; s < MOST; ++s) early[s] = s < splits ? part_o[(base + s * stride) * D + tid] : 0.f;
     }
     if (tid < 64) {
-        const float ms = tid < splits ? part_ml[(base + tid) * 2] : -INFINITY;
-        const float ls = tid < splits ? part_ml[(base + tid) * 2 + 1] : 0.f;
+        const float ms = tid < splits ? part_ml[(base + tid * stride) * 2] : -INFINITY;
+        const float ls = tid < splits ? part_ml[(base + tid * stride) * 2 + 1] : 0.f;
         const float m = wave_max(ms);
         const float fs = (ms == -INFINITY) ? 0.f : exp2f(ms - m);
         f[tid] = fs;
@@ -503,15 +522,15 @@ __device__ __forceinline__ void join_shares_of(const float* __restrict__ part_o,
 }
 
 // Joins the shares of a row's keys: out = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m), the
-// shares of (row, head) lying at part_o[base + s][D] and part_ml[base + s][2].  The factors are
+// shares of (row, head) lying at part_o[base + s stride][D] and part_ml[base + s stride][2].  The factors are
 // worked out once (one thread per share) and left in LDS.  128 threads (D <= 128); at most 64 shares.
 template <int D>
 __device__ __forceinline__ void join_shares(const float* __restrict__ part_o,
                                             const float* __restrict__ part_ml, size_t base,
-                                            int splits, bf16* __restrict__ out_row) {
-    if (splits <= 8) join_shares_of<D, 8>(part_o, part_ml, base, splits, out_row);
-    else if (splits <= 32) join_shares_of<D, 32>(part_o, part_ml, base, splits, out_row);
-    else join_shares_of<D, 64>(part_o, part_ml, base, splits, out_row);
+                                            size_t stride, int splits, bf16* __restrict__ out_row) {
+    if (splits <= 8) join_shares_of<D, 8>(part_o, part_ml, base, stride, splits, out_row);
+    else if (splits <= 32) join_shares_of<D, 32>(part_o, part_ml, base, stride, splits, out_row);
+    else join_shares_of<D, 64>(part_o, part_ml, base, stride, splits, out_row);
 }
 
 template <int D>
@@ -519,10 +538,18 @@ __global__ __launch_bounds__(128) void attn_decode_join_kernel(const float* __re
                                                                const float* __restrict__ part_ml,
                                                                const int4* __restrict__ decode_rows,
                                                                bf16* __restrict__ out, int nh,
-                                                               int splits) {
+                                                               int splits, int by_items) {
     const int di = blockIdx.x, h = blockIdx.y;
-    const int t = decode_rows[di].x;
-    join_shares<D>(part_o, part_ml, ((size_t)di * nh + h) * splits, splits, out + ((size_t)t * nh + h) * D);
+    const int4 row = decode_rows[di];
+    bf16* out_row = out + ((size_t)row.x * nh + h) * D;
+    if (by_items) {
+        // the row's items are neighbours in the list: the first in the low 20 bits, their number above;
+        // the only item of a row has written the row itself
+        const int first = row.w & 0xFFFFF, count = row.w >> 20;
+        if (count > 1) join_shares<D>(part_o, part_ml, (size_t)first * nh + h, nh, count, out_row);
+    } else {
+        join_shares<D>(part_o, part_ml, ((size_t)di * nh + h) * splits, 1, splits, out_row);
+    }
 }
 
 // The same for the rows of prefill tiles, whose shares lie at the rows' places in the batch.
@@ -536,7 +563,7 @@ __global__ __launch_bounds__(128) void attn_prefill_join_kernel(const float* __r
     const int r = blockIdx.x & 63, h = blockIdx.y;
     if (r >= tile[2]) return;
     const int t = tile[1] + r;
-    join_shares<D>(part_o, part_ml, ((size_t)t * nh + h) * splits, splits, out + ((size_t)t * nh + h) * D);
+    join_shares<D>(part_o, part_ml, ((size_t)t * nh + h) * splits, 1, splits, out + ((size_t)t * nh + h) * D);
 }
 
 // A lane's part of one raw q row of 128 entries, as the matrix-core operand holds it (entries
@@ -1121,11 +1148,11 @@ static int decode_deep_state() {
 
 template <int D>
 static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* out,
-                         float* part_o, float* part_ml, const int4* decode_rows,
-                         const int* table, int max_blocks, int ND, int nh,
+                         float* part_o, float* part_ml, const int4* decode_rows, const int* items,
+                         int num_items, const int* table, int max_blocks, int ND, int nh,
                          int nkv, float scale_log2, int window, int splits, bool even_lengths,
                          DecodePrologue pro, hipStream_t s) {
-    dim3 grid(splits, nkv, ND);
+    const dim3 grid = items ? dim3(num_items, nkv, 1) : dim3(splits, nkv, ND);
     // One workgroup per request and kv head (no shares): requests of unequal length leave the
     // long ones running alone at the end, each at the pace its waves draw on memory; eight
     // waves double that (64 requests of 16 to 2,176 tokens: 59 instead of 65 us; equal lengths
@@ -1137,13 +1164,15 @@ static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* 
     // instead of 57.4 us, 16 in two 104.7 instead of 107.4, one request with its join 16.1 instead
     // of 17.2, 8 of 1,024 tokens 15.7 instead of 16.8).  Two shares of more requests than CUs
     // likewise.
-    const long long workgroups = (long long)ND * nkv * splits;
+    const long long workgroups = items ? (long long)num_items * nkv : (long long)ND * nkv * splits;
     // Whole requests of about the same length, more of them than CUs: nobody is left running
     // alone, and four waves a workgroup are as good or better (with cold caches 48 requests of
     // 1,024 tokens 48.8 instead of 53.5 us, 64 requests 58.9 instead of 61.7, 32 of 8,192 192
     // instead of 194).
     const bool alone_at_the_end = !even_lengths || workgroups <= device_cus();
+    // (a list of items is made for requests of unequal length: eight waves)
     const int waves = g_decode_waves ? g_decode_waves
+                      : items ? 8
                       : (splits == 1 && max_blocks >= 32 && workgroups < 4ll * device_cus() && alone_at_the_end) ? 8
                       : (splits > 1 && workgroups <= device_cus()) ? 8
                       : (splits == 2 && workgroups > 2ll * device_cus()) ? 8 : 4;
@@ -1157,16 +1186,16 @@ static int launch_decode(const bf16* qkv, int q_stride, bf16* k, bf16* v, bf16* 
     const bool deep = waves == 4 && g_decode_deep && decode_deep_state<D>() == 1;
 #define LC_DECODE(NW, DEEP)                                                                             \
     attn_decode_kernel<D, NW, DEEP><<<grid, 64 * NW, 0, s>>>(qkv, q_stride, k, v, out, part_o, part_ml, \
-                                                             decode_rows, table, max_blocks, nh, nkv,   \
-                                                             scale_log2, window, splits, pro)
+                                                             decode_rows, items, table, max_blocks, nh, \
+                                                             nkv, scale_log2, window, splits, pro)
     if (waves == 8) LC_DECODE(8, false);
     else if (deep) LC_DECODE(4, true);
     else LC_DECODE(4, false);
 #undef LC_DECODE
     LC_LAUNCH_CHECK("attn_decode");
-    if (splits > 1) {
+    if (splits > 1 || items) {
         attn_decode_join_kernel<D><<<dim3(ND, nh), 128, 0, s>>>(
-            part_o, part_ml, decode_rows, out, nh, splits);
+            part_o, part_ml, decode_rows, out, nh, splits, items ? 1 : 0);
         LC_LAUNCH_CHECK("attn_decode_join");
     }
     return 0;
@@ -1316,6 +1345,21 @@ LC_API int lc_attn_decode_splits(int num_decode, int nkv, int max_ctx) {
     return (int)splits;
 }
 
+// Whether a step's decode rows are better served through the planner's list of work items, which
+// gives a long request more shares than a short one, than with the same number of shares for
+// every request: longest and total are the requests' lengths in tokens.  With few requests (the
+// workgroups of one share each fill half of the CUs at most) as soon as the lengths are uneven; with many
+// only when a few requests hold most of the keys, because the list brings half as many workgroups
+// more and always a join (with cold caches: one request of 8,192 tokens among 63 of 512 103 -> 45 us,
+// 16 requests of 100 to 8,000 tokens 57.1 -> 52.8, 8 such 37.4 -> 33.6; but 64 of 16 to 2,200 tokens
+// 57.1 -> 65.6, 128 such 107 -> 122, 64 of 1,024 53.3 -> 63.9, 8 of 1,024 14.6 -> 18.8).
+LC_API int lc_attn_decode_by_items(int num_decode, int nkv, int longest, long long total) {
+    if (num_decode < 2 || total <= 0) return 0;
+    const long long spread = (long long)longest * num_decode;       // against the total: 1 for equal lengths
+    if ((long long)num_decode * nkv * 2 <= device_cus()) return spread * 4 > total * 5;
+    return spread >= total * 3;
+}
+
 #define LC_DISPATCH_D(d, CALL)                   \
     switch (d) {                                 \
         case 32: return CALL(32);                \
@@ -1330,12 +1374,17 @@ LC_API int lc_attn_decode_splits(int num_decode, int nkv, int max_ctx) {
 // the kernel that sums shares does): with its own preparation of whole heads of 128.
 LC_API int lc_attn_decode_takes_shares(int d, int rot) { return d == 128 && (rot == 0 || rot == 128); }
 
+// decode_rows: four numbers a row (token row, request, position, and with items: the row's first
+// item in the low 20 bits, its number of items above).  items (or null): num_items work items of
+// eight numbers (token row, request, position, row, first page, end page, the row's number of
+// items, 0), a row's items neighbours in the list and their page ranges in ascending order, the
+// last one reaching the row's last page; part_o and part_ml then hold num_items x nh entries.
 // prologue != 0: qkv holds the raw projections; the kernel norms and rotates q and k itself
 // (q_w, k_w, rope_table may be null; rot entries of a head rotate) and, if write_kv != 0, writes
 // the tokens' k and v to the cache.  Otherwise qkv is ready and the cache holds the tokens.
 LC_API int lc_attn_decode_bf16(const void* qkv, int q_stride, void* k_cache, void* v_cache,
                                void* out, float* part_o, float* part_ml, const int* decode_rows,
-                               const int* block_table,
+                               const int* items, int num_items, const int* block_table,
                                int max_blocks, int num_decode, int nh, int nkv, int d, int page_size,
                                float scale, int window, int splits, int even_lengths, int prologue, const float* q_w,
                                const float* k_w, float eps, const float* rope_table, int rot,
@@ -1359,12 +1408,15 @@ LC_API int lc_attn_decode_bf16(const void* qkv, int q_stride, void* k_cache, voi
     LC_CHECK((uintptr_t)decode_rows % 16 == 0, "attn_decode_bf16: the decode rows must be 16-byte aligned");
     LC_CHECK(splits >= 1 && splits <= 65535 && (splits == 1 || (part_o && part_ml)),
              "attn_decode_bf16: %d shares need a workspace", splits);
+    LC_CHECK(!items || (num_items >= 1 && splits == 1 && part_o && part_ml && (uintptr_t)items % 16 == 0),
+             "attn_decode_bf16: a list of items (%d) needs a workspace, 16-byte alignment and no equal shares beside it (%d)",
+             num_items, splits);
     LC_CHECK(q_stride % 8 == 0 && (uintptr_t)qkv % 16 == 0, "attn_decode_bf16: q must be 16-byte aligned");
     LC_CHECK(!prologue || ((uintptr_t)q_w % 16 == 0 && (uintptr_t)k_w % 16 == 0 && (uintptr_t)rope_table % 16 == 0),
              "attn_decode_bf16: the norms' weights and the rotary table must be 16-byte aligned");
     const float sl2 = scale * 1.4426950408889634f;
 #define CALL(DD) launch_decode<DD>((const bf16*)qkv, q_stride, (bf16*)k_cache, (bf16*)v_cache,             \
-        (bf16*)out, part_o, part_ml, (const int4*)decode_rows, block_table, max_blocks,                     \
+        (bf16*)out, part_o, part_ml, (const int4*)decode_rows, items, num_items, block_table, max_blocks,   \
         num_decode, nh, nkv, sl2, window, splits, even_lengths != 0, pro, stream)
     LC_DISPATCH_D(d, CALL)
 #undef CALL

@@ -8,6 +8,8 @@ if the library cannot be built or opened.  Parts call these through the module
 from __future__ import annotations
 
 import ctypes
+import heapq
+import threading
 from dataclasses import dataclass, replace
 from typing import Optional
 
@@ -21,7 +23,7 @@ _lib = None
 DT_F32, DT_BF16 = 0, 1
 
 # argument kinds: p pointer, i int, f float
-_ARG = {"p": ctypes.c_void_p, "i": ctypes.c_int, "f": ctypes.c_float}
+_ARG = {"p": ctypes.c_void_p, "i": ctypes.c_int, "f": ctypes.c_float, "q": ctypes.c_longlong}
 _SIGNATURES = {
     "lc_embedding": "ppipiiifp",
     "lc_rmsnorm": "ppppfpiiiipiip",
@@ -55,8 +57,9 @@ _SIGNATURES = {
     "lc_attn_decode_waves": "i",
     "lc_attn_decode_deep": "i",
     "lc_attn_decode_deep_ok": "i",
+    "lc_attn_decode_by_items": "iiiq",
     "lc_attn_decode_force_splits": "i",
-    "lc_attn_decode_bf16": "pippppppp" + "iiiiii" + "f" + "iii" + "ippfpii" + "pii" + "p",
+    "lc_attn_decode_bf16": "pipppppppip" + "iiiiii" + "f" + "iii" + "ippfpii" + "pii" + "p",
     "lc_attn_decode_takes_shares": "ii",
     "lc_gemm_bf16_sum_shares": "ppiiiip",
     "lc_attn_prefill_bf16": "pippppp" + "iiiiii" + "f" + "i" + "ipfpi" + "ipp" + "p",
@@ -76,13 +79,13 @@ class KernelError(RuntimeError):
 
 def register_signatures(signatures) -> None:
     """Entry points of the kernel library beyond the ones listed above, ``{name: kinds}`` with one
-    letter per argument (p pointer, i int, f float; they return an int, 0 for success): a part
+    letter per argument (p pointer, i int, q 64-bit int, f float; they return an int, 0 for success): a part
     that brings kernels of its own (a source file added to ``csrc``) declares them here and
     launches them with :func:`call`; no table in this file has to know them."""
     for name, kinds in signatures.items():
         bad = [c for c in kinds if c not in _ARG]
         if bad:
-            raise KernelError(f"entry point {name}: unknown argument kinds {bad} (p, i or f)")
+            raise KernelError(f"entry point {name}: unknown argument kinds {bad} (p, i, q or f)")
         if _SIGNATURES.get(name, kinds) != kinds:
             raise KernelError(f"entry point {name} is already declared as '{_SIGNATURES[name]}'")
         if _lib is not None:
@@ -547,11 +550,30 @@ class AttentionBatch:
     ctx_len: Optional[torch.Tensor] = None
     slots: Optional[torch.Tensor] = None
     num_decode: int = 0
-    decode_rows: Optional[torch.Tensor] = None     # [ND, 4] of the length-1 portions: token row, request, position, 0
+    decode_rows: Optional[torch.Tensor] = None     # [ND, 4] of the length-1 portions: token row, request, position, its items
+    decode_items: Optional[torch.Tensor] = None    # [NI, 8]: the rows' pages cut into work items by length (None: not prepared)
     prefill_tiles: Optional[torch.Tensor] = None   # [NT, 4]: request, first token row, rows, first position
     max_ctx: int = 0                               # longest cached length in the batch
     all_decode: bool = False
     even_lengths: bool = False                     # the longest decoding request is within a tenth of the mean length
+    decode_longest: int = 0                        # tokens of the longest decoding request, and of all of them
+    decode_total: int = 0
+
+
+class _Switch(threading.local):
+    on = True
+
+
+_decode_by_items = _Switch()     # per thread, like the library's own switches
+
+
+def decode_by_items(on):
+    """Whether the decode kernel takes the planner's list of work items: True where the library
+    says it pays (the default), False never, "always" wherever there is a list (tests and
+    tuning); returns the setting before."""
+    before = _decode_by_items.on
+    _decode_by_items.on = on if on == "always" else bool(on)
+    return before
 
 
 PREFILL_TILE = 64               # query rows of one work item of the prefill attention kernel
@@ -595,8 +617,87 @@ def plan_attention(layout):
         # so that none of them starts late and runs on alone at the end (64 requests of 16 to 2,200
         # tokens: 58 instead of 70 us a layer; the order changes no token's result)
         decode = decode[np.argsort(-lengths, kind="stable")]
-    return ({"decode_rows": decode, "prefill_tiles": tiles},
-            {"num_decode": int(singles.size), "all_decode": int(singles.size) == R, "even_lengths": even})
+    items = _decode_items(decode, lengths[np.argsort(-lengths, kind="stable")] if lengths.size > 1 else lengths)
+    # (whether the list pays, the kernel's library says from the longest and the total length)
+    return ({"decode_rows": decode, "decode_items": items, "prefill_tiles": tiles},
+            {"num_decode": int(singles.size), "all_decode": int(singles.size) == R, "even_lengths": even,
+             "decode_longest": int(lengths.max()) if lengths.size else 0,
+             "decode_total": int(lengths.sum()) if lengths.size else 0})
+
+
+ITEM_PAGES_MIN = 8       # kernel pages of the smallest work item that a request is cut into
+ITEM_SHARES_MOST = 32    # items of one request at most (the join kernel takes up to 64)
+
+
+def decode_item_count(num_decode: int) -> int:
+    """Work items that the planner makes for a step with ``num_decode`` single tokens: a number
+    that follows from the count alone, so that steps of one make-up have lists of one size (a
+    captured step is replayed with the next step's list in the same buffer)."""
+    return max(num_decode + num_decode // 2, min(64, 8 * num_decode)) if num_decode else 0
+
+
+def _decode_items(decode: np.ndarray, lengths: np.ndarray) -> np.ndarray:
+    """The decode rows' pages (of ATTENTION_PAGE_GRANULE tokens) cut into ``decode_item_count``
+    work items so that the largest item is as small as may be: every row one item, the spare ones
+    to whichever row has the largest items then (at most ITEM_SHARES_MOST a row, none smaller than
+    ITEM_PAGES_MIN pages).  Eight numbers an item: token row, request, position, row, first page,
+    end page, the row's number of items, 0; a row's items are neighbours; items that are left over
+    have no shares and do nothing.  Writes each row's first item and number of items into
+    ``decode[:, 3]``.  ``lengths`` in the order of ``decode``."""
+    nd = int(decode.shape[0])
+    total = decode_item_count(nd)
+    items = np.zeros((total, 8), dtype=np.int32)
+    if nd == 0:
+        return items
+    lengths = np.asarray(lengths, dtype=np.int64)
+    pages = (lengths + ATTENTION_PAGE_GRANULE - 1) // ATTENTION_PAGE_GRANULE
+    shares = np.ones(nd, dtype=np.int64)
+    # lengths so even that no launcher would take the list: every row its one item, no search
+    uneven = int(lengths.max()) * nd * 4 > int(lengths.sum()) * 5
+    spare = total - nd
+    if uneven and spare > 0:
+        most = np.minimum(ITEM_SHARES_MOST, np.maximum(1, pages // ITEM_PAGES_MIN))
+        heap = [(-int(pages[r]), r) for r in np.nonzero(most > 1)[0].tolist()]
+        heapq.heapify(heap)
+        while spare > 0 and heap:
+            _, r = heapq.heappop(heap)
+            shares[r] += 1
+            spare -= 1
+            if shares[r] < most[r]:
+                heapq.heappush(heap, (-int((pages[r] + shares[r] - 1) // shares[r]), r))
+    first = np.cumsum(shares) - shares
+    decode[:, 3] = first | (shares << 20)
+    used = int(shares.sum())
+    row = np.repeat(np.arange(nd, dtype=np.int64), shares)
+    nth = np.arange(used, dtype=np.int64) - first[row]        # which of its row's items
+    n, k = pages[row], shares[row]                            # sizes that differ by one page at most, none empty
+    items[:used, 0:3] = decode[row, 0:3]
+    items[:used, 3] = row
+    items[:used, 4] = nth * n // k
+    items[:used, 5] = (nth + 1) * n // k
+    items[:used, 6] = k
+    return items
+    pages = (np.asarray(lengths, dtype=np.int64) + ATTENTION_PAGE_GRANULE - 1) // ATTENTION_PAGE_GRANULE
+    shares = np.ones(nd, dtype=np.int64)
+    most = np.minimum(ITEM_SHARES_MOST, np.maximum(1, pages // ITEM_PAGES_MIN))
+    spare = total - nd
+    if spare > 0:
+        heap = [(-int(pages[r]), r) for r in range(nd) if most[r] > 1]
+        heapq.heapify(heap)
+        while spare > 0 and heap:
+            _, r = heapq.heappop(heap)
+            shares[r] += 1
+            spare -= 1
+            if shares[r] < most[r]:
+                heapq.heappush(heap, (-int((pages[r] + shares[r] - 1) // shares[r]), r))
+    at = 0
+    for r in range(nd):
+        k, n = int(shares[r]), int(pages[r])
+        decode[r, 3] = at | (k << 20)
+        for s in range(k):      # sizes that differ by one page at most, none empty
+            items[at] = (decode[r, 0], decode[r, 1], decode[r, 2], r, s * n // k, (s + 1) * n // k, k, 0)
+            at += 1
+    return items
 
 
 # Tokens of a cache page as the matrix-core attention kernels index it: a page of a multiple of
@@ -623,6 +724,9 @@ def attention_batch(batch, pages, plan=None) -> AttentionBatch:
                               ctx_len=batch.ctx_len, slots=pages.slots, max_ctx=batch.max_ctx)
         if plan is not None:
             done = replace(done, decode_rows=plan.arrays["decode_rows"],
+                           decode_items=plan.arrays.get("decode_items"),
+                           decode_longest=plan.info.get("decode_longest", 0),
+                           decode_total=plan.info.get("decode_total", 0),
                            prefill_tiles=plan.arrays["prefill_tiles"],
                            num_decode=plan.info["num_decode"], all_decode=plan.info["all_decode"],
                            even_lengths=plan.info["even_lengths"])
@@ -713,13 +817,23 @@ def attention(qkv, batch: AttentionBatch, k_cache: torch.Tensor,
         mb = batch.block_table.shape[1]
         nd = batch.num_decode
         if nd > 0:
-            splits = lib.lc_attn_decode_splits(nd, nkv, batch.max_ctx)
+            # requests of unequal length: the planner's list of work items, which cuts the long ones
+            # into more shares than the short ones; else every request into the same number
+            # (a captured step keeps the choice of its capture)
+            items = None
+            if batch.decode_items is not None and _decode_by_items.on is not False and (
+                    _decode_by_items.on == "always"
+                    or lib.lc_attn_decode_by_items(nd, nkv, batch.decode_longest, batch.decode_total)):
+                items = batch.decode_items
+            splits = 1 if items is not None else lib.lc_attn_decode_splits(nd, nkv, batch.max_ctx)
             part_o = part_ml = None
-            if splits > 1:
-                part_o = torch.empty((nd * nh * splits * d,), dtype=torch.float32, device=qkv.device)
-                part_ml = torch.empty((nd * nh * splits * 2,), dtype=torch.float32, device=qkv.device)
+            parts = items.shape[0] if items is not None else (nd * splits if splits > 1 else 0)
+            if parts:
+                part_o = torch.empty((parts * nh * d,), dtype=torch.float32, device=qkv.device)
+                part_ml = torch.empty((parts * nh * 2,), dtype=torch.float32, device=qkv.device)
             _call("lc_attn_decode_bf16", _ptr(qkv if shares is None else None), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
                   _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(batch.decode_rows),
+                  _ptr(items), items.shape[0] if items is not None else 0,
                   _ptr(batch.block_table), mb, nd, nh,
                   nkv, d, page_size, scale, window, splits, 1 if batch.even_lengths else 0,
                   1 if in_kernel else 0,

@@ -3,6 +3,7 @@ than the tiny models': widths and vocabularies that are no power of two, head si
 of 16, odd head counts and groups, several page sizes, in float32 and bfloat16."""
 import random
 
+import numpy as np
 import pytest
 import torch
 
@@ -159,7 +160,9 @@ def paged_case(lengths, new, nh, nkv, d, page, dtype, seed, spare=3):
         q_start.append(q_start[-1] + k)
     T = len(tok_req)
     qkv = rnd(T, (nh + 2 * nkv) * d, dtype=dtype, seed=seed + 3)
-    dec = [[q_start[r], r, lengths[r] - 1, 0] for r in range(R) if new[r] == 1]
+    dec = np.asarray([[q_start[r], r, lengths[r] - 1, 0] for r in range(R) if new[r] == 1], dtype=np.int32).reshape(-1, 4)
+    dec_lengths = np.asarray([lengths[r] for r in range(R) if new[r] == 1], dtype=np.int64)
+    items = ops._decode_items(dec, dec_lengths)       # the planner's list of work items, taken where a test asks
     tiles = []
     for r in range(R):
         if new[r] > 1:
@@ -168,8 +171,10 @@ def paged_case(lengths, new, nh, nkv, d, page, dtype, seed, spare=3):
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
     batch = AttentionBatch(tok_req=i32(tok_req), positions=i32(positions), block_table=table.to(DEV),
                            q_start=i32(q_start), ctx_len=i32(lengths), num_decode=len(dec),
-                           decode_rows=i32(dec).view(-1, 4), prefill_tiles=i32(tiles).view(-1, 4),
-                           max_ctx=max(lengths), all_decode=len(dec) == R)
+                           decode_rows=torch.from_numpy(dec).to(DEV), prefill_tiles=i32(tiles).view(-1, 4),
+                           decode_items=torch.from_numpy(items).to(DEV),
+                           decode_longest=int(dec_lengths.max()) if len(dec) else 0,
+                           decode_total=int(dec_lengths.sum()), max_ctx=max(lengths), all_decode=len(dec) == R)
     return qkv, batch, kc, vc
 
 
@@ -521,21 +526,25 @@ def test_attention_prefill_of_heads_of_128_in_pairs(nh, nkv, window):
 @pytest.mark.parametrize("nh,nkv,d,window,rot,normed", [(32, 8, 128, 0, 128, True), (6, 2, 96, 24, 96, True),
                                                         (8, 1, 64, 0, 32, False), (4, 4, 32, 0, 0, True),
                                                         (16, 1, 32, 0, 32, True)])
-@pytest.mark.parametrize("waves,deep", [(0, 1), (4, 1), (4, 0), (8, 1)])
-def test_attention_decode_with_prologue_in_the_kernel(nh, nkv, d, window, rot, normed, waves, deep):
+@pytest.mark.parametrize("waves,deep,items", [(0, 1, False), (4, 1, False), (4, 0, False), (8, 1, False),
+                                              (0, 1, "always"), (4, 1, "always")])
+def test_attention_decode_with_prologue_in_the_kernel(nh, nkv, d, window, rot, normed, waves, deep, items):
     """A step of single tokens with raw q, k, v: the decode kernel norms, rotates and writes
     the cache itself.  Output and cache must equal those of the separate kernel followed by
     the plain decode kernel, for short and long contexts (one or many shares of the pages),
     a token at a page's first and last place, part of the head rotated or none; with workgroups
-    of four and of eight waves, the four-wave ones with two pages in flight and with one."""
+    of four and of eight waves, the four-wave ones with two pages in flight and with one; with
+    every request's pages in the same number of shares, and cut into the planner's work items."""
     lib = ops.library()
     lib.lc_attn_decode_waves(waves)
     lib.lc_attn_decode_deep(deep)
+    ops.decode_by_items(items)
     try:
         decode_prologue_case(nh, nkv, d, window, rot, normed)
     finally:
         lib.lc_attn_decode_waves(0)
         lib.lc_attn_decode_deep(1)
+        ops.decode_by_items(True)
 
 
 def decode_prologue_case(nh, nkv, d, window, rot, normed):
@@ -816,12 +825,13 @@ def test_attention_prefill_shares_of_the_keys(nh, nkv, d, window, lengths, new):
 
 
 @pytest.mark.parametrize("nh,nkv,d,window", [(32, 8, 128, 0), (6, 2, 96, 700), (8, 1, 64, 0), (4, 2, 32, 0)])
-@pytest.mark.parametrize("waves", [0, 4])
-def test_attention_decode_of_many_requests_of_unequal_length(nh, nkv, d, window, waves):
+@pytest.mark.parametrize("waves,items", [(0, False), (4, False), (0, "always"), (0, True)])
+def test_attention_decode_of_many_requests_of_unequal_length(nh, nkv, d, window, waves, items):
     """So many requests that each gets one workgroup per kv head (of eight waves then), lengths
     from one token to thousands; also with workgroups of four waves, which walk their pages
     with two in flight: every number of pages a wave, from none on, the first and the last turn
-    of the three sets of page registers."""
+    of the three sets of page registers; and through the planner's list of work items, which cuts
+    the long requests into more shares than the short ones."""
     rng = random.Random(5)
     lengths = [rng.choice([1, 15, 16, 17, 100, 700, 2100, 3000]) for _ in range(70)]
     lengths[:14] = [16 * 4 * n + k for n in range(7) for k in (1, 16)]     # 0 to 6 whole rounds of four waves, and one page more
@@ -829,10 +839,12 @@ def test_attention_decode_of_many_requests_of_unequal_length(nh, nkv, d, window,
     if nkv >= 8:
         assert ops.library().lc_attn_decode_splits(len(lengths), nkv, max(lengths)) == 1
     ops.library().lc_attn_decode_waves(waves)
+    ops.decode_by_items(items)
     try:
         got = ops.attention(qkv, batch, kc, vc, nh, nkv, d, 16, d ** -0.5, window)
     finally:
         ops.library().lc_attn_decode_waves(0)
+        ops.decode_by_items(True)
     want = ref.attention(qkv.cpu(), AttentionBatch(batch.tok_req.cpu(), batch.positions.cpu(),
                                                    batch.block_table.cpu()),
                          kc.cpu(), vc.cpu(), nh, nkv, d, 16, d ** -0.5, window)

@@ -876,7 +876,7 @@ def test_kernel_signatures_can_be_registered_from_outside():
     with pytest.raises(ops.KernelError, match="already declared"):
         ops.register_signatures({"lc_attn_page_granule": "i"})
     with pytest.raises(ops.KernelError, match="unknown argument kinds"):
-        ops.register_signatures({"lc_new_kernel": "pq"})
+        ops.register_signatures({"lc_new_kernel": "pz"})
     with pytest.raises(ops.KernelError, match="lacks the entry point"):
         ops.register_signatures({"lc_no_such_entry_point": "pi"})
     assert "lc_no_such_entry_point" not in ops._SIGNATURES
