@@ -26,7 +26,9 @@ batch and launching, plus queueing the sampler; ``host_split_ms`` has the parts,
 for the engine's loop from ``LLMEngine.stats()``).  ``points`` holds, in tokens a second:
 decode at the other batch sizes at the headline's context (``decode_b1``, ``decode_b64``) and
 at a context of 1,024 tokens (``decode_b1_ctx1024``, ...: the length of the prompts that the
-baseline's runs decode after; there also a batch of 256, ``decode_b256_ctx1024``), the same batch driven through ``LLMEngine`` and its scheduler
+baseline's runs decode after; there also a batch of 256, ``decode_b256_ctx1024``), a batch of 64
+requests of uneven length (one at the headline's context among 63 of 512 tokens:
+``decode_b64_one_long``), the headline's batch driven through ``LLMEngine`` and its scheduler
 after real prompts of the context length (``decode_b8_engine``), the 2,048-token prompt fed in
 portions of 576, the reference's step budget (src/scheduler.cc:48; ``prefill_576``), and the
 other shapes (``32b_decode_b1``, ``32b_decode_b32``, ``32b_prefill_2048``, ``0.6b_mixed``).
@@ -132,16 +134,19 @@ class ModelBench:
         self.torch.cuda.empty_cache()
 
     def decode_run(self, batch, context, steps, warmup):
-        """Time ``steps`` decode steps of ``batch`` requests that hold ``context`` tokens each.
-        Returns a dict: ms, tokens a second, the bytes a step must read, gpu ms, host ms and its parts."""
+        """Time ``steps`` decode steps of ``batch`` requests that hold ``context`` tokens each (a
+        list: one length a request).  Returns a dict: ms, tokens a second, the bytes a step must
+        read, gpu ms, host ms and its parts."""
         from lucciola_amd.engine.batch import PENDING, Carry, StepEntry
         from lucciola_amd.sampling.sampler import SamplingParams
         torch, runner, sampler = self.torch, self.runner, self.sampler
-        names = [f"d{batch}_{context}_{i}" for i in range(batch)]
+        contexts = list(context) if isinstance(context, (list, tuple)) else [context] * batch
+        assert len(contexts) == batch
+        names = [f"d{batch}_{contexts[0]}_{contexts[-1]}_{i}" for i in range(batch)]
         cache = runner.cache
-        for n in names:
+        for n, c in zip(names, contexts):
             cache.admit(n)
-            cache.reserve(n, context - 1)
+            cache.reserve(n, c - 1)
             cache.commit(n)
         gen = torch.Generator().manual_seed(batch)
         tokens = torch.randint(0, self.V, (batch,), generator=gen).tolist()
@@ -182,7 +187,7 @@ class ModelBench:
         gpu_ms = first.elapsed_time(last) / steps
         split = {k: (runner.times[k] - before[k]) * 1e3 / steps for k in before}
         split["sample"] = state["sample_s"] * 1e3 / steps
-        ctx_mid = context + warmup + steps / 2.0
+        ctx_mid = sum(contexts) / batch + warmup + steps / 2.0
         for n in names:
             runner.finish(n)
         bytes_step = self.weight_bytes + batch * self.H * self.esize + batch * ctx_mid * self.kv_bytes_per_token
@@ -341,6 +346,8 @@ def main() -> int:
                     help="further batch sizes measured at the short context only (those that fit the cache)")
     ap.add_argument("--short-context", type=int, default=1024,
                     help="also decode at this context, at the headline's batch and the batches of --points (0: skip)")
+    ap.add_argument("--uneven-point", type=int, default=1, choices=[0, 1],
+                    help="1: also decode a batch of 64 with one request at the full context among 63 of 512 tokens")
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--run-ahead", type=int, default=1, choices=[0, 1],
                     help="1: a step is queued before the host has read the tokens of the one before")
@@ -412,6 +419,12 @@ def main() -> int:
             key = f"decode_b{b}_ctx{args.short_context}"
             values[key], fractions[key] = round(r["tps"], 2), round(r["frac"], 4)
             say(f"decode batch {b} at context {args.short_context}: {r['ms']:.3f} ms/step, {r['frac']:.3f} of the HBM peak")
+    if args.uneven_point and 64 in points and args.context >= 8192:
+        # requests of uneven length, as a serving batch has them: one long request among 63 short ones
+        r = bench.decode_run(64, [args.context] + [512] * 63, point_steps, 3)
+        values["decode_b64_one_long"], fractions["decode_b64_one_long"] = round(r["tps"], 2), round(r["frac"], 4)
+        say(f"decode batch 64, one request of {args.context} tokens among 63 of 512: {r['ms']:.3f} ms/step, "
+            f"{r['frac']:.3f} of the HBM peak")
     head = bench.decode_run(args.batch, args.context, args.steps, args.warmup)
     ms, tps = head["ms"], head["tps"]
     say(f"decode batch {args.batch}: {ms:.3f} ms/step (gpu {head['gpu_ms']:.3f}, host {head['host_ms']:.3f})")

@@ -172,6 +172,28 @@ class _Packer:
         return t.view(shape) if shape is not None else t
 
 
+@dataclass
+class PreparedBatch:
+    """A step's batch laid out on the host, before anything is sent: what ``upload_batch`` needs,
+    and ``graph_hint``, what the planners say about the shape of the kernels' launches for this
+    batch beyond its layout (a captured step is replayed only for batches of the same hint)."""
+
+    packer: "_Packer"
+    handles: Dict[str, int]
+    group_handles: list
+    planned: list
+    num_requests: int
+    num_tokens: int
+    requests: List[Hashable]
+    q_start: List[int]
+    first_position: List[int]
+    slot_list: List[int]
+    max_position: int
+    max_ctx: int
+    num_wanted: int
+    graph_hint: tuple
+
+
 def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
                 pad_blocks: Optional[int] = None, into: Optional[torch.Tensor] = None,
                 refresh_only: bool = False, carry_rows: Optional[dict] = None,
@@ -184,6 +206,15 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
     ``carry_rows``: for entries whose one token is PENDING, the row of the carry it comes from
     (the caller copies it in on the device; the host's copy holds token 0 there);
     ``planners``: the model's ``batch_planners()``, whose arrays travel in the same copy."""
+    prepared = prepare_batch(entries, cache, pad_blocks, carry_rows, planners)
+    return upload_batch(prepared, device, into, refresh_only)
+
+
+def prepare_batch(entries: Sequence[StepEntry], cache: CacheManager, pad_blocks: Optional[int] = None,
+                  carry_rows: Optional[dict] = None,
+                  planners: Optional[Dict[Any, Callable]] = None) -> PreparedBatch:
+    """The host's half of ``build_batch``: every array of the batch and of the planners, packed
+    for one copy, nothing sent yet."""
     bs = cache.block_size
     R = len(entries)
     requests = [e.request for e in entries]
@@ -271,21 +302,36 @@ def build_batch(entries: Sequence[StepEntry], cache: CacheManager, device,
             mb *= pieces
         group_handles.append((pk.add(flat), mb, pk.add(slots), g.kernel_page))
 
-    buffer = pk.upload(device, into)
-    if refresh_only:
-        return None
     max_ctx = int(max(ctx_len)) if R else 0
     if pad_blocks is not None:
         max_ctx = pad_blocks * bs      # what the layout allows, not what this batch holds
+    hint = tuple(info.get("graph_hint") for _, _, info in planned)
+    return PreparedBatch(
+        packer=pk, handles={"tok": h_tok, "feed": h_feed, "pos": h_pos, "req": h_req, "want": h_want,
+                            "slot": h_slot, "qs": h_qs, "ctx": h_ctx},
+        group_handles=group_handles, planned=planned, num_requests=R, num_tokens=T, requests=requests,
+        q_start=q_start, first_position=first_pos, slot_list=slot_list,
+        max_position=int(positions.max()) if T else 0, max_ctx=max_ctx, num_wanted=num_wanted,
+        graph_hint=hint)
+
+
+def upload_batch(prepared: PreparedBatch, device, into: Optional[torch.Tensor] = None,
+                 refresh_only: bool = False) -> Optional[StepBatch]:
+    """The other half: one copy to the device (``into``: over the buffer of an earlier batch of
+    the same layout) and, unless ``refresh_only``, the views of it."""
+    pk, h, R = prepared.packer, prepared.handles, prepared.num_requests
+    buffer = pk.upload(device, into)
+    if refresh_only:
+        return None
     groups = [PagesView(block_table=pk.view(h_bt, (R, mb)), slots=pk.view(h_sl), page_size=page)
-              for (h_bt, mb, h_sl, page) in group_handles]
-    plans = {key: Plan({name: pk.view(h, shape) for name, (h, shape) in handles.items()}, info)
-             for key, handles, info in planned}
+              for (h_bt, mb, h_sl, page) in prepared.group_handles]
+    plans = {key: Plan({name: pk.view(hd, shape) for name, (hd, shape) in handles.items()}, info)
+             for key, handles, info in prepared.planned}
     return StepBatch(
-        num_tokens=T, num_requests=R, requests=requests, q_start=q_start,
-        first_position=first_pos, slot_list=slot_list,
-        max_position=int(positions.max()) if T else 0,
-        token_ids=pk.view(h_tok), positions=pk.view(h_pos), tok_req=pk.view(h_req),
-        want_rows=pk.view(h_want), slot_ids=pk.view(h_slot), feed=pk.view(h_feed),
-        q_offsets=pk.view(h_qs), ctx_len=pk.view(h_ctx), max_ctx=max_ctx, groups=groups,
-        plans=plans, num_wanted=num_wanted, buffer=buffer)
+        num_tokens=prepared.num_tokens, num_requests=R, requests=prepared.requests, q_start=prepared.q_start,
+        first_position=prepared.first_position, slot_list=prepared.slot_list,
+        max_position=prepared.max_position,
+        token_ids=pk.view(h["tok"]), positions=pk.view(h["pos"]), tok_req=pk.view(h["req"]),
+        want_rows=pk.view(h["want"]), slot_ids=pk.view(h["slot"]), feed=pk.view(h["feed"]),
+        q_offsets=pk.view(h["qs"]), ctx_len=pk.view(h["ctx"]), max_ctx=prepared.max_ctx, groups=groups,
+        plans=plans, num_wanted=prepared.num_wanted, buffer=buffer)

@@ -19,7 +19,7 @@ from ..cache.page_pool import OutOfPages
 from ..config.engine_config import EngineConfig
 from ..models.causal_lm import CausalLM
 from ..kernels import ops
-from .batch import PENDING, Carry, SiteView, StepBatch, StepEntry, build_batch
+from .batch import PENDING, Carry, SiteView, StepBatch, StepEntry, build_batch, prepare_batch, upload_batch
 
 
 class _CapturedStep:
@@ -198,9 +198,9 @@ class ModelRunner:
     # ------------------------------------------------------------------ graph replay
     def _graph_step(self, entries: Sequence[StepEntry], carry: Optional[Carry]) -> torch.Tensor:
         """A step of single tokens, one per request, each wanting its logits: captured once per
-        (number of requests, block-table width) as a HIP graph and replayed afterwards.  Only the
-        batch description changes between replays, and it lives in one device buffer that is
-        overwritten in place.  """
+        (number of requests, block-table width, what the planners say of the launches' shapes) as
+        a HIP graph and replayed afterwards.  Only the batch description changes between replays,
+        and it lives in one device buffer that is overwritten in place.  """
         widest = max((len(g.tables[e.request]) for g in self.cache.groups for e in entries),
                      default=1)
         pad = max(64, -(-widest // 64) * 64)
@@ -215,13 +215,16 @@ class ModelRunner:
         if epoch != self._graph_epoch:      # a part has made a table anew: addresses changed
             self._graphs.clear()
             self._graph_epoch = epoch
-        key = (rows, pad)
+        t_in = time.perf_counter()
+        prepared = prepare_batch(entries, self.cache, pad_blocks=pad,
+                                 carry_rows=carry.rows if carry else None, planners=self.planners)
+        # a kernel's launch may depend on more than the layout (the attention's shares on how
+        # uneven the requests' lengths are): a captured step serves the batches of its own kind
+        key = (rows, pad, prepared.graph_hint)
         captured = self._graphs.get(key)
         next_position = max(self.cache.length(e.request) for e in entries)
         if captured is None or not self.model.ready(next_position):
-            t_in = time.perf_counter()
-            batch = build_batch(entries, self.cache, self.device, pad_blocks=pad,
-                                carry_rows=carry.rows if carry else None, planners=self.planners)
+            batch = upload_batch(prepared, self.device)
             if carry:
                 ops.feed_tokens(batch.token_ids, batch.feed, carry.ids)
             sites = self._sites(batch)
@@ -239,9 +242,7 @@ class ModelRunner:
             self.graph_captures += 1
             self.times["launch"] += time.perf_counter() - t_in      # a capture: the step run twice
             return logits[:real]
-        t_in = time.perf_counter()
-        build_batch(entries, self.cache, self.device, pad_blocks=pad, into=captured.batch.buffer,
-                    refresh_only=True, carry_rows=carry.rows if carry else None, planners=self.planners)
+        upload_batch(prepared, self.device, into=captured.batch.buffer, refresh_only=True)
         t_built = time.perf_counter()
         if carry:       # outside the graph: the carry is at another address every step
             ops.feed_tokens(captured.batch.token_ids, captured.batch.feed, carry.ids)

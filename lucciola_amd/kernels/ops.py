@@ -605,7 +605,8 @@ def plan_attention(layout):
         tile_list.sort(key=lambda t: -(t[3] + t[2]))
         tiles = np.asarray(tile_list, dtype=np.int32).reshape(-1, 4)
     # lengths after this step of the requests that decode: a hint for the decode kernel (how
-    # it lays its work out, never what it computes); a captured step keeps the hint of its capture
+    # it lays its work out, never what it computes); "graph_hint" below keeps a captured step
+    # to the batches whose hints are its own
     lengths = np.asarray(first, dtype=np.int64)[singles] + 1
     decode = np.zeros((singles.size, 4), dtype=np.int32)
     decode[:, 0] = np.asarray(q_start, dtype=np.int64)[singles]
@@ -619,10 +620,15 @@ def plan_attention(layout):
         decode = decode[np.argsort(-lengths, kind="stable")]
     items = _decode_items(decode, lengths[np.argsort(-lengths, kind="stable")] if lengths.size > 1 else lengths)
     # (whether the list pays, the kernel's library says from the longest and the total length)
+    longest, total = (int(lengths.max()), int(lengths.sum())) if lengths.size else (0, 0)
+    # what a captured step must share with the batches it is replayed for: the classes of lengths
+    # between which the decode kernel's launch changes (even; up to a quarter above the mean;
+    # up to three times the mean; beyond: the thresholds of lc_attn_decode_by_items)
+    spread = longest * int(lengths.size)
+    hint = (even, 0 if spread * 4 <= total * 5 else 1 if spread < total * 3 else 2)
     return ({"decode_rows": decode, "decode_items": items, "prefill_tiles": tiles},
             {"num_decode": int(singles.size), "all_decode": int(singles.size) == R, "even_lengths": even,
-             "decode_longest": int(lengths.max()) if lengths.size else 0,
-             "decode_total": int(lengths.sum()) if lengths.size else 0})
+             "decode_longest": longest, "decode_total": total, "graph_hint": hint})
 
 
 ITEM_PAGES_MIN = 8       # kernel pages of the smallest work item that a request is cut into
@@ -819,7 +825,6 @@ def attention(qkv, batch: AttentionBatch, k_cache: torch.Tensor,
         if nd > 0:
             # requests of unequal length: the planner's list of work items, which cuts the long ones
             # into more shares than the short ones; else every request into the same number
-            # (a captured step keeps the choice of its capture)
             items = None
             if batch.decode_items is not None and _decode_by_items.on is not False and (
                     _decode_by_items.on == "always"

@@ -105,7 +105,9 @@ class Part:
         batch's one copy, and host-side numbers.  Parts with equal keys share one plan; the
         part finds it as ``site.batch.plans[key]`` (``.arrays`` on the device, ``.info``).
         For batches of the same make-up the arrays must have the same sizes (captured steps
-        refresh them in place)."""
+        refresh them in place).  Where a kernel's launch depends on more of the batch than its
+        make-up, ``info["graph_hint"]`` (hashable) names the class of batches that share a
+        launch: a captured step is replayed only for batches of its own hint."""
         return None
 
 

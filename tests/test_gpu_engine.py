@@ -838,6 +838,37 @@ def test_many_requests_decode_together(requests):
     compare(got, cfg, weights, prompts, TOL["bfloat16"])
 
 
+def test_requests_of_uneven_length_decode_through_work_items():
+    """One long request among short ones decodes through the planner's list of work items (the
+    long request's pages in many shares, the short ones whole), from captured steps; when the
+    long one ends, the same number of rows and the same table width go on with lengths of another
+    class, which is a captured step of its own.  Every logit row against the plain implementation."""
+    cfg = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 512,
+           "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 128,
+           "intermediate_size": 768, "vocab_size": 300, "rope_theta": 100000.0,
+           "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 4096,
+           "initializer_range": 0.03}
+    weights = peaked(random_weights(cfg, 31))
+    lengths = [20, 20, 20, 20, 20, 700]      # (a step of five to eight rows is filled up with copies of its first)
+    prompts = prompts_for(cfg, lengths, 32)
+    names = list(prompts)
+    tail = 6
+    steps = [([(n, prompts[n][:-tail], [])], []) for n in names]
+    for k in range(tail):
+        live = names if k < 3 else names[:-1]         # the long request ends after three steps
+        ends = [names[-1]] if k == 2 else (names[:-1] if k == tail - 1 else [])
+        steps.append(([(n, [prompts[n][len(prompts[n]) - tail + k]], [0]) for n in live], ends))
+    prompts[names[-1]] = prompts[names[-1]][:-3]       # what the plain implementation sees of it
+    runner = make_runner(cfg, weights, 16, 80, "bfloat16", DEV, max_seqs=8)
+    got = replay(runner, steps)
+    lib = ops_library()
+    assert lib.lc_attn_decode_by_items(8, 2, 700, 700 + 7 * 20) == 1
+    assert lib.lc_attn_decode_by_items(8, 2, 20, 8 * 20) == 0
+    assert sorted(runner._graphs) == [(8, 64, ((False, 2),)), (8, 64, ((True, 0),))], list(runner._graphs)
+    assert runner.graph_captures == 2 and runner.graph_replays == tail - 2
+    compare(got, cfg, weights, prompts, TOL["bfloat16"])
+
+
 def ops_library():
     from lucciola_amd.kernels import ops
     return ops.library()
