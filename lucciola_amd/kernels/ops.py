@@ -583,8 +583,10 @@ ATTENTION_PLAN = "paged_attention"
 def plan_attention(layout):
     """The work lists of the attention kernels for one step's batch (a planner in the sense of
     ``Part.batch_planner``): the portions of length one, which the decode kernel serves, four
-    numbers each (token row, request, position, 0: all a workgroup needs to know of its token in
-    one load, not one look-up after the other), and the tiles of up to PREFILL_TILE query rows that the longer portions are
+    numbers each (token row, request, position, and where its work items lie: all a workgroup
+    needs to know of its token in one load, not one look-up after the other), the same rows' pages
+    cut into work items by length (:func:`_decode_items`), which the kernel takes instead where
+    few requests hold most of the keys, and the tiles of up to PREFILL_TILE query rows that the longer portions are
     cut into, four numbers each (request, first token row, rows, first position).  The tiles
     that see the most keys come first: the kernel's workgroups start in this order, and whoever
     is done takes the longest that is left (the order changes no tile's result).  The decoding
@@ -682,27 +684,6 @@ def _decode_items(decode: np.ndarray, lengths: np.ndarray) -> np.ndarray:
     items[:used, 4] = nth * n // k
     items[:used, 5] = (nth + 1) * n // k
     items[:used, 6] = k
-    return items
-    pages = (np.asarray(lengths, dtype=np.int64) + ATTENTION_PAGE_GRANULE - 1) // ATTENTION_PAGE_GRANULE
-    shares = np.ones(nd, dtype=np.int64)
-    most = np.minimum(ITEM_SHARES_MOST, np.maximum(1, pages // ITEM_PAGES_MIN))
-    spare = total - nd
-    if spare > 0:
-        heap = [(-int(pages[r]), r) for r in range(nd) if most[r] > 1]
-        heapq.heapify(heap)
-        while spare > 0 and heap:
-            _, r = heapq.heappop(heap)
-            shares[r] += 1
-            spare -= 1
-            if shares[r] < most[r]:
-                heapq.heappush(heap, (-int((pages[r] + shares[r] - 1) // shares[r]), r))
-    at = 0
-    for r in range(nd):
-        k, n = int(shares[r]), int(pages[r])
-        decode[r, 3] = at | (k << 20)
-        for s in range(k):      # sizes that differ by one page at most, none empty
-            items[at] = (decode[r, 0], decode[r, 1], decode[r, 2], r, s * n // k, (s + 1) * n // k, k, 0)
-            at += 1
     return items
 
 
