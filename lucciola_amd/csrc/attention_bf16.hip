@@ -172,9 +172,8 @@ __device__ __forceinline__ void attend_range(AttnState<D, QT>& st, const bf16x8 
     }
 }
 
-// The same walk with two pages in flight beside the one being multiplied, for the decode kernel:
-// where a request's pages are one workgroup's alone (requests of unequal length, whose long ones
-// run on at the end) a wave's pace is what it keeps in flight.  The compiler counts the loads it
+// The same walk with two pages in flight beside the one being multiplied, for the decode kernel's
+// workgroups of four waves (what it gains, and where not, stands at the launch).  The compiler counts the loads it
 // knows of and, across a loop's back edge, waits for all of them; so a page's loads are inline
 // assembly that it does not count, the waits are counted here, and three sets of page registers
 // take turns, unrolled, so that no set is ever copied.  A set is written by the hardware long
