@@ -869,6 +869,83 @@ def test_toy_mixer_with_a_paged_cache_of_its_own_layout():
         ARCHITECTURES.unregister("Toy4ForCausalLM")
 
 
+class ToyHinted(Part):
+    """A mixer of one matrix whose launch depends on more of the batch than its make-up: its
+    planner counts the cached tokens of the step's requests, and where that number is odd the
+    mixer doubles its output, a choice made on the host when the step is launched.  The planner
+    says so through ``graph_hint``, so a captured step is replayed only for its own kind."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size):
+        super().__init__(hidden_size=hidden_size)
+        self.H = hidden_size
+
+    def declare(self):
+        return {"proj": ParamDecl((self.H, self.H))}
+
+    def bind(self, tensors, ctx):
+        self.w, self.dtype = tensors["proj"], ctx.dtype
+
+    def batch_planner(self):
+        def plan(layout):
+            odd = sum(layout.first_position) % 2
+            return {"toy_odd": [odd]}, {"odd": odd, "graph_hint": odd}
+        return "toy_hinted", plan
+
+    def forward(self, x, site):
+        y = ops.gemm(x, self.w, self.dtype)
+        return y * 2 if site.batch.plans["toy_hinted"].info["odd"] else y
+
+
+class ToyScaleInGraphs(ToyScale):
+    graph_safe = True       # one product of the library, whose arguments stay put between steps
+
+
+def test_toy_mixer_whose_launch_follows_a_hint_of_its_planner():
+    """Three requests decode side by side, so the number of cached tokens is odd in every other
+    step: with captured steps the runner keeps one step per hint, and every replay gives what
+    an engine without graphs gives (a step replayed for a batch of the other kind would double,
+    or not, at the wrong time)."""
+    import numpy as np  # noqa: F401
+    MIXERS.register("toy_hinted", ToyHinted, replace=True)
+    FEED_FORWARDS.register("toy_scale", ToyScaleInGraphs, replace=True)
+    try:
+        H = 64
+        norm = PartSpec("rms", {"size": H, "eps": 1e-5})
+        layers = []
+        for i in range(2):
+            names = {"mixer_norm.weight": f"l{i}.n1", "feed_forward_norm.weight": f"l{i}.n2",
+                     "feed_forward.proj": f"l{i}.ff", "mixer.proj": f"l{i}.mix"}
+            layers.append(prenorm_layer(PartSpec("toy_hinted", {"hidden_size": H}),
+                                        PartSpec("toy_scale", {"hidden_size": H}), norm, norm, names))
+        spec = ModelSpec(hidden_size=H, vocab_size=40, embedding_name="emb", layers=layers,
+                         run_order=[RunEntry(0), RunEntry(1)], final_norm=norm,
+                         final_norm_names={"weight": "final"}, head_name="head", init_std=0.2)
+        weights = dict(random_tensors(declared_tensors(spec), 9, spec.init_std, torch.bfloat16))
+        prompts = prompts_for({"vocab_size": 40}, [30, 30, 30], 4)
+        results = {}
+        for use_graphs in (False, True):
+            model = _build(spec, DictSource(weights), "bfloat16", "cuda:0")
+            assert model.graph_safe()
+            runner = ModelRunner(model, EngineConfig(dtype="bfloat16", block_size=16, max_blocks=16, max_seqs=4,
+                                                     device="cuda:0", use_graphs=use_graphs))
+            for name, ids in prompts.items():
+                runner.step([StepEntry(name, ids[:10], [])])
+            rows = []
+            for step in range(10, 22):
+                rows.append(runner.step([StepEntry(n, [prompts[n][step]], [0]) for n in prompts]).float().cpu())
+            results[use_graphs] = torch.stack(rows)
+            if use_graphs:
+                assert sorted(k[2] for k in runner._graphs) == [(0,), (1,)]
+                assert runner.graph_captures == 2 and runner.graph_replays == 10
+        assert torch.equal(results[True], results[False])
+        assert not torch.equal(results[True][0], results[True][1])
+    finally:
+        MIXERS.unregister("toy_hinted")
+        FEED_FORWARDS.unregister("toy_scale")
+
+
 def test_kernel_signatures_can_be_registered_from_outside():
     """A part that brings kernels of its own declares their entry points itself: here one that
     the library already has is declared under the public door and launched through it."""
