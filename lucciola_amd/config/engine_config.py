@@ -43,7 +43,7 @@ class EngineConfig:
     device: str = "cuda:0"
     use_graphs: bool = True         # replay decode steps from HIP graphs (bfloat16 on the GPU)
     graph_max_batch: int = 256      # largest decode batch that is captured
-    graph_cache_size: int = 16      # captured steps kept
+    graph_cache_size: int = 32      # captured steps kept (one per number of rows, table width and planners' hint)
     run_ahead: bool = True          # queue a step before the host has the tokens of the one before
     time_steps: bool = False        # bracket every step with two events: LLMEngine.stats() gives its GPU time
 
